@@ -1,0 +1,182 @@
+/*
+ * moe_gfx950.h -- C ABI of libmoe_gfx950.so: the MoE dispatch / expert hot path as
+ * hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions
+ *  - every pointer is a DEVICE pointer unless the comment says "host";
+ *  - every call only enqueues work on `stream` (a hipStream_t passed as void*); nothing here
+ *    synchronises, allocates or frees device memory: outputs and workspaces are the caller's;
+ *  - return value: MOE_OK or a negative MOE_ERR_* code; moe_last_error() gives the text for the
+ *    calling thread;
+ *  - counts / offsets / indices are int32, contiguous (reference utils.py:14-17,31);
+ *  - `dtype` is the activation storage type (MOE_F32 or MOE_BF16); rows must be a multiple of
+ *    16 bytes long (H % 4 == 0 for f32, H % 8 == 0 for bf16);
+ *  - expert ex lives on rank ex / E_l as local expert ex % E_l (reference utils.py:217-218).
+ *
+ * The reference has no FFI: its operator API is Python (utils.py, the layers/ files).  Each entry
+ * point below names the reference routine whose device work it replaces.
+ */
+#ifndef MOE_GFX950_H
+#define MOE_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* moe_stream_t; /* hipStream_t */
+
+enum { MOE_F32 = 0, MOE_BF16 = 1 };
+enum { MOE_ACT_NONE = 0, MOE_ACT_GELU = 1, MOE_ACT_SILU = 2, MOE_ACT_SWIGLU = 3 };
+enum {
+    MOE_OK = 0,
+    MOE_ERR_INVALID = -1,     /* bad argument (shape, alignment, null pointer) */
+    MOE_ERR_UNSUPPORTED = -2, /* valid but outside what the kernels cover */
+    MOE_ERR_WORKSPACE = -3,   /* workspace too small */
+    MOE_ERR_LAUNCH = -4       /* HIP reported a launch error */
+};
+
+/* Limits of the kernels. */
+#define MOE_MAX_EXPERTS 512
+#define MOE_MAX_TOPK 16
+#define MOE_COUNT_BLOCK 64 /* tokens per counting block */
+
+int moe_abi_version(void);
+/* Text of the last error on the calling thread ("" if none). host pointer, valid until the next call. */
+const char* moe_last_error(void);
+
+/* ---- a1: router softmax + top-k ------------------------------------------------------------
+ * Replaces `F.softmax(einsum('th,he->te', tokens, router)); topk(...)` (reference utils.py:200-202).
+ * logits[t,e] = bias[e] + fp32 fmaf chain over ascending h; selection on the logits, descending,
+ * ties to the lower expert id; topk_gate = softmax probability of each selected expert (not
+ * renormalised).  x [T,H], router [H,E] in `dtype`; bias fp32 [E] or NULL.
+ * logits_ws: fp32 [T,E] scratch (also an output: the raw logits). */
+int moe_route_topk(const void* x, const void* router, const float* bias, int dtype, int T, int H, int E,
+                   int k, float* logits_ws, int32_t* topk_idx /*[T,k]*/, float* topk_gate /*[T,k]*/,
+                   moe_stream_t stream);
+
+/* ---- a2/a4/a5/a6/a7 + payload order of a3 ----------------------------------------------------
+ * Replaces the bucket loop and count/offset bookkeeping of route_and_pack_padding_free
+ * (reference utils.py:204-238), build_expert_offsets (utils.py:20-31), _build_dst_offsets
+ * (benchmark.py:44-49) and the local part of compute_capacity_from_pca (utils.py:118-121).
+ * Outputs: send_counts [W,E_l]; expert_offs [W,E_l] (exclusive prefix inside each dst block);
+ * dst_sizes [W]; dst_offsets [W]; caps[0] = max(1, max dst_sizes) (this shard's bound on M),
+ * caps[1] = max(1, max send_counts) (its bound on CAP); pos [T,k] = row of slot (t,kk) in the
+ * padding-free payload ((dst, el, token) order); row_token [T*k] = token of payload row r. */
+size_t moe_count_workspace_bytes(int T, int k, int E);
+int moe_count_and_offsets(const int32_t* topk_idx, int T, int k, int E, int W, int32_t* send_counts,
+                          int32_t* expert_offs, int32_t* dst_sizes, int32_t* dst_offsets, int32_t* caps,
+                          int32_t* pos, int32_t* row_token, void* ws, size_t ws_bytes, moe_stream_t stream);
+
+/* ---- a4/a5 on their own: build_expert_offsets (reference utils.py:20-31) and _build_dst_offsets
+ * (benchmark.py:44-49) for a given counts [W,E_l].  dst_sizes / dst_offsets may be NULL. */
+int moe_build_expert_offsets(const int32_t* counts, int W, int E_l, int32_t* expert_offs, int32_t* dst_sizes,
+                             int32_t* dst_offsets, moe_stream_t stream);
+
+/* ---- a7: M / CAP over several shards ---------------------------------------------------------
+ * out[0] = max(1, max_i values[i]) (README.md:4-7 for M; utils.py:121 for the floor).  Stands
+ * in for the all-reduce MAX of compute_capacity_from_pca when all shards live on one GPU. */
+int moe_max_floor1(const int32_t* values, int n, int32_t* out, moe_stream_t stream);
+
+/* ---- a3: padding-free payload (reference utils.py:235-246) ------------------------------------
+ * payload[r,:] = x[row_token[r],:], r < R. */
+int moe_pack_payload(const void* x, int dtype, int T, int H, const int32_t* row_token, int R, void* payload,
+                     moe_stream_t stream);
+
+/* ---- a8: fixed [W,M,H] send layout (reference README.md:5-7) ----------------------------------
+ * send[dst,m,:] = x[row_token[dst_offsets[dst]+m],:] for m < dst_sizes[dst], else zeros.
+ * map_ws: int32 [W*M] scratch.  status (nullable): set to 1 if some dst_sizes[dst] > M (rows beyond
+ * M are dropped). */
+int moe_pack(const void* x, int dtype, int T, int H, const int32_t* row_token, const int32_t* dst_sizes,
+             const int32_t* dst_offsets, int W, int M, void* send_buf, int32_t* map_ws, int32_t* status,
+             moe_stream_t stream);
+
+/* ---- a9: receive layout (reference baseline.py:178-222; kernels.py:93-102,124-125) ------------
+ * recv [W,M,H]: slot s holds what source s sent to this rank ((el, token) order, zero padded);
+ * recv_counts [W,E_l]: recv_counts[s,e] rows from source s for local expert e.
+ * token_buf[e,s,j,:] = recv[s, expert_offs_s[e]+j, :] for j < recv_counts[s,e], else zeros;
+ * pca[e,s] = recv_counts[s,e].  status (nullable): 1 on count > CAP.
+ * map_ws (here and in every entry point below that takes one): int32 scratch of
+ * moe_recv_map_ints(W, E_l, n_out) elements, n_out = rows of the output buffer. */
+size_t moe_recv_map_ints(int W, int E_l, int n_out);
+int moe_unpack_token_buf(const void* recv, int dtype, int W, int M, int H, const int32_t* recv_counts, int E_l,
+                         int CAP, void* token_buf, int32_t* pca, int32_t* map_ws, int32_t* status,
+                         moe_stream_t stream);
+
+/* Same placement from a padding-free flat payload (src-major, expert-minor blocks): the device
+ * form of reorder_flat_to_token_buf (reference baseline.py:178-222).  flat [R,H]. */
+int moe_reorder_flat_to_token_buf(const void* flat, int dtype, int R, int H, const int32_t* recv_counts, int W,
+                                  int E_l, int CAP, void* token_buf, int32_t* map_ws, int32_t* status,
+                                  moe_stream_t stream);
+
+/* ---- a10: expert-major unpack (reference layers/token_shuffle.py:31-56; kernels.py:179-205) ---
+ * shuffled[off[e,s]+j,:] = token_buf[e,s,j,:], off = exclusive prefix of pca over flattened (e,s).
+ * S_rows = rows allocated in `shuffled` (>= sum pca); rows past the sum are zero-filled.
+ * expert_cnt (nullable) [E_l] = sum_s pca[e,s] (reference layers/expert.py:26-27).
+ */
+int moe_shuffle(const void* token_buf, int dtype, int E_l, int W, int CAP, int H, const int32_t* pca,
+                void* shuffled, int S_rows, int32_t* expert_cnt, int32_t* map_ws, moe_stream_t stream);
+
+/* recv [W,M,H] -> shuffled [S_rows,H] directly (token_buf never materialised). */
+int moe_unpack_expert_major(const void* recv, int dtype, int W, int M, int H, const int32_t* recv_counts,
+                            int E_l, void* shuffled, int S_rows, int32_t* expert_cnt, int32_t* map_ws,
+                            moe_stream_t stream);
+
+/* ---- a11: grouped GEMM (reference layers/expert.py:31-60; kernels.py:240-289) -----------------
+ * out[rows of e] = tokens[rows of e] @ weights[e], fp32 accumulate, cast to `dtype`;
+ * rows of e = [sum cnt[:e], +cnt[e]).  tokens [S_rows,K]; weights [E_l,K,N] (N contiguous, the
+ * reference layout); out [S_rows,N].  Rows past sum(cnt) are left untouched.
+ * For bf16 the weights are re-tiled into ws first (moe_prepack_bytes(...) bytes). */
+size_t moe_prepack_bytes(int dtype, int E_l, int K, int N);
+int moe_grouped_gemm(const void* tokens, const void* weights, const int32_t* expert_cnt, int dtype, int S_rows,
+                     int K, int N, int E_l, void* out, void* ws, size_t ws_bytes, moe_stream_t stream);
+
+/* One-time weight re-tiling for the MFMA kernels: [E_l,K,N] (N contiguous) -> [E_l,Npad,K]
+ * (K contiguous, Npad = N rounded up to the kernel's N tile).  With w_up != NULL the two
+ * matrices are interleaved in 32-column groups (gate, up, gate, up, ...) so one kernel computes
+ * silu(x Wg) * (x Wu); the packed matrix then has 2N columns. */
+int moe_prepack_weights(const void* w, const void* w_up, int dtype, int E_l, int K, int N, void* packed,
+                        moe_stream_t stream);
+
+/* ---- a12: expert MLP (not in the reference; shapes from the workload descriptions) ------------
+ * act GELU/SILU: y = act(x W1) W2;  SWIGLU: y = (silu(x Wg) * (x Wu)) Wd.
+ * MOE_BF16: w1 = moe_prepack_weights(W1 or (Wg,Wu)) with K=H, N=F; w2 = moe_prepack_weights(W2)
+ * with K=F, N=H; w_up must be NULL; H and F multiples of 64.
+ * MOE_F32: w1 [E_l,H,F], w_up [E_l,H,F] (SwiGLU only, else NULL), w2 [E_l,F,H], reference layout.
+ * hidden_ws: [S_rows,F] in `dtype`.  fp32 accumulation; hidden activation and output rounded
+ * once to `dtype`. */
+int moe_grouped_mlp(const void* tokens, const int32_t* expert_cnt, int dtype, int S_rows, int H, int F,
+                    int E_l, int act, const void* w1, const void* w_up, const void* w2, void* hidden_ws,
+                    void* out, moe_stream_t stream);
+
+/* fp8 (OCP e4m3) SwiGLU expert.  Weights: e4m3 codes pre-packed like the bf16 ones (1 byte per
+ * element) with per-output-channel fp32 scales (sg, su [E_l,F]; sd [E_l,H]).  Activations
+ * (bf16) are quantised per row inside: xq_ws [S_rows,H] u8, xs_ws [S_rows] f32, h_ws [S_rows,F]
+ * bf16, hq_ws [S_rows,F] u8, hs_ws [S_rows] f32. */
+int moe_prepack_weights_fp8(const uint8_t* w, const uint8_t* w_up, int E_l, int K, int N, uint8_t* packed,
+                            moe_stream_t stream);
+int moe_quantize_rows_fp8(const void* x_bf16, int rows, int cols, uint8_t* q, float* scale,
+                          const int32_t* n_rows_dev, moe_stream_t stream);
+int moe_grouped_mlp_fp8(const void* tokens_bf16, const int32_t* expert_cnt, int S_rows, int H, int F, int E_l,
+                        const uint8_t* wgu_packed, const float* sg, const float* su, const uint8_t* wd_packed,
+                        const float* sd, uint8_t* xq_ws, float* xs_ws, void* h_ws, uint8_t* hq_ws, float* hs_ws,
+                        void* out, moe_stream_t stream);
+
+/* ---- a13: return path and combine (not in the reference; defined by the task statement) -------
+ * ret[s, expert_offs_s[e]+j, :] = y[off[e,s]+j, :], zero padding: the [W,M,H] buffer this rank
+ * sends back, slot s in the order source s sent its rows. */
+int moe_return_pack(const void* y, int dtype, int S_rows, int H, const int32_t* recv_counts, int W, int E_l,
+                    int M, void* ret, int32_t* map_ws, moe_stream_t stream);
+
+/* out[t,:] = sum_kk gate[t,kk] * ret[dst, pos[t,kk]-dst_offsets[dst], :], dst = idx[t,kk]/E_l;
+ * fp32 multiply then add in ascending kk (no fma), one rounding to `dtype`. */
+int moe_combine(const void* ret, int dtype, int W, int M, int H, const int32_t* topk_idx, const int32_t* pos,
+                const float* gate, const int32_t* dst_offsets, int T, int k, int E_l, void* out,
+                moe_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOE_GFX950_H */

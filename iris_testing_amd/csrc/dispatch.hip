@@ -1,0 +1,550 @@
+// Per-destination counting, offsets, deterministic payload order, and the row-movement kernels
+// (pack into [W,M,H], unpack to [E_l,W,CAP,H] / expert-major [S,H], return pack, combine).
+//
+// Replaces the Python bucket loop of route_and_pack_padding_free (reference utils.py:204-246),
+// build_expert_offsets (utils.py:20-31), _build_dst_offsets (benchmark.py:44-49),
+// reorder_flat_to_token_buf (baseline.py:178-222) and the intended token_shuffle kernel
+// (layers/token_shuffle.py:31-56; kernels.py:179-205).
+//
+// Order of rows inside a (dst, el) bucket is ascending token index (utils.py:210-219).  An
+// atomic-counter scatter would not reproduce that, so the position of every routed slot is
+// computed as   expert_start[ex] + (rows of ex in earlier 64-token blocks) + (rows of ex in
+// earlier lanes of this block),  with LDS histograms, a wave prefix scan and wave ballots.
+// All integer work: results are bit-exact by construction.
+#include "common.h"
+
+namespace {
+
+constexpr int CB = MOE_COUNT_BLOCK;  // 64 tokens = one wave per counting block
+
+// ---- 1. per-block histogram: hist[e][b] = #slots of block b routed to expert e --------------------
+__global__ __launch_bounds__(256) void block_hist_kernel(const int32_t* __restrict__ idx, int32_t* __restrict__ hist,
+                                                          int T, int k, int E, int NB) {
+    extern __shared__ int32_t lds_hist[];  // [4][E]
+    const int wave = threadIdx.x / WAVE;
+    int32_t* my = lds_hist + wave * E;
+    for (int i = threadIdx.x; i < 4 * E; i += blockDim.x) lds_hist[i] = 0;
+    __syncthreads();
+    const int b = blockIdx.x * 4 + wave;
+    const int t = b * CB + lane_id();
+    if (b < NB && t < T) {
+        for (int j = 0; j < k; ++j) {
+            const int e = idx[(size_t)t * k + j];
+            if ((unsigned)e < (unsigned)E) atomicAdd(&my[e], 1);
+        }
+    }
+    __syncthreads();
+    if (b < NB)
+        for (int e = lane_id(); e < E; e += WAVE) hist[(size_t)e * NB + b] = my[e];
+}
+
+__device__ __forceinline__ int wave_incl_scan(int v) {
+#pragma unroll
+    for (int off = 1; off < WAVE; off <<= 1) {
+        const int o = __shfl_up(v, off, WAVE);
+        if (lane_id() >= off) v += o;
+    }
+    return v;
+}
+
+// ---- 2. per-expert exclusive scan over blocks (one wave per expert) --------------------------------
+__global__ __launch_bounds__(WAVE) void scan_blocks_kernel(const int32_t* __restrict__ hist, int32_t* __restrict__ base,
+                                                            int32_t* __restrict__ counts, int NB) {
+    const int e = blockIdx.x;
+    int running = 0;
+    for (int c = 0; c < NB; c += WAVE) {
+        const int b = c + lane_id();
+        const int v = b < NB ? hist[(size_t)e * NB + b] : 0;
+        const int inc = wave_incl_scan(v);
+        if (b < NB) base[(size_t)e * NB + b] = running + inc - v;
+        running += __shfl(inc, WAVE - 1, WAVE);
+    }
+    if (lane_id() == 0) counts[e] = running;
+}
+
+// ---- 3. expert prefix -> all count/offset outputs (one wave) ---------------------------------------
+__global__ __launch_bounds__(WAVE) void offsets_kernel(const int32_t* __restrict__ counts, int E, int W,
+                                                        int32_t* __restrict__ expert_start /*[E+1]*/,
+                                                        int32_t* __restrict__ send_counts, int32_t* __restrict__ expert_offs,
+                                                        int32_t* __restrict__ dst_sizes, int32_t* __restrict__ dst_offsets,
+                                                        int32_t* __restrict__ caps) {
+    __shared__ int32_t es[MOE_MAX_EXPERTS + 1];
+    const int lane = lane_id();
+    const int per = (E + WAVE - 1) / WAVE;
+    const int lo = min(lane * per, E), hi = min(lo + per, E);
+    int sum = 0, cmax = 0;
+    for (int e = lo; e < hi; ++e) { const int c = counts[e]; sum += c; cmax = max(cmax, c); }
+    const int incl = wave_incl_scan(sum);
+    int run = incl - sum;
+    for (int e = lo; e < hi; ++e) { es[e] = run; run += counts[e]; }
+    if (lane == WAVE - 1) es[E] = incl;
+#pragma unroll
+    for (int off = WAVE / 2; off >= 1; off >>= 1) cmax = max(cmax, __shfl_xor(cmax, off, WAVE));
+    __syncthreads();
+    const int E_l = E / W;
+    for (int e = lane; e <= E; e += WAVE) expert_start[e] = es[e];
+    for (int e = lane; e < E; e += WAVE) {
+        send_counts[e] = counts[e];
+        expert_offs[e] = es[e] - es[(e / E_l) * E_l];
+    }
+    int mmax = 0;
+    for (int d = lane; d < W; d += WAVE) {
+        const int sz = es[(d + 1) * E_l] - es[d * E_l];
+        dst_sizes[d] = sz;
+        dst_offsets[d] = es[d * E_l];
+        mmax = max(mmax, sz);
+    }
+#pragma unroll
+    for (int off = WAVE / 2; off >= 1; off >>= 1) mmax = max(mmax, __shfl_xor(mmax, off, WAVE));
+    if (lane == 0) { caps[0] = max(mmax, 1); caps[1] = max(cmax, 1); }
+}
+
+// ---- 4. stable positions: one wave per 64-token block ----------------------------------------------
+__global__ __launch_bounds__(256) void rank_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ base,
+                                                    const int32_t* __restrict__ expert_start, int32_t* __restrict__ pos,
+                                                    int32_t* __restrict__ row_token, int T, int k, int E, int NB) {
+    const int wave = threadIdx.x / WAVE;
+    const int lane = lane_id();
+    const int b = blockIdx.x * 4 + wave;
+    if (b >= NB) return;
+    const int t = b * CB + lane;
+    const bool live = t < T;
+    int mine[MOE_MAX_TOPK];
+#pragma unroll
+    for (int j = 0; j < MOE_MAX_TOPK; ++j) mine[j] = (live && j < k) ? idx[(size_t)t * k + j] : -1;
+    const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (WAVE - lane));
+    for (int e0 = 0; e0 < E; e0 += WAVE) {
+        // lane l prefetches the start row of expert e0+l for this block
+        const int el = e0 + lane;
+        const int start_l = el < E ? expert_start[el] + base[(size_t)el * NB + b] : 0;
+        const int n = min(WAVE, E - e0);
+        for (int i = 0; i < n; ++i) {
+            const int e = e0 + i;
+            int jm = -1;
+#pragma unroll
+            for (int j = 0; j < MOE_MAX_TOPK; ++j)
+                if (mine[j] == e) jm = j;
+            const unsigned long long m = __ballot(jm >= 0);
+            if (m == 0ull) continue;
+            const int start = __shfl(start_l, i, WAVE);
+            if (jm >= 0) {
+                const int p = start + __popcll(m & lt_mask);
+                pos[(size_t)t * k + jm] = p;
+                row_token[p] = t;
+            }
+        }
+    }
+}
+
+// ---- small integer helpers --------------------------------------------------------------------------
+__global__ void max_floor1_kernel(const int32_t* __restrict__ v, int n, int32_t* __restrict__ out) {
+    __shared__ int32_t red[256];
+    int m = 1;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) m = max(m, v[i]);
+    red[threadIdx.x] = m;
+    __syncthreads();
+    for (int s = blockDim.x / 2; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) red[threadIdx.x] = max(red[threadIdx.x], red[threadIdx.x + s]);
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[0] = red[0];
+}
+
+// send map: map[d*M+m] = token for m < dst_sizes[d], else -1
+__global__ void send_map_kernel(const int32_t* __restrict__ row_token, const int32_t* __restrict__ dst_sizes,
+                                const int32_t* __restrict__ dst_offsets, int W, int M, int32_t* __restrict__ map,
+                                int32_t* __restrict__ status) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= W * M) return;
+    const int d = i / M, m = i % M;
+    const int n = dst_sizes[d];
+    if (m == 0 && n > M && status) *status = 1;
+    map[i] = m < n ? row_token[dst_offsets[d] + m] : -1;
+}
+
+// Tables derived from recv_counts [W,E_l] (one block):
+//   src_off[s*E_l+e] = exclusive prefix over e of recv_counts[s,:]   (row inside slot s)
+//   row_off[e*W+s]   = exclusive prefix over flattened (e,s) of recv_counts[s,e]  (+ total at [E_l*W])
+//   flat_off[s*E_l+e]= exclusive prefix over flattened (s,e)         (row in a padding-free flat payload)
+__global__ __launch_bounds__(WAVE) void recv_tables_kernel(const int32_t* __restrict__ rc, int W, int E_l,
+                                                            int32_t* __restrict__ src_off, int32_t* __restrict__ row_off,
+                                                            int32_t* __restrict__ flat_off, int32_t* __restrict__ pca,
+                                                            int32_t* __restrict__ expert_cnt) {
+    const int n = W * E_l;
+    const int lane = lane_id();
+    const int per = (n + WAVE - 1) / WAVE;
+    const int lo = min(lane * per, n), hi = min(lo + per, n);
+    // (e,s)-major prefix
+    int sum = 0;
+    for (int i = lo; i < hi; ++i) sum += rc[(i % W) * E_l + (i / W)];
+    int incl = wave_incl_scan(sum);
+    int run = incl - sum;
+    for (int i = lo; i < hi; ++i) { row_off[i] = run; run += rc[(i % W) * E_l + (i / W)]; }
+    if (lane == WAVE - 1) row_off[n] = incl;
+    // (s,e)-major prefix
+    sum = 0;
+    for (int i = lo; i < hi; ++i) sum += rc[i];
+    incl = wave_incl_scan(sum);
+    run = incl - sum;
+    for (int i = lo; i < hi; ++i) { flat_off[i] = run; run += rc[i]; }
+    if (lane == WAVE - 1) flat_off[n] = incl;
+    // per-source prefix over experts, pca transpose, per-expert totals
+    for (int s = lane; s < W; s += WAVE) {
+        int r = 0;
+        for (int e = 0; e < E_l; ++e) { src_off[s * E_l + e] = r; r += rc[s * E_l + e]; }
+    }
+    for (int i = lane; i < n; i += WAVE) {
+        if (pca) pca[i] = rc[(i % W) * E_l + (i / W)];
+    }
+    if (expert_cnt)
+        for (int e = lane; e < E_l; e += WAVE) {
+            int c = 0;
+            for (int s = 0; s < W; ++s) c += rc[s * E_l + e];
+            expert_cnt[e] = c;
+        }
+}
+
+
+// expert_offs[d,e] = exclusive prefix over e of counts[d,:]; dst_sizes / dst_offsets over d (one wave)
+__global__ __launch_bounds__(WAVE) void expert_offsets_kernel(const int32_t* __restrict__ counts, int W, int E_l,
+                                                               int32_t* __restrict__ expert_offs, int32_t* __restrict__ dst_sizes,
+                                                               int32_t* __restrict__ dst_offsets) {
+    __shared__ int32_t sizes[MOE_MAX_EXPERTS];
+    const int lane = lane_id();
+    for (int d = lane; d < W; d += WAVE) {
+        int r = 0;
+        for (int e = 0; e < E_l; ++e) { expert_offs[d * E_l + e] = r; r += counts[d * E_l + e]; }
+        sizes[d] = r;
+        if (dst_sizes) dst_sizes[d] = r;
+    }
+    __syncthreads();
+    if (dst_offsets && lane == 0) {
+        int r = 0;
+        for (int d = 0; d < W; ++d) { dst_offsets[d] = r; r += sizes[d]; }
+    }
+}
+
+__device__ __forceinline__ int upper_seg(const int32_t* off, int n, int r) {
+    // largest i in [0,n) with off[i] <= r   (off ascending, off[0] = 0)
+    int lo = 0, hi = n;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (off[mid] <= r) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+// mode 0: shuffled row r -> recv row (s*M + src_off[s,e] + j)
+// mode 1: token_buf row (e,s,j) -> recv row, or -1
+// mode 2: return slot (s,m) -> shuffled row off[e,s]+j, or -1
+// mode 3: token_buf row (e,s,j) -> flat payload row flat_off[s,e]+j, or -1
+// mode 4: shuffled row r -> token_buf row ((e*W+s)*CAP + j)
+__global__ void recv_map_kernel(int mode, const int32_t* __restrict__ rc, const int32_t* __restrict__ src_off,
+                                const int32_t* __restrict__ row_off, const int32_t* __restrict__ flat_off, int W,
+                                int E_l, int M, int CAP, int n_out, int32_t* __restrict__ map,
+                                int32_t* __restrict__ status) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_out) return;
+    const int n = W * E_l;
+    int out = -1;
+    if (mode == 0 || mode == 4) {
+        const int S = row_off[n];
+        if (i < S) {
+            const int seg = upper_seg(row_off, n + 1, i);  // seg = e*W+s, skips empty segments by construction
+            const int e = seg / W, s = seg % W, j = i - row_off[seg];
+            out = mode == 0 ? s * M + src_off[s * E_l + e] + j : (e * W + s) * CAP + j;
+        }
+    } else if (mode == 1 || mode == 3) {
+        const int j = i % CAP, s = (i / CAP) % W, e = i / (CAP * W);
+        const int c = rc[s * E_l + e];
+        if (j == 0 && c > CAP && status) *status = 1;
+        if (j < c) out = mode == 1 ? s * M + src_off[s * E_l + e] + j : flat_off[s * E_l + e] + j;
+    } else {  // mode 2
+        const int s = i / M, m = i % M;
+        const int tot = src_off[s * E_l + E_l - 1] + rc[s * E_l + E_l - 1];
+        if (m < tot) {
+            const int e = upper_seg(src_off + s * E_l, E_l, m);
+            // upper_seg returns the LAST expert whose offset <= m, which is the non-empty one owning m
+            out = row_off[e * W + s] + (m - src_off[s * E_l + e]);
+        }
+    }
+    map[i] = out;
+}
+
+// ---- row gather: dst[r,:] = map[r] >= 0 ? src[map[r],:] : 0 ; one wave per row, 16-byte lanes ----
+template <int WPB>
+__global__ __launch_bounds__(WPB * WAVE) void gather_rows_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
+                                                                  const int32_t* __restrict__ map, int n_rows,
+                                                                  int row_vec /* 16-byte units per row */) {
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    for (int r = blockIdx.x * WPB + wave; r < n_rows; r += gridDim.x * WPB) {
+        const int m = map[r];
+        uint4* d = dst + (size_t)r * row_vec;
+        if (m >= 0) {
+            const uint4* s = src + (size_t)m * row_vec;
+            int c = lane;
+            for (; c + 3 * WAVE < row_vec; c += 4 * WAVE) {
+                const uint4 a0 = s[c], a1 = s[c + WAVE], a2 = s[c + 2 * WAVE], a3 = s[c + 3 * WAVE];
+                d[c] = a0; d[c + WAVE] = a1; d[c + 2 * WAVE] = a2; d[c + 3 * WAVE] = a3;
+            }
+            for (; c < row_vec; c += WAVE) d[c] = s[c];
+        } else {
+            const uint4 z = make_uint4(0, 0, 0, 0);
+            for (int c = lane; c < row_vec; c += WAVE) d[c] = z;
+        }
+    }
+}
+
+// ---- combine: out[t,:] = sum_kk gate[t,kk] * ret[slot(t,kk),:] --------------------------------------
+template <typename XT>
+struct Vec16;
+template <>
+struct Vec16<bf16_t> {
+    static constexpr int N = 8;
+    __device__ static void unpack(const uint4& v, float* f) {
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { f[2 * i] = __uint_as_float(w[i] << 16); f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u); }
+    }
+    __device__ static uint4 pack(const float* f) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = (uint32_t)f32_to_bf16(f[2 * i]) | ((uint32_t)f32_to_bf16(f[2 * i + 1]) << 16);
+        return make_uint4(w[0], w[1], w[2], w[3]);
+    }
+};
+template <>
+struct Vec16<float> {
+    static constexpr int N = 4;
+    __device__ static void unpack(const uint4& v, float* f) {
+        f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y); f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
+    }
+    __device__ static uint4 pack(const float* f) {
+        return make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3]));
+    }
+};
+
+template <typename XT, int WPB>
+__global__ __launch_bounds__(WPB * WAVE) void combine_kernel(const uint4* __restrict__ ret, const int32_t* __restrict__ idx,
+                                                              const int32_t* __restrict__ pos, const float* __restrict__ gate,
+                                                              const int32_t* __restrict__ dst_offsets, int T, int k, int E_l,
+                                                              int M, int row_vec, uint4* __restrict__ out) {
+    constexpr int N = Vec16<XT>::N;
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    for (int t = blockIdx.x * WPB + wave; t < T; t += gridDim.x * WPB) {
+        size_t rows[MOE_MAX_TOPK];
+        float g[MOE_MAX_TOPK];
+#pragma unroll
+        for (int j = 0; j < MOE_MAX_TOPK; ++j) {
+            if (j < k) {
+                const int d = idx[(size_t)t * k + j] / E_l;
+                rows[j] = ((size_t)d * M + (pos[(size_t)t * k + j] - dst_offsets[d])) * row_vec;
+                g[j] = gate[(size_t)t * k + j];
+            }
+        }
+        for (int c = lane; c < row_vec; c += WAVE) {
+            float acc[N];
+#pragma unroll
+            for (int i = 0; i < N; ++i) acc[i] = 0.f;
+#pragma unroll
+            for (int j = 0; j < MOE_MAX_TOPK; ++j) {
+                if (j < k) {
+                    float f[N];
+                    Vec16<XT>::unpack(ret[rows[j] + c], f);
+#pragma unroll
+                    for (int i = 0; i < N; ++i) acc[i] = __fadd_rn(acc[i], __fmul_rn(g[j], f[i]));
+                }
+            }
+            out[(size_t)t * row_vec + c] = Vec16<XT>::pack(acc);
+        }
+    }
+}
+
+int gather_rows(const void* src, void* dst, const int32_t* map, int n_rows, int row_bytes, hipStream_t s) {
+    if (n_rows == 0) return MOE_OK;
+    const int blocks = min(ceil_div(n_rows, 4), 65535 * 8);
+    gather_rows_kernel<4><<<blocks, 4 * WAVE, 0, s>>>((const uint4*)src, (uint4*)dst, map, n_rows, row_bytes / 16);
+    return moe_check_launch("gather_rows");
+}
+
+struct RecvTables {
+    int32_t *src_off, *row_off, *flat_off;
+};
+// map_ws layout for the recv-driven entry points: [n_out map][tables]
+// three prefix tables plus room for a transposed copy of the counts
+size_t recv_tables_ints(int W, int E_l) { return (size_t)3 * (W * E_l + 1) + (size_t)W * E_l; }
+
+int check_rows(const char* who, int dtype, int H) {
+    if (dtype != MOE_F32 && dtype != MOE_BF16) return moe_fail(MOE_ERR_INVALID, "%s: dtype %d", who, dtype);
+    if (H <= 0 || (H * dtype_size(dtype)) % 16 != 0)
+        return moe_fail(MOE_ERR_INVALID, "%s: rows must be 16-byte multiples (H=%d)", who, H);
+    return MOE_OK;
+}
+
+}  // namespace
+
+extern "C" size_t moe_count_workspace_bytes(int T, int k, int E) {
+    (void)k;
+    const size_t NB = (size_t)ceil_div(T > 0 ? T : 1, CB);
+    // hist[E][NB] + base[E][NB] + counts[E] + expert_start[E+1]
+    return sizeof(int32_t) * (2 * (size_t)E * NB + 2 * (size_t)E + 1);
+}
+
+extern "C" int moe_count_and_offsets(const int32_t* topk_idx, int T, int k, int E, int W, int32_t* send_counts,
+                                     int32_t* expert_offs, int32_t* dst_sizes, int32_t* dst_offsets, int32_t* caps,
+                                     int32_t* pos, int32_t* row_token, void* ws, size_t ws_bytes, moe_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    MOE_REQUIRE(T >= 0 && E > 0 && W > 0, MOE_ERR_INVALID, "count: bad shape T=%d E=%d W=%d", T, E, W);
+    MOE_REQUIRE(E % W == 0, MOE_ERR_INVALID, "num_experts_total must be divisible by world_size (E=%d W=%d)", E, W);
+    MOE_REQUIRE(k >= 1 && k <= MOE_MAX_TOPK, MOE_ERR_UNSUPPORTED, "count: topk=%d outside [1,%d]", k, MOE_MAX_TOPK);
+    MOE_REQUIRE(E <= MOE_MAX_EXPERTS, MOE_ERR_UNSUPPORTED, "count: E=%d > %d", E, MOE_MAX_EXPERTS);
+    MOE_REQUIRE(send_counts && expert_offs && dst_sizes && dst_offsets && caps && ws, MOE_ERR_INVALID, "count: null pointer");
+    MOE_REQUIRE(T == 0 || (topk_idx && pos && row_token), MOE_ERR_INVALID, "count: null pointer");
+    MOE_REQUIRE(ws_bytes >= moe_count_workspace_bytes(T, k, E), MOE_ERR_WORKSPACE, "count: workspace %zu < %zu", ws_bytes,
+                moe_count_workspace_bytes(T, k, E));
+    const int NB = ceil_div(T > 0 ? T : 1, CB);
+    int32_t* hist = (int32_t*)ws;
+    int32_t* base = hist + (size_t)E * NB;
+    int32_t* counts = base + (size_t)E * NB;
+    int32_t* expert_start = counts + E;
+    block_hist_kernel<<<ceil_div(NB, 4), 256, 4 * E * sizeof(int32_t), s>>>(topk_idx, hist, T, k, E, NB);
+    scan_blocks_kernel<<<E, WAVE, 0, s>>>(hist, base, counts, NB);
+    offsets_kernel<<<1, WAVE, 0, s>>>(counts, E, W, expert_start, send_counts, expert_offs, dst_sizes, dst_offsets, caps);
+    if (T > 0) rank_kernel<<<ceil_div(NB, 4), 256, 0, s>>>(topk_idx, base, expert_start, pos, row_token, T, k, E, NB);
+    return moe_check_launch("count_and_offsets");
+}
+
+extern "C" int moe_build_expert_offsets(const int32_t* counts, int W, int E_l, int32_t* expert_offs, int32_t* dst_sizes,
+                                        int32_t* dst_offsets, moe_stream_t stream) {
+    MOE_REQUIRE(W > 0 && E_l > 0 && W <= MOE_MAX_EXPERTS, MOE_ERR_INVALID, "build_expert_offsets: bad shape W=%d E_l=%d", W, E_l);
+    MOE_REQUIRE(counts && expert_offs, MOE_ERR_INVALID, "build_expert_offsets: null pointer");
+    expert_offsets_kernel<<<1, WAVE, 0, (hipStream_t)stream>>>(counts, W, E_l, expert_offs, dst_sizes, dst_offsets);
+    return moe_check_launch("build_expert_offsets");
+}
+
+extern "C" int moe_max_floor1(const int32_t* values, int n, int32_t* out, moe_stream_t stream) {
+    MOE_REQUIRE(n >= 0 && out && (n == 0 || values), MOE_ERR_INVALID, "max_floor1: bad arguments");
+    max_floor1_kernel<<<1, 256, 0, (hipStream_t)stream>>>(values, n, out);
+    return moe_check_launch("max_floor1");
+}
+
+extern "C" int moe_pack_payload(const void* x, int dtype, int T, int H, const int32_t* row_token, int R, void* payload,
+                                moe_stream_t stream) {
+    int rc = check_rows("pack_payload", dtype, H);
+    if (rc) return rc;
+    MOE_REQUIRE(R >= 0 && T >= 0, MOE_ERR_INVALID, "pack_payload: bad shape");
+    if (R == 0) return MOE_OK;
+    MOE_REQUIRE(x && row_token && payload, MOE_ERR_INVALID, "pack_payload: null pointer");
+    return gather_rows(x, payload, row_token, R, H * dtype_size(dtype), (hipStream_t)stream);
+}
+
+extern "C" int moe_pack(const void* x, int dtype, int T, int H, const int32_t* row_token, const int32_t* dst_sizes,
+                        const int32_t* dst_offsets, int W, int M, void* send_buf, int32_t* map_ws, int32_t* status,
+                        moe_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    int rc = check_rows("pack", dtype, H);
+    if (rc) return rc;
+    MOE_REQUIRE(W > 0 && M >= 1 && T >= 0, MOE_ERR_INVALID, "pack: bad shape W=%d M=%d", W, M);
+    MOE_REQUIRE((long long)W * M < (1ll << 31), MOE_ERR_UNSUPPORTED, "pack: W*M too large");
+    MOE_REQUIRE(send_buf && map_ws && dst_sizes && dst_offsets, MOE_ERR_INVALID, "pack: null pointer");
+    const int n = W * M;
+    send_map_kernel<<<ceil_div(n, 256), 256, 0, s>>>(row_token, dst_sizes, dst_offsets, W, M, map_ws, status);
+    return gather_rows(x, send_buf, map_ws, n, H * dtype_size(dtype), s);
+}
+
+static int recv_driven(const char* who, int mode, const void* src, void* dst, int dtype, int H, const int32_t* rc_dev,
+                       int W, int E_l, int M, int CAP, int n_out, int32_t* pca, int32_t* expert_cnt, int32_t* map_ws,
+                       int32_t* status, hipStream_t s) {
+    int rc = check_rows(who, dtype, H);
+    if (rc) return rc;
+    MOE_REQUIRE(W > 0 && E_l > 0 && W * E_l <= MOE_MAX_EXPERTS, MOE_ERR_INVALID, "%s: bad W=%d E_l=%d", who, W, E_l);
+    MOE_REQUIRE(n_out >= 0 && rc_dev && map_ws, MOE_ERR_INVALID, "%s: bad arguments", who);
+    int32_t* tables = map_ws + n_out;
+    const int n = W * E_l;
+    int32_t* src_off = tables;
+    int32_t* row_off = tables + (n + 1);
+    int32_t* flat_off = tables + 2 * (n + 1);
+    recv_tables_kernel<<<1, WAVE, 0, s>>>(rc_dev, W, E_l, src_off, row_off, flat_off, pca, expert_cnt);
+    if (n_out == 0) return moe_check_launch(who);
+    MOE_REQUIRE(dst && (src || mode == 3), MOE_ERR_INVALID, "%s: null pointer", who);  // an empty flat payload has no storage
+    recv_map_kernel<<<ceil_div(n_out, 256), 256, 0, s>>>(mode, rc_dev, src_off, row_off, flat_off, W, E_l, M, CAP, n_out,
+                                                        map_ws, status);
+    return gather_rows(src, dst, map_ws, n_out, H * dtype_size(dtype), s);
+}
+
+extern "C" size_t moe_recv_map_ints(int W, int E_l, int n_out) { return (size_t)n_out + recv_tables_ints(W, E_l); }
+
+extern "C" int moe_unpack_token_buf(const void* recv, int dtype, int W, int M, int H, const int32_t* recv_counts,
+                                    int E_l, int CAP, void* token_buf, int32_t* pca, int32_t* map_ws, int32_t* status,
+                                    moe_stream_t stream) {
+    MOE_REQUIRE(M >= 1 && CAP >= 1, MOE_ERR_INVALID, "unpack_token_buf: M=%d CAP=%d", M, CAP);
+    MOE_REQUIRE((long long)E_l * W * CAP < (1ll << 31), MOE_ERR_UNSUPPORTED, "unpack_token_buf: too many rows");
+    return recv_driven("unpack_token_buf", 1, recv, token_buf, dtype, H, recv_counts, W, E_l, M, CAP, E_l * W * CAP, pca,
+                       nullptr, map_ws, status, (hipStream_t)stream);
+}
+
+extern "C" int moe_reorder_flat_to_token_buf(const void* flat, int dtype, int R, int H, const int32_t* recv_counts,
+                                             int W, int E_l, int CAP, void* token_buf, int32_t* map_ws, int32_t* status,
+                                             moe_stream_t stream) {
+    (void)R;
+    MOE_REQUIRE(CAP >= 1, MOE_ERR_INVALID, "reorder: CAP=%d", CAP);
+    MOE_REQUIRE((long long)E_l * W * CAP < (1ll << 31), MOE_ERR_UNSUPPORTED, "reorder: too many rows");
+    return recv_driven("reorder_flat_to_token_buf", 3, flat, token_buf, dtype, H, recv_counts, W, E_l, 1, CAP,
+                       E_l * W * CAP, nullptr, nullptr, map_ws, status, (hipStream_t)stream);
+}
+
+extern "C" int moe_unpack_expert_major(const void* recv, int dtype, int W, int M, int H, const int32_t* recv_counts,
+                                       int E_l, void* shuffled, int S_rows, int32_t* expert_cnt, int32_t* map_ws,
+                                       moe_stream_t stream) {
+    MOE_REQUIRE(M >= 1, MOE_ERR_INVALID, "unpack_expert_major: M=%d", M);
+    return recv_driven("unpack_expert_major", 0, recv, shuffled, dtype, H, recv_counts, W, E_l, M, 1, S_rows, nullptr,
+                       expert_cnt, map_ws, nullptr, (hipStream_t)stream);
+}
+
+// token_buf -> shuffled: pca is [E_l,W]; the tables kernel wants [W,E_l] counts, so transpose first.
+__global__ void transpose_counts_kernel(const int32_t* __restrict__ in, int rows, int cols, int32_t* __restrict__ out) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < rows * cols) out[(i % cols) * rows + (i / cols)] = in[i];
+}
+
+extern "C" int moe_shuffle(const void* token_buf, int dtype, int E_l, int W, int CAP, int H, const int32_t* pca,
+                           void* shuffled, int S_rows, int32_t* expert_cnt, int32_t* map_ws, moe_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    MOE_REQUIRE(W > 0 && E_l > 0 && W * E_l <= MOE_MAX_EXPERTS && CAP >= 1 && S_rows >= 0 && pca && map_ws,
+                MOE_ERR_INVALID, "shuffle: bad arguments");
+    // recv_counts[s,e] = pca[e,s], kept behind the tables in map_ws
+    int32_t* rc_t = map_ws + S_rows + recv_tables_ints(W, E_l);
+    transpose_counts_kernel<<<ceil_div(W * E_l, 256), 256, 0, s>>>(pca, E_l, W, rc_t);
+    return recv_driven("shuffle", 4, token_buf, shuffled, dtype, H, rc_t, W, E_l, 1, CAP, S_rows, nullptr, expert_cnt,
+                       map_ws, nullptr, s);
+}
+
+extern "C" int moe_return_pack(const void* y, int dtype, int S_rows, int H, const int32_t* recv_counts, int W, int E_l,
+                               int M, void* ret, int32_t* map_ws, moe_stream_t stream) {
+    (void)S_rows;
+    MOE_REQUIRE(M >= 1, MOE_ERR_INVALID, "return_pack: M=%d", M);
+    MOE_REQUIRE((long long)W * M < (1ll << 31), MOE_ERR_UNSUPPORTED, "return_pack: W*M too large");
+    return recv_driven("return_pack", 2, y, ret, dtype, H, recv_counts, W, E_l, M, 1, W * M, nullptr, nullptr, map_ws,
+                       nullptr, (hipStream_t)stream);
+}
+
+extern "C" int moe_combine(const void* ret, int dtype, int W, int M, int H, const int32_t* topk_idx, const int32_t* pos,
+                           const float* gate, const int32_t* dst_offsets, int T, int k, int E_l, void* out,
+                           moe_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    int rc = check_rows("combine", dtype, H);
+    if (rc) return rc;
+    MOE_REQUIRE(W > 0 && M >= 1 && T >= 0 && E_l > 0, MOE_ERR_INVALID, "combine: bad shape");
+    MOE_REQUIRE(k >= 1 && k <= MOE_MAX_TOPK, MOE_ERR_UNSUPPORTED, "combine: topk=%d outside [1,%d]", k, MOE_MAX_TOPK);
+    if (T == 0) return MOE_OK;
+    MOE_REQUIRE(ret && topk_idx && pos && gate && dst_offsets && out, MOE_ERR_INVALID, "combine: null pointer");
+    const int row_vec = H * dtype_size(dtype) / 16;
+    const int blocks = min(ceil_div(T, 4), 65535 * 8);
+    if (dtype == MOE_F32)
+        combine_kernel<float, 4><<<blocks, 4 * WAVE, 0, s>>>((const uint4*)ret, topk_idx, pos, gate, dst_offsets, T, k, E_l,
+                                                            M, row_vec, (uint4*)out);
+    else
+        combine_kernel<bf16_t, 4><<<blocks, 4 * WAVE, 0, s>>>((const uint4*)ret, topk_idx, pos, gate, dst_offsets, T, k,
+                                                             E_l, M, row_vec, (uint4*)out);
+    return moe_check_launch("combine");
+}

@@ -1,0 +1,651 @@
+// Persistent grouped expert GEMM / MLP on gfx950 MFMA (bf16 and OCP fp8) with LDS-staged tiles,
+// plus an fp32 path for the plumbing-size workload.
+//
+// Replaces the reference's intended expert layer (layers/expert.py:31-60) and grouped_gemm kernel
+// (kernels.py:240-289): out[rows of group g] = tokens[rows of g] @ weights[g], fp32 accumulate,
+// persistent grid walking a tile list that spans all groups.  Differences in kind, not a port:
+//   * tiles are 256(or 128) x 256 x 128 bytes of K, four wave64s each owning a 128(64) x 128 block of
+//     32x32x16 MFMAs;
+//   * operands go HBM -> LDS directly (global_load_lds, 16 bytes per lane), double buffered, with
+//     an XOR swizzle of the 16-byte chunks so that MFMA fragment reads are bank-conflict free;
+//   * weights are re-tiled once into a K-contiguous layout (gate/up interleaved for SwiGLU) so both
+//     MFMA operands are read as 128-bit fragments;
+//   * ragged group tails are masked (the reference assumes full tiles, kernels.py:270,282);
+//   * the tile walk is XCD-aware: the 32 workgroups that share an L2 take a compact 4 x 8 patch of
+//     a 16 x 16 super-tile.
+#include "common.h"
+
+namespace moe_gg {
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int ROWB = 128;  // bytes of K per tile row per stage
+constexpr int CHUNKS = ROWB / 16;
+constexpr int SUP = 16;  // super-tile edge, in tiles
+constexpr int GG_MAXG = MOE_MAX_EXPERTS;
+constexpr int GG_BN = 256;
+
+struct GemmParams {
+    const uint8_t* A;         // [S_rows, K] activations (bf16 or fp8)
+    const uint8_t* B;         // packed weights [E_l, Npad, K]
+    void* C;                  // [S_rows, ldc] bf16
+    const int32_t* cnt;       // [E_l] rows per group
+    const float* row_scale;   // fp8: [S_rows] per-row activation scale
+    const float* col_scale;   // fp8: [E_l, ncs] per-output-channel scale (gate for SwiGLU)
+    const float* col_scale2;  // fp8 SwiGLU: [E_l, ncs] up scales
+    int E_l, K, N, Npad, ldc, S_rows, ncs;
+};
+
+__device__ __forceinline__ float act_silu(float x) { return x / (1.0f + __expf(-x)); }
+__device__ __forceinline__ float act_gelu(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }
+
+template <bool FP8>
+__device__ __forceinline__ void mma(floatx16& acc, const uint4& a, const uint4& b) {
+    if constexpr (FP8) {
+        // 16 bytes per lane = two 8-byte K groups; both operands are split the same way, so every
+        // k of the 32 covered by the lane pair is multiplied exactly once.
+        const long a0 = (long)(((unsigned long)a.y << 32) | a.x), a1 = (long)(((unsigned long)a.w << 32) | a.z);
+        const long b0 = (long)(((unsigned long)b.y << 32) | b.x), b1 = (long)(((unsigned long)b.w << 32) | b.z);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a0, b0, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a1, b1, acc, 0, 0, 0);
+    } else {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
+                                                      acc, 0, 0, 0);
+    }
+}
+
+__device__ __forceinline__ int seg_of(const int* off, int n, int r) {
+    int lo = 0, hi = n;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (off[mid] <= r) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+enum { EPI_NONE = 0, EPI_GELU = 1, EPI_SILU = 2, EPI_SWIGLU = 3 };
+
+// ---- pieces of the main loop ---------------------------------------------------------------------
+// HBM -> LDS, 16 bytes per lane, no register staging.  One instruction moves 8 tile rows (64 lanes x
+// 16 B); wave w of a round moves rows [w*8, w*8+8) of that round.
+template <int RA, int RB, int LR>
+__device__ __forceinline__ void gg_issue(uint4* sA, uint4* sB, const uint8_t* ap, const uint8_t* bp,
+                                         const uint32_t* a_off, uint32_t b_off0, uint32_t b_step, int wave) {
+#pragma unroll
+    for (int r = 0; r < RA; ++r)
+        __builtin_amdgcn_global_load_lds(ap + a_off[r], (lds_ptr_t)(sA + (r * LR + wave * 8) * CHUNKS), 16, 0, 0);
+#pragma unroll
+    for (int r = 0; r < RB; ++r)
+        __builtin_amdgcn_global_load_lds(bp + b_off0 + r * b_step, (lds_ptr_t)(sB + (r * LR + wave * 8) * CHUNKS), 16, 0, 0);
+}
+
+template <int TM, int TN>
+__device__ __forceinline__ void gg_frags(const uint4* fa, const uint4* fb, int pos, uint4 (&a)[TM], uint4 (&b)[TN]) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) a[i] = fa[i * 32 * CHUNKS + pos];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) b[j] = fb[j * 32 * CHUNKS + pos];
+}
+
+// weights are the MFMA A operand and activations the B operand, so acc holds the transposed product
+template <int TM, int TN, bool FP8>
+__device__ __forceinline__ void gg_mmas(floatx16 (&acc)[TM][TN], const uint4 (&a)[TM], const uint4 (&b)[TN]) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) mma<FP8>(acc[i][j], b[j], a[i]);
+}
+
+template <int N>
+__device__ __forceinline__ void gg_wait_vm() {
+    if constexpr (N == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else if constexpr (N == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else if constexpr (N == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    else if constexpr (N == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    else static_assert(N == 0, "add the wait count");
+}
+
+
+// acc(i,j) holds the TRANSPOSED 32x32 product (weights as the MFMA A operand, activations as B):
+// lane l owns token row l%32 and output columns 8*(v/4) + 4*(l/32) + v%4, v = 0..15, i.e. four runs
+// of four consecutive columns -> 8-byte bf16 stores.
+// NWM x 2 wave64s per workgroup; every wave owns a (BM/NWM) x 128 block of the tile.
+template <int BM, int NWM, int EPI, bool FP8>
+__global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const GemmParams p) {
+    constexpr int BN = GG_BN;
+    constexpr int ES = FP8 ? 1 : 2;
+    constexpr int BK = ROWB / ES;
+    constexpr int NW = NWM * 2;                       // waves per workgroup
+    constexpr int TM = BM / (NWM * 32), TN = BN / 64;  // 32x32 MFMA tiles per wave
+    constexpr int LR = NW * 8;                        // rows fetched per load round (8 per wave)
+    constexpr int RA = BM / LR, RB = BN / LR;         // load rounds per stage
+    constexpr int NKK = CHUNKS / 2;            // fragment steps per stage (4)
+
+    __shared__ __align__(1024) uint4 sA0[BM * CHUNKS];
+    __shared__ __align__(1024) uint4 sB0[BN * CHUNKS];
+    __shared__ __align__(1024) uint4 sA1[BM * CHUNKS];
+    __shared__ __align__(1024) uint4 sB1[BN * CHUNKS];
+    __shared__ int g_tile_start[GG_MAXG + 1];
+    __shared__ int g_row_start[GG_MAXG + 1];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int Nt = p.Npad / BN;
+    static_assert(TM * 32 * NWM == BM && LR % 16 == 0, "tile shape");
+
+    if (tid == 0) {
+        int ts = 0, rs = 0;
+        for (int g = 0; g < p.E_l; ++g) {
+            g_tile_start[g] = ts;
+            g_row_start[g] = rs;
+            const int c = max(p.cnt[g], 0);
+            ts += ((c + BM - 1) / BM) * Nt;
+            rs += c;
+        }
+        g_tile_start[p.E_l] = ts;
+        g_row_start[p.E_l] = rs;
+    }
+    __syncthreads();
+    const int total = g_tile_start[p.E_l];
+    const int nk = p.K / BK;
+
+    // XCD-aware position inside a round of gridDim.x tiles: workgroups b, b+8, b+16, ... share an L2.
+    int my = blockIdx.x;
+    if (gridDim.x == 256) {
+        const int xcd = blockIdx.x & 7, l = blockIdx.x >> 3;
+        my = (((xcd >> 1) * 4 + (l >> 3)) * SUP) + ((xcd & 1) * 8 + (l & 7));
+    }
+
+    // lane-constant pieces of the addressing
+    const int lrow = wave * 8 + (lane >> 3);            // row inside a load round
+    const int lchunk = (lane & 7) ^ ((lrow >> 1) & 7);  // global 16-byte chunk this lane fetches
+    const int fswz = (lane >> 1) & 7;                   // swizzle of the fragment row (row % 16 = lane % 16)
+    const int khalf = lane >> 5;
+    const uint4* fa0 = sA0 + (wm * (BM / NWM) + (lane & 31)) * CHUNKS;
+    const uint4* fa1 = sA1 + (wm * (BM / NWM) + (lane & 31)) * CHUNKS;
+    const uint4* fb0 = sB0 + (wn * (BN / 2) + (lane & 31)) * CHUNKS;
+    const uint4* fb1 = sB1 + (wn * (BN / 2) + (lane & 31)) * CHUNKS;
+
+    for (int base = 0; base < total; base += gridDim.x) {
+        const int lin = base + my;
+        if (lin >= total) continue;  // uniform over the workgroup
+        // ---- decode lin -> (group, m tile, n tile): group-major, 16-row bands, 16-col super-columns
+        const int g = seg_of(g_tile_start, p.E_l + 1, lin);
+        const int cnt_g = g_row_start[g + 1] - g_row_start[g];
+        const int Mt = (cnt_g + BM - 1) / BM;
+        const int idx = lin - g_tile_start[g];
+        const int band = idx / (SUP * Nt), rem = idx % (SUP * Nt);
+        const int hr = min(SUP, Mt - band * SUP);
+        const int sc = rem / (hr * SUP), rem2 = rem % (hr * SUP);
+        const int wc = min(SUP, Nt - sc * SUP);
+        const int mt = band * SUP + rem2 / wc, nt = sc * SUP + rem2 % wc;
+
+        const int row0 = g_row_start[g] + mt * BM;
+        const int rv = min(min(BM, cnt_g - mt * BM), p.S_rows - row0);  // valid rows of this tile
+        if (rv <= 0) continue;
+
+        const uint8_t* Ab = p.A + (size_t)row0 * p.K * ES;
+        const uint8_t* Bb = p.B + ((size_t)g * p.Npad + (size_t)nt * BN) * p.K * ES;
+        const uint32_t ldk = (uint32_t)(p.K * ES);
+        uint32_t a_off[RA];
+#pragma unroll
+        for (int r = 0; r < RA; ++r) a_off[r] = (uint32_t)min(r * LR + lrow, rv - 1) * ldk + lchunk * 16;
+        const uint32_t b_off0 = (uint32_t)lrow * ldk + lchunk * 16;
+        const uint32_t b_step = (uint32_t)LR * ldk;
+
+        floatx16 acc[TM][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+        uint4 a0[TM], b0[TN], a1[TM], b1[TN];
+        const int pos0 = (0 + khalf) ^ fswz, pos1 = (2 + khalf) ^ fswz, pos2 = (4 + khalf) ^ fswz, pos3 = (6 + khalf) ^ fswz;
+        static_assert(NKK == 4, "GG_STAGE is written for four fragment steps");
+
+        // One K stage: fragments of step kk+1 are requested before the MFMAs of step kk are issued;
+        // the stage hand-over (loads landed + barrier + refill of the buffer just drained) sits before
+        // the last MFMA block so that its latency hides behind that block.
+#define GG_ISSUE(sA, sB, ks) \
+    gg_issue<RA, RB, LR>(sA, sB, Ab + (size_t)(ks) * ROWB, Bb + (size_t)(ks) * ROWB, a_off, b_off0, b_step, wave)
+#define GG_STAGE(fa, fb, na, nb, curA, curB, ks)                           \
+    do {                                                                   \
+        gg_frags<TM, TN>(fa, fb, pos1, a1, b1);                            \
+        gg_mmas<TM, TN, FP8>(acc, a0, b0);                                 \
+        __builtin_amdgcn_sched_barrier(0);                                 \
+        gg_frags<TM, TN>(fa, fb, pos2, a0, b0);                            \
+        gg_mmas<TM, TN, FP8>(acc, a1, b1);                                 \
+        __builtin_amdgcn_sched_barrier(0);                                 \
+        gg_frags<TM, TN>(fa, fb, pos3, a1, b1);                            \
+        gg_mmas<TM, TN, FP8>(acc, a0, b0);                                 \
+        __builtin_amdgcn_sched_barrier(0);                                 \
+        if ((ks) + 1 < nk) {                                               \
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");    \
+            __syncthreads();                                               \
+            if ((ks) + 2 < nk) GG_ISSUE(curA, curB, (ks) + 2);             \
+            gg_frags<TM, TN>(na, nb, pos0, a0, b0);                        \
+        }                                                                  \
+        __builtin_amdgcn_sched_barrier(0);                                 \
+        gg_mmas<TM, TN, FP8>(acc, a1, b1);                                 \
+        __builtin_amdgcn_sched_barrier(0);                                 \
+    } while (0)
+
+        __syncthreads();  // every wave is done with LDS of the previous tile
+        GG_ISSUE(sA0, sB0, 0);
+        if (nk > 1) {
+            GG_ISSUE(sA1, sB1, 1);
+            gg_wait_vm<RA + RB>();
+        } else {
+            gg_wait_vm<0>();
+        }
+        __syncthreads();
+        gg_frags<TM, TN>(fa0, fb0, pos0, a0, b0);
+        for (int ks = 0; ks < nk; ks += 2) {
+            GG_STAGE(fa0, fb0, fa1, fb1, sA0, sB0, ks);
+            if (ks + 1 < nk) GG_STAGE(fa1, fb1, fa0, fb0, sA1, sB1, ks + 1);
+        }
+#undef GG_STAGE
+#undef GG_ISSUE
+
+        // ---- epilogue: acc -> (scales) -> activation -> bf16 -> C
+        bf16_t* C = (bf16_t*)p.C;
+        const int chalf = khalf * 4;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int r = wm * (BM / NWM) + i * 32 + (lane & 31);
+            const bool ok = r < rv;
+            const size_t grow = (size_t)(row0 + (ok ? r : 0));
+            float rs = 1.f;
+            if constexpr (FP8) rs = p.row_scale[grow];
+            bf16_t* crow = C + grow * p.ldc;
+#pragma unroll
+            for (int j = 0; j < TN; j += (EPI == EPI_SWIGLU ? 2 : 1)) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float x[4];
+                    int col;
+                    if constexpr (EPI == EPI_SWIGLU) {
+                        // packed columns alternate gate/up in groups of 32: tile j = gate, j+1 = up
+                        col = ((nt * BN + wn * (BN / 2) + j * 32) >> 1) + 8 * q + chalf;
+                        float cg[4] = {1.f, 1.f, 1.f, 1.f}, cu[4] = {1.f, 1.f, 1.f, 1.f};
+                        if constexpr (FP8) {
+                            if (col < p.N) {
+                                const float4 g4 = *(const float4*)(p.col_scale + (size_t)g * p.ncs + col);
+                                const float4 u4 = *(const float4*)(p.col_scale2 + (size_t)g * p.ncs + col);
+                                cg[0] = g4.x * rs; cg[1] = g4.y * rs; cg[2] = g4.z * rs; cg[3] = g4.w * rs;
+                                cu[0] = u4.x * rs; cu[1] = u4.y * rs; cu[2] = u4.z * rs; cu[3] = u4.w * rs;
+                            }
+                        }
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            float gv = acc[i][j][4 * q + e], uv = acc[i][j + 1][4 * q + e];
+                            if constexpr (FP8) { gv *= cg[e]; uv *= cu[e]; }
+                            x[e] = act_silu(gv) * uv;
+                        }
+                    } else {
+                        col = nt * BN + wn * (BN / 2) + j * 32 + 8 * q + chalf;
+                        float cs[4] = {1.f, 1.f, 1.f, 1.f};
+                        if constexpr (FP8) {
+                            if (col < p.N) {
+                                const float4 c4 = *(const float4*)(p.col_scale + (size_t)g * p.ncs + col);
+                                cs[0] = c4.x * rs; cs[1] = c4.y * rs; cs[2] = c4.z * rs; cs[3] = c4.w * rs;
+                            }
+                        }
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            float v = acc[i][j][4 * q + e];
+                            if constexpr (FP8) v *= cs[e];
+                            if constexpr (EPI == EPI_GELU) v = act_gelu(v);
+                            if constexpr (EPI == EPI_SILU) v = act_silu(v);
+                            x[e] = v;
+                        }
+                    }
+                    if (ok && col < p.N) {
+                        uint2 o;
+                        o.x = (uint32_t)f32_to_bf16(x[0]) | ((uint32_t)f32_to_bf16(x[1]) << 16);
+                        o.y = (uint32_t)f32_to_bf16(x[2]) | ((uint32_t)f32_to_bf16(x[3]) << 16);
+                        *(uint2*)(crow + col) = o;
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---- one-time weight re-tiling: w [E_l,K,N] (N contiguous) -> out [E_l,Npad,K] (K contiguous) -------
+// With w_up, gate and up columns are interleaved in groups of 32: packed col = (n/32)*64 + {0,32} + n%32.
+template <typename T>
+__global__ __launch_bounds__(256) void prepack_kernel(const T* __restrict__ w, const T* __restrict__ w_up, T* __restrict__ out,
+                                                       int K, int N, int Npad) {
+    __shared__ T tile[64][64 + 2];
+    const int e = blockIdx.z;
+    const int k0 = blockIdx.y * 64, n0 = blockIdx.x * 64;  // n0 in source columns
+    const T* src = w + (size_t)e * K * N;
+    const T* src2 = w_up ? w_up + (size_t)e * K * N : nullptr;
+    T* dst = out + (size_t)e * Npad * K;
+    for (int pass = 0; pass < (src2 ? 2 : 1); ++pass) {
+        const T* s = pass ? src2 : src;
+        for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+            const int kk = i / 64, nn = i % 64;
+            tile[kk][nn] = (k0 + kk < K && n0 + nn < N) ? s[(size_t)(k0 + kk) * N + n0 + nn] : (T)0;
+        }
+        __syncthreads();
+        for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+            const int nn = i / 64, kk = i % 64;
+            const int n = n0 + nn;
+            if (n < N && k0 + kk < K) {
+                const int np = src2 ? ((n >> 5) * 64 + pass * 32 + (n & 31)) : n;
+                dst[(size_t)np * K + k0 + kk] = tile[kk][nn];
+            }
+        }
+        __syncthreads();
+    }
+}
+
+template <typename T>
+__global__ void zero_pad_rows_kernel(T* __restrict__ out, int K, int Nreal, int Npad) {
+    // rows [Nreal, Npad) of every expert's packed matrix
+    const int e = blockIdx.y;
+    const size_t n = (size_t)(Npad - Nreal) * K;
+    T* dst = out + ((size_t)e * Npad + Nreal) * K;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = (T)0;
+}
+
+// ---- fp32 path: plain tiled FMA kernel, weights in the reference layout ------------------------------
+// C[rows of g] = epi(A[rows of g] @ W[g] (, A @ Wup[g])); 64x64 tiles, 16x16 threads, 4x4 per thread.
+template <int EPI>
+__global__ __launch_bounds__(256) void grouped_gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ Wt,
+                                                                const float* __restrict__ Wup, float* __restrict__ C,
+                                                                const int32_t* __restrict__ cnt, int E_l, int K, int N,
+                                                                int S_rows) {
+    __shared__ float As[16][64 + 4];
+    __shared__ float Bs[16][64];
+    __shared__ float Us[EPI == EPI_SWIGLU ? 16 : 1][64];
+    __shared__ int s_g, s_row0, s_rv;
+    if (threadIdx.x == 0) {
+        int mt = blockIdx.y, rs = 0, g = 0, found = 0;
+        for (; g < E_l; ++g) {
+            const int c = max(cnt[g], 0);
+            const int t = (c + 63) / 64;
+            if (mt < t) { found = 1; s_row0 = rs + mt * 64; s_rv = min(min(64, c - mt * 64), S_rows - (rs + mt * 64)); break; }
+            mt -= t;
+            rs += c;
+        }
+        s_g = found ? g : -1;
+    }
+    __syncthreads();
+    const int g = s_g;
+    if (g < 0 || s_rv <= 0) return;
+    const int row0 = s_row0, rv = s_rv, n0 = blockIdx.x * 64;
+    const float* W = Wt + (size_t)g * K * N;
+    const float* U = EPI == EPI_SWIGLU ? Wup + (size_t)g * K * N : nullptr;
+    const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+    float acc[4][4] = {}, acu[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += 16) {
+        for (int i = threadIdx.x; i < 64 * 16; i += 256) {
+            const int r = i / 16, kk = i % 16;
+            As[kk][r] = (r < rv && k0 + kk < K) ? A[(size_t)(row0 + r) * K + k0 + kk] : 0.f;
+        }
+        for (int i = threadIdx.x; i < 16 * 64; i += 256) {
+            const int kk = i / 64, nn = i % 64;
+            const bool ok = k0 + kk < K && n0 + nn < N;
+            Bs[kk][nn] = ok ? W[(size_t)(k0 + kk) * N + n0 + nn] : 0.f;
+            if constexpr (EPI == EPI_SWIGLU) Us[kk][nn] = ok ? U[(size_t)(k0 + kk) * N + n0 + nn] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = Bs[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+            if constexpr (EPI == EPI_SWIGLU) {
+                float u[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) u[j] = Us[kk][tx * 4 + j];
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acu[i][j] = fmaf(a[i], u[j], acu[i][j]);
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int r = ty * 4 + i;
+        if (r >= rv) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = n0 + tx * 4 + j;
+            if (c >= N) continue;
+            float x = acc[i][j];
+            if constexpr (EPI == EPI_GELU) x = act_gelu(x);
+            if constexpr (EPI == EPI_SILU) x = act_silu(x);
+            if constexpr (EPI == EPI_SWIGLU) x = act_silu(x) * acu[i][j];
+            C[(size_t)(row0 + r) * N + c] = x;
+        }
+    }
+}
+
+// ---- per-row fp8 quantisation of bf16 rows (one wave per row) -------------------------------------
+__global__ __launch_bounds__(256) void quantize_rows_fp8_kernel(const bf16_t* __restrict__ x, int rows, int cols,
+                                                                 uint8_t* __restrict__ q, float* __restrict__ scale,
+                                                                 const int32_t* __restrict__ n_rows_dev) {
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const int limit = n_rows_dev ? min(rows, *n_rows_dev) : rows;
+    for (int r = blockIdx.x * 4 + wave; r < limit; r += gridDim.x * 4) {
+        const uint4* src = (const uint4*)(x + (size_t)r * cols);
+        const int nv = cols / 8;
+        float amax = 0.f;
+        for (int c = lane; c < nv; c += WAVE) {
+            const uint4 v = src[c];
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                amax = fmaxf(amax, fabsf(__uint_as_float(w[i] << 16)));
+                amax = fmaxf(amax, fabsf(__uint_as_float(w[i] & 0xffff0000u)));
+            }
+        }
+#pragma unroll
+        for (int off = WAVE / 2; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, WAVE));
+        const bool zero = amax == 0.f;
+        const float inv = zero ? 1.f : __fdiv_rn(448.f, amax);
+        if (lane == 0) scale[r] = zero ? 1.f : __fdiv_rn(amax, 448.f);
+        uint2* dst = (uint2*)(q + (size_t)r * cols);
+        for (int c = lane; c < nv; c += WAVE) {
+            const uint4 v = src[c];
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+            float f[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                f[2 * i] = __fmul_rn(__uint_as_float(w[i] << 16), inv);
+                f[2 * i + 1] = __fmul_rn(__uint_as_float(w[i] & 0xffff0000u), inv);
+            }
+            int lo = 0, hi = 0;
+            lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], lo, false);
+            lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
+            hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], hi, false);
+            hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
+            dst[c] = make_uint2((uint32_t)lo, (uint32_t)hi);
+        }
+    }
+}
+
+int num_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
+        if (cus <= 0) cus = 256;
+    }
+    return cus;
+}
+
+int round_up(int a, int b) { return (a + b - 1) / b * b; }
+
+template <bool FP8>
+int launch_gemm(const GemmParams& p, int epi, hipStream_t s) {
+    const int grid = num_cus();
+    const bool small_m = p.S_rows < 1024 * p.E_l;  // average group under four 256-row tiles
+#define GG_LAUNCH(BMv, NWMv, EPIv) grouped_gemm_kernel<BMv, NWMv, EPIv, FP8><<<grid, NWMv * 2 * WAVE, 0, s>>>(p)
+#define GG_EPI(EPIv)                          \
+    do {                                      \
+        if (small_m) GG_LAUNCH(128, 2, EPIv); \
+        else GG_LAUNCH(256, 4, EPIv);         \
+    } while (0)
+    switch (epi) {
+        case EPI_NONE: GG_EPI(EPI_NONE); break;
+        case EPI_GELU: GG_EPI(EPI_GELU); break;
+        case EPI_SILU: GG_EPI(EPI_SILU); break;
+        case EPI_SWIGLU: GG_EPI(EPI_SWIGLU); break;
+        default: return moe_fail(MOE_ERR_INVALID, "grouped_gemm: activation %d", epi);
+    }
+#undef GG_EPI
+#undef GG_LAUNCH
+    return moe_check_launch("grouped_gemm");
+}
+
+int launch_f32(const float* A, const float* W, const float* U, float* C, const int32_t* cnt, int E_l, int K, int N, int S_rows,
+               int epi, hipStream_t s) {
+    if (S_rows == 0) return MOE_OK;
+    dim3 grid(ceil_div(N, 64), ceil_div(S_rows, 64) + E_l);
+    switch (epi) {
+        case EPI_NONE: grouped_gemm_f32_kernel<EPI_NONE><<<grid, 256, 0, s>>>(A, W, U, C, cnt, E_l, K, N, S_rows); break;
+        case EPI_GELU: grouped_gemm_f32_kernel<EPI_GELU><<<grid, 256, 0, s>>>(A, W, U, C, cnt, E_l, K, N, S_rows); break;
+        case EPI_SILU: grouped_gemm_f32_kernel<EPI_SILU><<<grid, 256, 0, s>>>(A, W, U, C, cnt, E_l, K, N, S_rows); break;
+        case EPI_SWIGLU: grouped_gemm_f32_kernel<EPI_SWIGLU><<<grid, 256, 0, s>>>(A, W, U, C, cnt, E_l, K, N, S_rows); break;
+        default: return moe_fail(MOE_ERR_INVALID, "grouped_gemm: activation %d", epi);
+    }
+    return moe_check_launch("grouped_gemm_f32");
+}
+
+template <typename T>
+int launch_prepack(const T* w, const T* w_up, int E_l, int K, int N, T* out, hipStream_t s) {
+    const int n_eff = N * (w_up ? 2 : 1);
+    const int Npad = round_up(n_eff, GG_BN);
+    if (Npad > n_eff) zero_pad_rows_kernel<T><<<dim3(64, E_l), 256, 0, s>>>(out, K, n_eff, Npad);
+    prepack_kernel<T><<<dim3(ceil_div(N, 64), ceil_div(K, 64), E_l), 256, 0, s>>>(w, w_up, out, K, N, Npad);
+    return moe_check_launch("prepack_weights");
+}
+
+}  // namespace moe_gg
+using namespace moe_gg;
+
+extern "C" size_t moe_prepack_bytes(int dtype, int E_l, int K, int N) {
+    if (dtype == MOE_F32) return 0;
+    const size_t es = dtype == MOE_BF16 ? 2 : 1;
+    return (size_t)E_l * (size_t)round_up(N, GG_BN) * (size_t)K * es;
+}
+
+extern "C" int moe_prepack_weights(const void* w, const void* w_up, int dtype, int E_l, int K, int N, void* packed,
+                                   moe_stream_t stream) {
+    MOE_REQUIRE(dtype == MOE_BF16, MOE_ERR_INVALID, "prepack_weights: bf16 only (dtype %d)", dtype);
+    MOE_REQUIRE(E_l > 0 && K > 0 && N > 0 && w && packed, MOE_ERR_INVALID, "prepack_weights: bad arguments");
+    MOE_REQUIRE(!w_up || N % 32 == 0, MOE_ERR_UNSUPPORTED, "prepack_weights: gate/up interleave needs N %% 32 == 0 (N=%d)", N);
+    return launch_prepack<uint16_t>((const uint16_t*)w, (const uint16_t*)w_up, E_l, K, N, (uint16_t*)packed, (hipStream_t)stream);
+}
+
+extern "C" int moe_prepack_weights_fp8(const uint8_t* w, const uint8_t* w_up, int E_l, int K, int N, uint8_t* packed,
+                                       moe_stream_t stream) {
+    MOE_REQUIRE(E_l > 0 && K > 0 && N > 0 && w && packed, MOE_ERR_INVALID, "prepack_weights_fp8: bad arguments");
+    MOE_REQUIRE(!w_up || N % 32 == 0, MOE_ERR_UNSUPPORTED, "prepack_weights_fp8: gate/up interleave needs N %% 32 == 0");
+    return launch_prepack<uint8_t>(w, w_up, E_l, K, N, packed, (hipStream_t)stream);
+}
+
+extern "C" int moe_grouped_gemm(const void* tokens, const void* weights, const int32_t* expert_cnt, int dtype, int S_rows,
+                                int K, int N, int E_l, void* out, void* ws, size_t ws_bytes, moe_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    MOE_REQUIRE(S_rows >= 0 && K > 0 && N > 0 && E_l > 0 && E_l <= GG_MAXG, MOE_ERR_INVALID, "grouped_gemm: bad shape");
+    if (S_rows == 0) return MOE_OK;
+    MOE_REQUIRE(tokens && weights && expert_cnt && out, MOE_ERR_INVALID, "grouped_gemm: null pointer");
+    if (dtype == MOE_F32)
+        return launch_f32((const float*)tokens, (const float*)weights, nullptr, (float*)out, expert_cnt, E_l, K, N, S_rows,
+                          EPI_NONE, s);
+    MOE_REQUIRE(dtype == MOE_BF16, MOE_ERR_INVALID, "grouped_gemm: dtype %d", dtype);
+    MOE_REQUIRE(K % 64 == 0 && N % 8 == 0, MOE_ERR_UNSUPPORTED, "grouped_gemm: bf16 needs K %% 64 == 0 and N %% 8 == 0 (K=%d N=%d)", K, N);
+    MOE_REQUIRE(ws && ws_bytes >= moe_prepack_bytes(dtype, E_l, K, N), MOE_ERR_WORKSPACE, "grouped_gemm: workspace too small");
+    int rc = launch_prepack<uint16_t>((const uint16_t*)weights, nullptr, E_l, K, N, (uint16_t*)ws, s);
+    if (rc) return rc;
+    GemmParams p{};
+    p.A = (const uint8_t*)tokens; p.B = (const uint8_t*)ws; p.C = out; p.cnt = expert_cnt;
+    p.E_l = E_l; p.K = K; p.N = N; p.Npad = round_up(N, GG_BN); p.ldc = N; p.S_rows = S_rows;
+    return launch_gemm<false>(p, EPI_NONE, s);
+}
+
+extern "C" int moe_grouped_mlp(const void* tokens, const int32_t* expert_cnt, int dtype, int S_rows, int H, int F, int E_l,
+                               int act, const void* w1, const void* w_up, const void* w2, void* hidden_ws, void* out,
+                               moe_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    MOE_REQUIRE(S_rows >= 0 && H > 0 && F > 0 && E_l > 0 && E_l <= GG_MAXG, MOE_ERR_INVALID, "grouped_mlp: bad shape");
+    MOE_REQUIRE(act == EPI_GELU || act == EPI_SILU || act == EPI_SWIGLU || act == EPI_NONE, MOE_ERR_INVALID,
+                "grouped_mlp: activation %d", act);
+    if (S_rows == 0) return MOE_OK;
+    MOE_REQUIRE(tokens && expert_cnt && w1 && w2 && hidden_ws && out, MOE_ERR_INVALID, "grouped_mlp: null pointer");
+    if (dtype == MOE_F32) {
+        MOE_REQUIRE(act != EPI_SWIGLU || w_up, MOE_ERR_INVALID, "grouped_mlp: swiglu needs w_up");
+        int rc = launch_f32((const float*)tokens, (const float*)w1, (const float*)w_up, (float*)hidden_ws, expert_cnt, E_l, H,
+                            F, S_rows, act, s);
+        if (rc) return rc;
+        return launch_f32((const float*)hidden_ws, (const float*)w2, nullptr, (float*)out, expert_cnt, E_l, F, H, S_rows,
+                          EPI_NONE, s);
+    }
+    MOE_REQUIRE(dtype == MOE_BF16, MOE_ERR_INVALID, "grouped_mlp: dtype %d", dtype);
+    MOE_REQUIRE(w_up == nullptr, MOE_ERR_INVALID, "grouped_mlp: bf16 takes gate/up interleaved in w1 (w_up must be NULL)");
+    MOE_REQUIRE(H % 64 == 0 && F % 64 == 0, MOE_ERR_UNSUPPORTED, "grouped_mlp: bf16 needs H, F multiples of 64 (H=%d F=%d)", H, F);
+    GemmParams p{};
+    p.A = (const uint8_t*)tokens; p.B = (const uint8_t*)w1; p.C = hidden_ws; p.cnt = expert_cnt;
+    p.E_l = E_l; p.K = H; p.N = F; p.ldc = F; p.S_rows = S_rows;
+    p.Npad = round_up(act == EPI_SWIGLU ? 2 * F : F, GG_BN);
+    int rc = launch_gemm<false>(p, act, s);
+    if (rc) return rc;
+    GemmParams q{};
+    q.A = (const uint8_t*)hidden_ws; q.B = (const uint8_t*)w2; q.C = out; q.cnt = expert_cnt;
+    q.E_l = E_l; q.K = F; q.N = H; q.Npad = round_up(H, GG_BN); q.ldc = H; q.S_rows = S_rows;
+    return launch_gemm<false>(q, EPI_NONE, s);
+}
+
+extern "C" int moe_quantize_rows_fp8(const void* x_bf16, int rows, int cols, uint8_t* q, float* scale,
+                                     const int32_t* n_rows_dev, moe_stream_t stream) {
+    MOE_REQUIRE(rows >= 0 && cols > 0 && cols % 8 == 0, MOE_ERR_INVALID, "quantize_rows_fp8: cols must be a multiple of 8");
+    if (rows == 0) return MOE_OK;
+    MOE_REQUIRE(x_bf16 && q && scale, MOE_ERR_INVALID, "quantize_rows_fp8: null pointer");
+    const int blocks = min(ceil_div(rows, 4), 65535 * 8);
+    quantize_rows_fp8_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>((const bf16_t*)x_bf16, rows, cols, q, scale, n_rows_dev);
+    return moe_check_launch("quantize_rows_fp8");
+}
+
+extern "C" int moe_grouped_mlp_fp8(const void* tokens_bf16, const int32_t* expert_cnt, int S_rows, int H, int F, int E_l,
+                                   const uint8_t* wgu_packed, const float* sg, const float* su, const uint8_t* wd_packed,
+                                   const float* sd, uint8_t* xq_ws, float* xs_ws, void* h_ws, uint8_t* hq_ws, float* hs_ws,
+                                   void* out, moe_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    MOE_REQUIRE(S_rows >= 0 && H > 0 && F > 0 && E_l > 0 && E_l <= GG_MAXG, MOE_ERR_INVALID, "grouped_mlp_fp8: bad shape");
+    MOE_REQUIRE(H % 128 == 0 && F % 128 == 0, MOE_ERR_UNSUPPORTED, "grouped_mlp_fp8: needs H, F multiples of 128 (H=%d F=%d)", H, F);
+    if (S_rows == 0) return MOE_OK;
+    MOE_REQUIRE(tokens_bf16 && expert_cnt && wgu_packed && sg && su && wd_packed && sd && xq_ws && xs_ws && h_ws && hq_ws &&
+                    hs_ws && out, MOE_ERR_INVALID, "grouped_mlp_fp8: null pointer");
+    int rc = moe_quantize_rows_fp8(tokens_bf16, S_rows, H, xq_ws, xs_ws, nullptr, stream);
+    if (rc) return rc;
+    GemmParams p{};
+    p.A = xq_ws; p.B = wgu_packed; p.C = h_ws; p.cnt = expert_cnt; p.row_scale = xs_ws; p.col_scale = sg; p.col_scale2 = su;
+    p.E_l = E_l; p.K = H; p.N = F; p.Npad = round_up(2 * F, GG_BN); p.ldc = F; p.S_rows = S_rows; p.ncs = F;
+    rc = launch_gemm<true>(p, EPI_SWIGLU, s);
+    if (rc) return rc;
+    rc = moe_quantize_rows_fp8(h_ws, S_rows, F, hq_ws, hs_ws, nullptr, stream);
+    if (rc) return rc;
+    GemmParams q{};
+    q.A = hq_ws; q.B = wd_packed; q.C = out; q.cnt = expert_cnt; q.row_scale = hs_ws; q.col_scale = sd;
+    q.E_l = E_l; q.K = F; q.N = H; q.Npad = round_up(H, GG_BN); q.ldc = H; q.S_rows = S_rows; q.ncs = H;
+    return launch_gemm<true>(q, EPI_NONE, s);
+}

@@ -1,0 +1,249 @@
+// Router: logits = x @ W_r (+ bias) with a pinned fp32 reduction order, then softmax gates
+// and top-k with wavefront-level reductions.
+//
+// Replaces the device work of `F.softmax(torch.einsum('th,he->te', tokens, router), dim=-1)`
+// followed by `torch.topk(..., topk)` in the reference (utils.py:200-202).
+//
+// Reduction order (what makes the indices reproducible bit-for-bit on a CPU):
+//   logit[t,e] = bias[e] + chain,  chain = fmaf(x[t,h], w[h,e], chain) for h = 0..H-1, chain0 = +0.0f
+// Every (t,e) chain lives in ONE thread; H is walked in ascending order through LDS tiles, so no
+// cross-lane or cross-block partial sums exist.  MFMA is deliberately not used here: its internal
+// summation order is not specified.
+#include "common.h"
+
+namespace {
+
+constexpr int RT_THREADS = 256;
+constexpr int RT_KC = 32;  // h per LDS tile
+constexpr int RT_TB = 64;  // tokens per block
+
+template <typename XT>
+struct VecLoad;
+template <>
+struct VecLoad<bf16_t> {
+    static constexpr int N = 8;
+    __device__ static void load(const bf16_t* p, float* out) {
+        uint4 v = *reinterpret_cast<const uint4*>(p);
+        uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            out[2 * i] = __uint_as_float(w[i] << 16);
+            out[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+};
+template <>
+struct VecLoad<float> {
+    static constexpr int N = 4;
+    __device__ static void load(const float* p, float* out) {
+        float4 v = *reinterpret_cast<const float4*>(p);
+        out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+    }
+};
+
+// Block = 256 threads = NEX expert-threads x NTY token-threads; thread computes TT tokens x EE experts.
+template <typename XT, int TT, int EE, int NEX>
+__global__ __launch_bounds__(RT_THREADS) void route_logits_kernel(const XT* __restrict__ x,
+                                                                   const XT* __restrict__ w,
+                                                                   const float* __restrict__ bias,
+                                                                   float* __restrict__ logits, int T, int H, int E) {
+    constexpr int NTY = RT_THREADS / NEX;
+    constexpr int TB = NTY * TT;
+    constexpr int EB = NEX * EE;
+    static_assert(TB == RT_TB, "token tile");
+    constexpr int XS = TB + 4;  // padded row stride (keeps 16-byte alignment of the per-thread token vector)
+    __shared__ __align__(16) float xs[RT_KC][XS];
+    __shared__ __align__(16) float ws[RT_KC][EB];
+
+    const int tid = threadIdx.x;
+    const int tx = tid % NEX, ty = tid / NEX;
+    const int t0 = blockIdx.x * TB, e0 = blockIdx.y * EB;
+
+    float acc[TT][EE];
+#pragma unroll
+    for (int i = 0; i < TT; ++i)
+#pragma unroll
+        for (int j = 0; j < EE; ++j) acc[i][j] = 0.0f;
+
+    constexpr int VN = VecLoad<XT>::N;
+    constexpr int CH_PER_TOK = RT_KC / VN;
+    constexpr int X_CHUNKS = TB * CH_PER_TOK;
+
+    for (int k0 = 0; k0 < H; k0 += RT_KC) {
+        const int kmax = min(RT_KC, H - k0);
+        // stage x tile [TB tokens][KC] -> xs[k][token] as fp32
+        for (int c = tid; c < X_CHUNKS; c += RT_THREADS) {
+            const int tt = c / CH_PER_TOK, kc = (c % CH_PER_TOK) * VN;
+            const int t = t0 + tt;
+            float v[VN];
+            if (t < T && k0 + kc + VN <= H) {
+                VecLoad<XT>::load(x + (size_t)t * H + k0 + kc, v);
+            } else {
+#pragma unroll
+                for (int j = 0; j < VN; ++j)
+                    v[j] = (t < T && k0 + kc + j < H) ? load_f32<XT>(x + (size_t)t * H + k0 + kc + j) : 0.0f;
+            }
+#pragma unroll
+            for (int j = 0; j < VN; ++j) xs[kc + j][tt] = v[j];
+        }
+        // stage router tile [KC][EB]
+        for (int c = tid; c < RT_KC * EB; c += RT_THREADS) {
+            const int kk = c / EB, ee = c % EB;
+            const int e = e0 + ee;
+            ws[kk][ee] = (kk < kmax && e < E) ? load_f32<XT>(w + (size_t)(k0 + kk) * E + e) : 0.0f;
+        }
+        __syncthreads();
+        if (kmax == RT_KC) {
+#pragma unroll 8
+            for (int kk = 0; kk < RT_KC; ++kk) {
+                float xv[TT], wv[EE];
+#pragma unroll
+                for (int i = 0; i < TT; ++i) xv[i] = xs[kk][ty * TT + i];
+#pragma unroll
+                for (int j = 0; j < EE; ++j) wv[j] = ws[kk][tx * EE + j];
+#pragma unroll
+                for (int i = 0; i < TT; ++i)
+#pragma unroll
+                    for (int j = 0; j < EE; ++j) acc[i][j] = fmaf(xv[i], wv[j], acc[i][j]);
+            }
+        } else {
+            for (int kk = 0; kk < kmax; ++kk) {
+#pragma unroll
+                for (int i = 0; i < TT; ++i)
+#pragma unroll
+                    for (int j = 0; j < EE; ++j)
+                        acc[i][j] = fmaf(xs[kk][ty * TT + i], ws[kk][tx * EE + j], acc[i][j]);
+            }
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < TT; ++i) {
+        const int t = t0 + ty * TT + i;
+        if (t >= T) continue;
+#pragma unroll
+        for (int j = 0; j < EE; ++j) {
+            const int e = e0 + tx * EE + j;
+            if (e < E) logits[(size_t)t * E + e] = bias ? __fadd_rn(acc[i][j], bias[e]) : acc[i][j];
+        }
+    }
+}
+
+// Softmax gates + top-k.  G lanes cooperate on one token (G = 8,16,32,64); lane gl holds experts
+// gl, gl+G, gl+2G, ...  Selection key: (logit descending, expert id ascending).
+constexpr int TK_MAXV = 8;  // values per lane -> E <= 8*G
+
+template <int G>
+__global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict__ logits, int32_t* __restrict__ idx,
+                                                         float* __restrict__ gate, int T, int E, int k) {
+    constexpr int TPW = WAVE / G;  // tokens per wave
+    const int lane = lane_id();
+    const int gl = lane % G;
+    const int wave_global = (blockIdx.x * blockDim.x + threadIdx.x) / WAVE;
+    const int n_waves = (gridDim.x * blockDim.x) / WAVE;
+    const float NEG_INF = -__builtin_huge_valf();
+
+    for (int tbase = wave_global * TPW; tbase < T; tbase += n_waves * TPW) {
+        const int t = tbase + lane / G;
+        const bool live = t < T;
+        float v[TK_MAXV];
+#pragma unroll
+        for (int i = 0; i < TK_MAXV; ++i) {
+            const int e = gl + i * G;
+            v[i] = (live && e < E) ? logits[(size_t)t * E + e] : NEG_INF;
+        }
+        unsigned taken = 0;
+        float row_max = 0.f;
+        float sel_v[MOE_MAX_TOPK];
+        int sel_e[MOE_MAX_TOPK];
+#pragma unroll
+        for (int j = 0; j < MOE_MAX_TOPK; ++j) {
+            if (j < k) {
+                float bv = NEG_INF;
+                int be = 0x7fffffff;
+#pragma unroll
+                for (int i = 0; i < TK_MAXV; ++i) {
+                    const int e = gl + i * G;
+                    const bool ok = (e < E) && !((taken >> i) & 1u);
+                    // ascending e within the lane: strict > keeps the lower id on ties
+                    if (ok && (be == 0x7fffffff || v[i] > bv)) { bv = v[i]; be = e; }
+                }
+#pragma unroll
+                for (int off = G / 2; off >= 1; off >>= 1) {
+                    const float ov = __shfl_xor(bv, off, WAVE);
+                    const int oe = __shfl_xor(be, off, WAVE);
+                    if (oe != 0x7fffffff && (be == 0x7fffffff || ov > bv || (ov == bv && oe < be))) { bv = ov; be = oe; }
+                }
+                if (be != 0x7fffffff && (be % G) == gl) taken |= 1u << (be / G);
+                sel_v[j] = bv;
+                sel_e[j] = be;
+                if (j == 0) row_max = bv;
+            }
+        }
+        // softmax denominator: per-lane ascending partial sum, then xor butterfly
+        float part = 0.f;
+#pragma unroll
+        for (int i = 0; i < TK_MAXV; ++i) {
+            const int e = gl + i * G;
+            if (e < E) part += expf(v[i] - row_max);
+        }
+#pragma unroll
+        for (int off = G / 2; off >= 1; off >>= 1) part += __shfl_xor(part, off, WAVE);
+        if (live && gl == 0) {
+#pragma unroll
+            for (int j = 0; j < MOE_MAX_TOPK; ++j) {
+                if (j < k) {
+                    idx[(size_t)t * k + j] = sel_e[j] == 0x7fffffff ? 0 : sel_e[j];
+                    gate[(size_t)t * k + j] = expf(sel_v[j] - row_max) / part;
+                }
+            }
+        }
+    }
+}
+
+template <typename XT>
+int launch_logits(const XT* x, const XT* w, const float* bias, float* logits, int T, int H, int E, hipStream_t s) {
+    const int gx = ceil_div(T, RT_TB);
+    if (E <= 8) {
+        route_logits_kernel<XT, 1, 2, 4><<<dim3(gx, ceil_div(E, 8)), RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
+    } else if (E <= 16) {
+        route_logits_kernel<XT, 1, 4, 4><<<dim3(gx, 1), RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
+    } else if (E <= 32) {
+        route_logits_kernel<XT, 2, 4, 8><<<dim3(gx, 1), RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
+    } else {
+        route_logits_kernel<XT, 4, 4, 16><<<dim3(gx, ceil_div(E, 64)), RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
+    }
+    return moe_check_launch("route_logits");
+}
+
+}  // namespace
+
+extern "C" int moe_route_topk(const void* x, const void* router, const float* bias, int dtype, int T, int H, int E,
+                              int k, float* logits_ws, int32_t* topk_idx, float* topk_gate, moe_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    MOE_REQUIRE(T >= 0 && H > 0 && E > 0, MOE_ERR_INVALID, "route_topk: bad shape T=%d H=%d E=%d", T, H, E);
+    MOE_REQUIRE(k >= 1 && k <= E, MOE_ERR_INVALID, "route_topk: topk=%d must be in [1, E=%d]", k, E);
+    MOE_REQUIRE(k <= MOE_MAX_TOPK, MOE_ERR_UNSUPPORTED, "route_topk: topk=%d > %d", k, MOE_MAX_TOPK);
+    MOE_REQUIRE(E <= MOE_MAX_EXPERTS, MOE_ERR_UNSUPPORTED, "route_topk: E=%d > %d", E, MOE_MAX_EXPERTS);
+    MOE_REQUIRE(dtype == MOE_F32 || dtype == MOE_BF16, MOE_ERR_INVALID, "route_topk: dtype %d", dtype);
+    MOE_REQUIRE((H * dtype_size(dtype)) % 16 == 0, MOE_ERR_INVALID, "route_topk: rows must be 16-byte multiples (H=%d)", H);
+    if (T == 0) return MOE_OK;
+    MOE_REQUIRE(x && router && logits_ws && topk_idx && topk_gate, MOE_ERR_INVALID, "route_topk: null pointer");
+    int rc = dtype == MOE_F32
+                 ? launch_logits<float>((const float*)x, (const float*)router, bias, logits_ws, T, H, E, s)
+                 : launch_logits<bf16_t>((const bf16_t*)x, (const bf16_t*)router, bias, logits_ws, T, H, E, s);
+    if (rc) return rc;
+    int G = 8;
+    while (G < 64 && G < E) G *= 2;
+    if (E > 8 * G) return moe_fail(MOE_ERR_UNSUPPORTED, "route_topk: E=%d too large", E);
+    const int tpw = WAVE / G;
+    const int waves = ceil_div(T, tpw);
+    const int blocks = min(ceil_div(waves, 4), 4096);
+    switch (G) {
+        case 8: topk_gate_kernel<8><<<blocks, 256, 0, s>>>(logits_ws, topk_idx, topk_gate, T, E, k); break;
+        case 16: topk_gate_kernel<16><<<blocks, 256, 0, s>>>(logits_ws, topk_idx, topk_gate, T, E, k); break;
+        case 32: topk_gate_kernel<32><<<blocks, 256, 0, s>>>(logits_ws, topk_idx, topk_gate, T, E, k); break;
+        default: topk_gate_kernel<64><<<blocks, 256, 0, s>>>(logits_ws, topk_idx, topk_gate, T, E, k); break;
+    }
+    return moe_check_launch("topk_gate");
+}

@@ -1,0 +1,78 @@
+"""Expert compute with the reference's ``expert`` signature (layers/expert.py:6-66), plus the full
+expert MLP the workloads define (Linear-act-Linear, SwiGLU, fp8) which the reference lacks.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from .. import ops
+from ..utils import _assert_cuda_int32
+
+
+class Expert(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx, tokens, weights, local_expert_cnt, aggregrate_exp_cnt):
+        """tokens [S,H], weights [E_local,H,F], local_expert_cnt [E_local] int32, total expert count
+        (unused by the math, kept for the signature) -> [S,F] (layers/expert.py:20-29,43,60)."""
+        assert tokens.is_cuda, "tokens must be CUDA"
+        _assert_cuda_int32(local_expert_cnt, "local_expert_cnt")
+        assert weights.shape[0] == local_expert_cnt.numel(), "one row count per local expert"
+        return ops.grouped_gemm(tokens.contiguous(), weights.contiguous(), local_expert_cnt.contiguous())
+
+    @staticmethod
+    def backward(ctx, do):
+        raise NotImplementedError("Backward pass not implemented yet.")
+
+
+expert = Expert.apply
+
+
+@dataclass
+class ExpertWeights:
+    """Weights of the local experts, prepared once for the kernels.
+
+    act in {"gelu","silu"}: y = act(x W1) W2.  act == "swiglu": y = (silu(x Wg) * (x Wu)) Wd.
+    bf16: re-tiled for the MFMA kernels; fp32: reference layout; fp8: e4m3 codes + per-channel scales.
+    """
+    act: str
+    hidden: int
+    ffn: int
+    e_local: int
+    dtype: torch.dtype
+    w1: torch.Tensor
+    w2: torch.Tensor
+    w_up: Optional[torch.Tensor] = None
+    scales: Optional[tuple] = None  # fp8: (sg, su, sd)
+
+    @classmethod
+    def prepare(cls, act: str, w1: torch.Tensor, w2: torch.Tensor, w_up: Optional[torch.Tensor] = None):
+        e_l, H, F = w1.shape
+        if w1.dtype == torch.float32:
+            return cls(act, H, F, e_l, w1.dtype, w1.contiguous(), w2.contiguous(),
+                       None if w_up is None else w_up.contiguous())
+        p1 = ops.prepack_weights(w1.contiguous(), None if w_up is None else w_up.contiguous())
+        p2 = ops.prepack_weights(w2.contiguous())
+        return cls(act, H, F, e_l, w1.dtype, p1, p2)
+
+    @classmethod
+    def prepare_fp8(cls, wg_q, sg, wu_q, su, wd_q, sd):
+        """e4m3 codes (uint8) [E_l,H,F] x2 and [E_l,F,H] with fp32 per-output-channel scales."""
+        e_l, H, F = wg_q.shape
+        p1 = ops.prepack_weights_fp8(wg_q.contiguous(), wu_q.contiguous())
+        p2 = ops.prepack_weights_fp8(wd_q.contiguous())
+        return cls("swiglu", H, F, e_l, torch.uint8, p1, p2, None, (sg.contiguous(), su.contiguous(), sd.contiguous()))
+
+
+def expert_mlp(tokens: torch.Tensor, weights: ExpertWeights, local_expert_cnt: torch.Tensor) -> torch.Tensor:
+    """Full expert MLP on expert-major rows -> [S,H]."""
+    assert tokens.is_cuda, "tokens must be CUDA"
+    _assert_cuda_int32(local_expert_cnt, "local_expert_cnt")
+    if weights.dtype == torch.uint8:
+        sg, su, sd = weights.scales
+        return ops.grouped_mlp_fp8(tokens.contiguous(), local_expert_cnt, weights.ffn, weights.w1, sg, su, weights.w2, sd)
+    return ops.grouped_mlp(tokens.contiguous(), local_expert_cnt, weights.act, weights.w1, weights.w2, weights.w_up,
+                           F=weights.ffn)

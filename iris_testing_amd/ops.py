@@ -1,0 +1,354 @@
+"""Tensor-level wrappers over the C ABI (one function per entry point of include/moe_gfx950.h).
+
+PyTorch is used for device memory and the current stream only; every computation happens in
+the HIP kernels.  Outputs and workspaces are allocated here (the C ABI itself allocates nothing)
+unless the caller passes them in.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib as L
+
+
+def _req_cuda(t: torch.Tensor, name: str) -> None:
+    assert t.is_cuda, f"{name} must be CUDA"
+    assert t.is_contiguous(), f"{name} must be contiguous"
+
+
+def _req_i32(t: torch.Tensor, name: str) -> None:
+    _req_cuda(t, name)
+    assert t.dtype == torch.int32, f"{name} must be int32"
+
+
+def _i32(n, device) -> torch.Tensor:
+    return torch.empty(n, dtype=torch.int32, device=device)
+
+
+# ---- a1 -------------------------------------------------------------------------------------
+def route_topk(x: torch.Tensor, router: torch.Tensor, topk: int, bias: Optional[torch.Tensor] = None
+               ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(topk_idx int32 [T,k], topk_gate fp32 [T,k], logits fp32 [T,E])."""
+    _req_cuda(x, "tokens")
+    _req_cuda(router, "router")
+    assert x.dtype == router.dtype, "tokens and router must share a dtype"
+    T, H = x.shape
+    H2, E = router.shape
+    assert H == H2, "router must be [H, E]"
+    if bias is not None:
+        _req_cuda(bias, "bias")
+        assert bias.dtype == torch.float32 and bias.shape == (E,)
+    dev = x.device
+    logits = torch.empty((T, E), dtype=torch.float32, device=dev)
+    idx = torch.empty((T, topk), dtype=torch.int32, device=dev)
+    gate = torch.empty((T, topk), dtype=torch.float32, device=dev)
+    L.check(L.lib().moe_route_topk(L.ptr(x), L.ptr(router), L.ptr(bias), L.dtype_code(x.dtype), T, H, E, topk,
+                                   L.ptr(logits), L.ptr(idx), L.ptr(gate), L.stream_ptr()))
+    return idx, gate, logits
+
+
+# ---- a2/a4/a5/a6/a7 -------------------------------------------------------------------------
+@dataclass
+class Counts:
+    send_counts: torch.Tensor   # [W,E_l] i32
+    expert_offs: torch.Tensor   # [W,E_l] i32
+    dst_sizes: torch.Tensor     # [W] i32
+    dst_offsets: torch.Tensor   # [W] i32
+    caps: torch.Tensor          # [2] i32: max(1,max dst_sizes), max(1,max send_counts)
+    pos: torch.Tensor           # [T,k] i32 payload row of slot (t,kk)
+    row_token: torch.Tensor     # [T*k] i32 token of payload row
+
+
+def count_and_offsets(topk_idx: torch.Tensor, num_experts_total: int, world_size: int) -> Counts:
+    _req_i32(topk_idx, "topk_idx")
+    assert num_experts_total % world_size == 0, "num_experts_total must be divisible by world_size"
+    T, k = topk_idx.shape
+    E, W = num_experts_total, world_size
+    dev = topk_idx.device
+    e_l = E // W
+    out = Counts(_i32((W, e_l), dev), _i32((W, e_l), dev), _i32((W,), dev), _i32((W,), dev), _i32((2,), dev),
+                 _i32((T, k), dev), _i32((T * k,), dev))
+    nbytes = L.lib().moe_count_workspace_bytes(T, k, E)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    L.check(L.lib().moe_count_and_offsets(L.ptr(topk_idx), T, k, E, W, L.ptr(out.send_counts), L.ptr(out.expert_offs),
+                                          L.ptr(out.dst_sizes), L.ptr(out.dst_offsets), L.ptr(out.caps), L.ptr(out.pos),
+                                          L.ptr(out.row_token), L.ptr(ws), nbytes, L.stream_ptr()))
+    return out
+
+
+def max_floor1(values: torch.Tensor) -> torch.Tensor:
+    _req_i32(values, "values")
+    out = _i32((1,), values.device)
+    L.check(L.lib().moe_max_floor1(L.ptr(values), values.numel(), L.ptr(out), L.stream_ptr()))
+    return out
+
+
+# ---- a3 / a8 --------------------------------------------------------------------------------
+def pack_payload(x: torch.Tensor, row_token: torch.Tensor) -> torch.Tensor:
+    _req_cuda(x, "tokens")
+    _req_i32(row_token, "row_token")
+    T, H = x.shape
+    R = row_token.numel()
+    out = torch.empty((R, H), dtype=x.dtype, device=x.device)
+    L.check(L.lib().moe_pack_payload(L.ptr(x), L.dtype_code(x.dtype), T, H, L.ptr(row_token), R, L.ptr(out),
+                                     L.stream_ptr()))
+    return out
+
+
+def pack_fixed_m(x: torch.Tensor, row_token: torch.Tensor, dst_sizes: torch.Tensor, dst_offsets: torch.Tensor,
+                 M: int, out: Optional[torch.Tensor] = None, map_ws: Optional[torch.Tensor] = None,
+                 status: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """send [W,M,H]: rows of every destination in (el, token) order, zero padded to M."""
+    _req_cuda(x, "tokens")
+    _req_i32(row_token, "row_token")
+    _req_i32(dst_sizes, "dst_sizes")
+    _req_i32(dst_offsets, "dst_offsets")
+    T, H = x.shape
+    W = dst_sizes.numel()
+    if out is None:
+        out = torch.empty((W, M, H), dtype=x.dtype, device=x.device)
+    assert out.shape == (W, M, H) and out.dtype == x.dtype and out.is_contiguous()
+    if map_ws is None:
+        map_ws = _i32((W * M,), x.device)
+    L.check(L.lib().moe_pack(L.ptr(x), L.dtype_code(x.dtype), T, H, L.ptr(row_token), L.ptr(dst_sizes),
+                             L.ptr(dst_offsets), W, M, L.ptr(out), L.ptr(map_ws), L.ptr(status), L.stream_ptr()))
+    return out
+
+
+# ---- a9 / a10 -------------------------------------------------------------------------------
+def _map_ws(W, E_l, n_out, device, map_ws=None):
+    need = L.lib().moe_recv_map_ints(W, E_l, n_out)
+    if map_ws is None:
+        return _i32((need,), device)
+    assert map_ws.dtype == torch.int32 and map_ws.numel() >= need and map_ws.is_cuda
+    return map_ws
+
+
+def unpack_token_buf(recv: torch.Tensor, recv_counts: torch.Tensor, capacity: int,
+                     token_buf: Optional[torch.Tensor] = None, pca: Optional[torch.Tensor] = None,
+                     status: Optional[torch.Tensor] = None, map_ws=None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """recv [W,M,H] + recv_counts [W,E_l] -> (token_buf [E_l,W,CAP,H] zero padded, pca [E_l,W])."""
+    _req_cuda(recv, "recv")
+    _req_i32(recv_counts, "recv_counts")
+    W, M, H = recv.shape
+    W2, E_l = recv_counts.shape
+    assert W == W2
+    dev = recv.device
+    if token_buf is None:
+        token_buf = torch.empty((E_l, W, capacity, H), dtype=recv.dtype, device=dev)
+    if tuple(token_buf.shape) != (E_l, W, capacity, H):
+        raise ValueError(f"token_buf shape {tuple(token_buf.shape)} mismatch expected ({E_l},{W},{capacity},{H}).")
+    if pca is None:
+        pca = _i32((E_l, W), dev)
+    ws = _map_ws(W, E_l, E_l * W * capacity, dev, map_ws)
+    L.check(L.lib().moe_unpack_token_buf(L.ptr(recv), L.dtype_code(recv.dtype), W, M, H, L.ptr(recv_counts), E_l,
+                                         capacity, L.ptr(token_buf), L.ptr(pca), L.ptr(ws), L.ptr(status),
+                                         L.stream_ptr()))
+    return token_buf, pca
+
+
+def reorder_flat(flat: torch.Tensor, recv_counts: torch.Tensor, capacity: int, token_buf: torch.Tensor,
+                 status: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _req_cuda(flat, "recv_payload_flat")
+    _req_i32(recv_counts, "recv_counts")
+    R, H = flat.shape
+    W, E_l = recv_counts.shape
+    ws = _map_ws(W, E_l, E_l * W * capacity, flat.device)
+    L.check(L.lib().moe_reorder_flat_to_token_buf(L.ptr(flat), L.dtype_code(flat.dtype), R, H, L.ptr(recv_counts), W,
+                                                  E_l, capacity, L.ptr(token_buf), L.ptr(ws), L.ptr(status),
+                                                  L.stream_ptr()))
+    return token_buf
+
+
+def shuffle_rows(token_buf: torch.Tensor, pca: torch.Tensor, S_rows: int, out: Optional[torch.Tensor] = None,
+                 expert_cnt: Optional[torch.Tensor] = None, map_ws=None) -> Tuple[torch.Tensor, torch.Tensor]:
+    _req_cuda(token_buf, "dispatched_tokens")
+    _req_i32(pca, "pca")
+    E_l, W, CAP, H = token_buf.shape
+    assert pca.shape == (E_l, W)
+    dev = token_buf.device
+    if out is None:
+        out = torch.empty((S_rows, H), dtype=token_buf.dtype, device=dev)
+    if expert_cnt is None:
+        expert_cnt = _i32((E_l,), dev)
+    ws = _map_ws(W, E_l, S_rows, dev, map_ws)
+    L.check(L.lib().moe_shuffle(L.ptr(token_buf), L.dtype_code(token_buf.dtype), E_l, W, CAP, H, L.ptr(pca), L.ptr(out),
+                                S_rows, L.ptr(expert_cnt), L.ptr(ws), L.stream_ptr()))
+    return out, expert_cnt
+
+
+def unpack_expert_major(recv: torch.Tensor, recv_counts: torch.Tensor, S_rows: int,
+                        out: Optional[torch.Tensor] = None, expert_cnt: Optional[torch.Tensor] = None,
+                        map_ws=None) -> Tuple[torch.Tensor, torch.Tensor]:
+    _req_cuda(recv, "recv")
+    _req_i32(recv_counts, "recv_counts")
+    W, M, H = recv.shape
+    E_l = recv_counts.shape[1]
+    dev = recv.device
+    if out is None:
+        out = torch.empty((S_rows, H), dtype=recv.dtype, device=dev)
+    if expert_cnt is None:
+        expert_cnt = _i32((E_l,), dev)
+    ws = _map_ws(W, E_l, S_rows, dev, map_ws)
+    L.check(L.lib().moe_unpack_expert_major(L.ptr(recv), L.dtype_code(recv.dtype), W, M, H, L.ptr(recv_counts), E_l,
+                                            L.ptr(out), S_rows, L.ptr(expert_cnt), L.ptr(ws), L.stream_ptr()))
+    return out, expert_cnt
+
+
+# ---- a11 / a12 ------------------------------------------------------------------------------
+def prepack_weights(w: torch.Tensor, w_up: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """[E_l,K,N] (reference layout) -> the MFMA kernels' K-contiguous layout (one-time, per weight)."""
+    _req_cuda(w, "weights")
+    assert w.dtype == torch.bfloat16, "prepack is for bf16 weights (fp32 uses the reference layout as is)"
+    E_l, K, N = w.shape
+    if w_up is not None:
+        _req_cuda(w_up, "w_up")
+        assert w_up.shape == w.shape and w_up.dtype == w.dtype
+    n_eff = N * (2 if w_up is not None else 1)
+    nbytes = L.lib().moe_prepack_bytes(L.MOE_BF16, E_l, K, n_eff)
+    out = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
+    L.check(L.lib().moe_prepack_weights(L.ptr(w), L.ptr(w_up), L.MOE_BF16, E_l, K, N, L.ptr(out), L.stream_ptr()))
+    return out
+
+
+def grouped_gemm(tokens: torch.Tensor, weights: torch.Tensor, expert_cnt: torch.Tensor,
+                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[rows of e] = tokens[rows of e] @ weights[e] (weights in the reference [E_l,K,N] layout)."""
+    _req_cuda(tokens, "tokens")
+    _req_cuda(weights, "weights")
+    _req_i32(expert_cnt, "local_expert_cnt")
+    assert tokens.dtype == weights.dtype
+    S, K = tokens.shape
+    E_l, K2, N = weights.shape
+    assert K == K2 and expert_cnt.numel() == E_l
+    if out is None:
+        out = torch.zeros((S, N), dtype=tokens.dtype, device=tokens.device)
+    code = L.dtype_code(tokens.dtype)
+    nbytes = L.lib().moe_prepack_bytes(code, E_l, K, N)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=tokens.device)
+    L.check(L.lib().moe_grouped_gemm(L.ptr(tokens), L.ptr(weights), L.ptr(expert_cnt), code, S, K, N, E_l, L.ptr(out),
+                                     L.ptr(ws), nbytes, L.stream_ptr()))
+    return out
+
+
+def grouped_mlp(tokens: torch.Tensor, expert_cnt: torch.Tensor, act: str, w1, w2, w_up=None, F: Optional[int] = None,
+                hidden_ws: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Expert MLP on expert-major rows.
+
+    bf16: ``w1``/``w2`` are prepack_weights() results (``w1`` = prepack(Wg, Wu) for swiglu), ``F`` is
+    required.  fp32: ``w1`` [E_l,H,F], ``w_up`` (swiglu only) [E_l,H,F], ``w2`` [E_l,F,H] in the
+    reference layout.
+    """
+    _req_cuda(tokens, "tokens")
+    _req_i32(expert_cnt, "local_expert_cnt")
+    S, H = tokens.shape
+    E_l = expert_cnt.numel()
+    if tokens.dtype == torch.float32:
+        F = w1.shape[2]
+    assert F is not None
+    dev = tokens.device
+    if hidden_ws is None:
+        hidden_ws = torch.empty((S, F), dtype=tokens.dtype, device=dev)
+    if out is None:
+        out = torch.zeros((S, H), dtype=tokens.dtype, device=dev)
+    L.check(L.lib().moe_grouped_mlp(L.ptr(tokens), L.ptr(expert_cnt), L.dtype_code(tokens.dtype), S, H, F, E_l,
+                                    L.ACT[act], L.ptr(w1), L.ptr(w_up), L.ptr(w2), L.ptr(hidden_ws), L.ptr(out),
+                                    L.stream_ptr()))
+    return out
+
+
+def prepack_weights_fp8(w: torch.Tensor, w_up: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """uint8 e4m3 codes [E_l,K,N] -> packed layout (1 byte per element)."""
+    _req_cuda(w, "weights")
+    assert w.dtype == torch.uint8
+    E_l, K, N = w.shape
+    n_eff = N * (2 if w_up is not None else 1)
+    nbytes = L.lib().moe_prepack_bytes(2, E_l, K, n_eff)
+    out = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
+    L.check(L.lib().moe_prepack_weights_fp8(L.ptr(w), L.ptr(w_up), E_l, K, N, L.ptr(out), L.stream_ptr()))
+    return out
+
+
+def quantize_rows_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    _req_cuda(x, "x")
+    assert x.dtype == torch.bfloat16
+    R, C = x.shape
+    q = torch.empty((R, C), dtype=torch.uint8, device=x.device)
+    s = torch.empty((R,), dtype=torch.float32, device=x.device)
+    L.check(L.lib().moe_quantize_rows_fp8(L.ptr(x), R, C, L.ptr(q), L.ptr(s), None, L.stream_ptr()))
+    return q, s
+
+
+def grouped_mlp_fp8(tokens: torch.Tensor, expert_cnt: torch.Tensor, F: int, wgu_packed, sg, su, wd_packed, sd,
+                    ws: Optional[dict] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _req_cuda(tokens, "tokens")
+    assert tokens.dtype == torch.bfloat16
+    S, H = tokens.shape
+    E_l = expert_cnt.numel()
+    dev = tokens.device
+    if ws is None:
+        ws = fp8_workspace(S, H, F, dev)
+    if out is None:
+        out = torch.zeros((S, H), dtype=torch.bfloat16, device=dev)
+    L.check(L.lib().moe_grouped_mlp_fp8(L.ptr(tokens), L.ptr(expert_cnt), S, H, F, E_l, L.ptr(wgu_packed), L.ptr(sg),
+                                        L.ptr(su), L.ptr(wd_packed), L.ptr(sd), L.ptr(ws["xq"]), L.ptr(ws["xs"]),
+                                        L.ptr(ws["h"]), L.ptr(ws["hq"]), L.ptr(ws["hs"]), L.ptr(out), L.stream_ptr()))
+    return out
+
+
+def fp8_workspace(S: int, H: int, F: int, dev) -> dict:
+    return {
+        "xq": torch.empty((S, H), dtype=torch.uint8, device=dev),
+        "xs": torch.empty((S,), dtype=torch.float32, device=dev),
+        "h": torch.empty((S, F), dtype=torch.bfloat16, device=dev),
+        "hq": torch.empty((S, F), dtype=torch.uint8, device=dev),
+        "hs": torch.empty((S,), dtype=torch.float32, device=dev),
+    }
+
+
+# ---- a13 ------------------------------------------------------------------------------------
+def return_pack(y: torch.Tensor, recv_counts: torch.Tensor, M: int, out: Optional[torch.Tensor] = None,
+                map_ws=None) -> torch.Tensor:
+    _req_cuda(y, "y")
+    _req_i32(recv_counts, "recv_counts")
+    S, H = y.shape
+    W, E_l = recv_counts.shape
+    if out is None:
+        out = torch.empty((W, M, H), dtype=y.dtype, device=y.device)
+    ws = _map_ws(W, E_l, W * M, y.device, map_ws)
+    L.check(L.lib().moe_return_pack(L.ptr(y), L.dtype_code(y.dtype), S, H, L.ptr(recv_counts), W, E_l, M, L.ptr(out),
+                                    L.ptr(ws), L.stream_ptr()))
+    return out
+
+
+def combine(ret: torch.Tensor, topk_idx: torch.Tensor, pos: torch.Tensor, gate: torch.Tensor,
+            dst_offsets: torch.Tensor, e_local: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _req_cuda(ret, "ret")
+    _req_i32(topk_idx, "topk_idx")
+    _req_i32(pos, "pos")
+    _req_i32(dst_offsets, "dst_offsets")
+    _req_cuda(gate, "gate")
+    assert gate.dtype == torch.float32
+    W, M, H = ret.shape
+    T, k = topk_idx.shape
+    if out is None:
+        out = torch.empty((T, H), dtype=ret.dtype, device=ret.device)
+    L.check(L.lib().moe_combine(L.ptr(ret), L.dtype_code(ret.dtype), W, M, H, L.ptr(topk_idx), L.ptr(pos), L.ptr(gate),
+                                L.ptr(dst_offsets), T, k, e_local, L.ptr(out), L.stream_ptr()))
+    return out
+
+
+def build_expert_offsets(send_counts: torch.Tensor, with_dst: bool = False):
+    """expert_offs [W,E_l] (and, with_dst, dst_sizes [W], dst_offsets [W]) for a counts matrix."""
+    _req_i32(send_counts, "send_counts")
+    W, E_l = send_counts.shape
+    dev = send_counts.device
+    offs = _i32((W, E_l), dev)
+    sizes = _i32((W,), dev) if with_dst else None
+    doffs = _i32((W,), dev) if with_dst else None
+    L.check(L.lib().moe_build_expert_offsets(L.ptr(send_counts), W, E_l, L.ptr(offs), L.ptr(sizes), L.ptr(doffs),
+                                             L.stream_ptr()))
+    return (offs, sizes, doffs) if with_dst else offs

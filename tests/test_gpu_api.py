@@ -1,0 +1,123 @@
+"""The reference-named operators (utils / baseline / layers) on the GPU: same call signatures,
+return types, in-place behaviour and exceptions as the reference, results equal to the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import O, assert_bits_equal, to_np
+
+pytestmark = pytest.mark.gpu
+
+from iris_testing_amd import utils  # noqa: E402
+from iris_testing_amd.baseline import reorder_flat_to_token_buf  # noqa: E402
+from iris_testing_amd.layers import SimulatedWorld, custom_a2a, expert, shuffle, simulated_world  # noqa: E402
+
+DEV = "cuda"
+
+
+def test_route_and_pack_padding_free_matches_oracle():
+    # the reference's own generator conventions (utils.py:142-173): rand tokens, 0.001*randn router
+    T, H, E, k, W = 192, 128, 8, 2, 4
+    tokens = utils.gen_local_tokens(1, T, H, torch.float32, DEV, 0, 0)
+    router = utils.gen_router(H, E, torch.float32, DEV, 0)
+    payload, counts, offs, sizes = utils.route_and_pack_padding_free(tokens, router, k, W, E)
+    o_payload, o_counts, o_offs, o_sizes = O.route_and_pack_padding_free(to_np(tokens), to_np(router), k, W, E)
+    assert counts.dtype == torch.int32 and offs.dtype == torch.int32 and sizes.dtype == torch.int32
+    assert_bits_equal(counts, o_counts, "send_counts")
+    assert_bits_equal(offs, o_offs, "dst_offsets")
+    assert_bits_equal(sizes, o_sizes, "dst_sizes")
+    assert_bits_equal(payload, o_payload, "send_payload")
+    assert_bits_equal(utils.build_expert_offsets(counts), O.build_expert_offsets(o_counts), "expert_offs")
+    assert utils.compute_capacity_from_pca(counts) == O.compute_capacity_from_pca(o_counts)
+    # agreement with the library routines the reference itself calls, on the same fp32 inputs
+    p = torch.softmax(tokens.cpu() @ router.cpu(), dim=-1)
+    ref_idx = torch.topk(p, k, dim=-1).indices
+    same = (np.sort(ref_idx.numpy(), 1) == np.sort(O.route(to_np(tokens), to_np(router), k)[0], 1)).all(1).mean()
+    print(f"top-k sets equal to torch.topk(softmax(x@W)) on {100 * same:.2f}% of tokens", flush=True)
+    assert same > 0.99
+
+
+def test_route_and_pack_errors_and_empty():
+    tokens = torch.zeros((0, 64), dtype=torch.float32, device=DEV)
+    router = torch.zeros((64, 8), dtype=torch.float32, device=DEV)
+    payload, counts, offs, sizes = utils.route_and_pack_padding_free(tokens, router, 2, 4, 8)
+    assert payload.shape == (0, 64) and int(counts.sum()) == 0
+    with pytest.raises(AssertionError):
+        utils.route_and_pack_padding_free(torch.zeros((4, 64), device=DEV), router, 2, 3, 8)  # 8 % 3 != 0
+    with pytest.raises(AssertionError):
+        utils.route_and_pack_padding_free(torch.zeros((4, 64)), router, 2, 4, 8)  # CPU tokens
+    with pytest.raises(AssertionError):
+        utils.build_expert_offsets(torch.zeros((4, 2), dtype=torch.int64, device=DEV))
+
+
+@pytest.mark.parametrize("e_local,hidden_dim,cap", [(2, 128, 32), (4, 256, 16)])
+def test_custom_a2a_uniform_pattern(e_local, hidden_dim, cap):
+    """The reference's placement test (unit_tests.py:126-220) on a simulated 8-rank world: every src
+    sends exactly `cap` rows to every (dst, expert); every block must land exactly.  Values are
+    integer codes in fp32 (the reference's bf16 codes collide)."""
+    W = 8
+    experts = e_local * W
+    dest_counts = torch.full((W, e_local), cap, device=DEV, dtype=torch.int32)
+    dst_offsets = (torch.arange(W, device=DEV, dtype=torch.int32) * (e_local * cap)).contiguous()
+
+    def payload_of(rank):
+        rows = torch.arange(W * e_local * cap, device=DEV, dtype=torch.float32)
+        return (rank * 1_000_000 + rows)[:, None].expand(-1, hidden_dim).contiguous()
+
+    world = SimulatedWorld(W, rank=3)
+    for src in range(W):
+        if src != 3:
+            world.post(src, payload_of(src), dest_counts, dst_offsets)
+    bufs = utils.alloc_shmem_buffers(None, W, e_local, cap, hidden_dim, torch.float32)
+    with simulated_world(world):
+        out = custom_a2a(payload_of(3), dest_counts, dst_offsets, bufs.pca, bufs.token_buf, bufs.counts_ready,
+                         bufs.token_sync, bufs.heap_bases, experts, cap)
+    assert out.data_ptr() == bufs.token_buf.data_ptr()
+    assert (bufs.pca == cap).all() and int(bufs.counts_ready) == W and (bufs.token_sync == W).all()
+    for e in range(e_local):
+        for src in range(W):
+            start = 3 * (e_local * cap) + e * cap  # dst_offsets[rank] + e * cap
+            assert torch.equal(out[e, src], payload_of(src)[start:start + cap]), (e, src)
+    # shuffle removes nothing here (no padding) and orders by (expert, src, row)
+    sh = shuffle(out, bufs.pca, bufs.token_sync)
+    assert torch.equal(sh, out.reshape(-1, hidden_dim))
+    with pytest.raises(RuntimeError):
+        shuffle(out, bufs.pca, torch.zeros_like(bufs.token_sync))
+    with pytest.raises(AssertionError):
+        custom_a2a(payload_of(3), dest_counts, dst_offsets, bufs.pca, bufs.token_buf, bufs.counts_ready,
+                   bufs.token_sync, None, experts + 1, cap)
+
+
+def test_reorder_flat_to_token_buf_and_errors():
+    rng = np.random.default_rng(0)
+    W, E_l, H, CAP = 4, 3, 32, 9
+    rc = rng.integers(0, CAP + 1, size=(W, E_l)).astype(np.int32)
+    rc[1, 2] = 0
+    flat = rng.standard_normal((int(rc.sum()), H)).astype(np.float32)
+    tb = torch.full((E_l, W, CAP, H), 5.0, device=DEV)
+    out = reorder_flat_to_token_buf(torch.from_numpy(flat).to(DEV), torch.from_numpy(rc).to(DEV), CAP, tb)
+    want = O.reorder_flat_to_token_buf(flat, rc, CAP, np.empty((E_l, W, CAP, H), np.float32))
+    assert out.data_ptr() == tb.data_ptr()
+    assert_bits_equal(out, want, "token_buf")
+    f, c = torch.from_numpy(flat).to(DEV), torch.from_numpy(rc).to(DEV)
+    with pytest.raises(ValueError):
+        reorder_flat_to_token_buf(f, c, CAP, torch.zeros((E_l, W, CAP + 1, H), device=DEV))  # wrong shape
+    with pytest.raises(ValueError):
+        reorder_flat_to_token_buf(f, c, int(rc.max()) - 1, torch.zeros((E_l, W, int(rc.max()) - 1, H), device=DEV))
+    with pytest.raises(RuntimeError):
+        reorder_flat_to_token_buf(f[:-1], c, CAP, tb)  # rows consumed != rows given
+    with pytest.raises(ValueError):
+        reorder_flat_to_token_buf(f, c.to(torch.int64), CAP, tb)
+    with pytest.raises(ValueError):
+        reorder_flat_to_token_buf(f.cpu(), c, CAP, tb)
+
+
+def test_expert_layer_signature():
+    rng = np.random.default_rng(1)
+    cnt = np.array([17, 0, 40, 5, 66], dtype=np.int32)
+    x = rng.standard_normal((int(cnt.sum()), 128)).astype(np.float32)
+    w = rng.standard_normal((5, 128, 128)).astype(np.float32)
+    out = expert(torch.from_numpy(x).to(DEV), torch.from_numpy(w).to(DEV), torch.from_numpy(cnt).to(DEV), 40)
+    want = O.grouped_gemm(x, w, cnt, "f32")
+    np.testing.assert_allclose(to_np(out), want, rtol=1e-2, atol=1e-3)  # the reference's intended rtol (unit_tests.py:237)
+    np.testing.assert_allclose(to_np(out), want, rtol=1e-4, atol=1e-4)

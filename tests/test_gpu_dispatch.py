@@ -1,0 +1,191 @@
+"""GPU parity, integer/byte part of the path: route indices, counts, offsets, M/CAP, payload order,
+packed [W,M,H], token_buf, expert-major rows, return buffer, combine -- all compared BIT-EXACTLY
+with the CPU oracle on identical seeded inputs, through the C ABI (iris_testing_amd.ops)."""
+import dataclasses
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import O, assert_bits_equal, oracle_recv, oracle_world, to_np
+
+pytestmark = pytest.mark.gpu
+
+from iris_testing_amd import ops  # noqa: E402
+from iris_testing_amd.configs import CONFIGS, gen_router, gen_router_bias, gen_shard_tokens  # noqa: E402
+
+DEV = "cuda"
+
+# (config name, tokens per shard or None for the full size)
+ROUTE_CASES = [("plumbing", None), ("small", None), ("mixtral", 2048), ("mixtral", None), ("finegrained", 512),
+               ("finegrained", None), ("zipf_k1", 1024), ("zipf_k2", None), ("zipf_k4", 1000), ("zipf_k8", None)]
+
+
+def _cfg(name, tokens):
+    cfg = CONFIGS[name]
+    return cfg if tokens is None else dataclasses.replace(cfg, tokens=tokens)
+
+
+def _inputs(cfg, shard=0):
+    x = gen_shard_tokens(cfg, shard)
+    w = gen_router(cfg)
+    b = gen_router_bias(cfg)
+    return x, w, b
+
+
+@pytest.mark.parametrize("name,tokens", ROUTE_CASES)
+def test_route_count_pack_bit_exact(name, tokens):
+    cfg = _cfg(name, tokens)
+    print(f"case {cfg}", flush=True)
+    x, w, b = _inputs(cfg)
+    xn, wn, bn = to_np(x), to_np(w), None if b is None else to_np(b)
+    xd, wd = x.to(DEV), w.to(DEV)
+    bd = None if b is None else b.to(DEV)
+
+    idx, gate, logits = ops.route_topk(xd, wd, cfg.topk, bd)
+    o_idx, o_gate, o_logits = O.route(xn, wn, cfg.topk, bn)
+    assert_bits_equal(logits, o_logits, "router logits")
+    assert_bits_equal(idx, o_idx, "top-k indices")
+    np.testing.assert_allclose(to_np(gate), o_gate, rtol=1e-5, atol=1e-30, err_msg="softmax gates")
+
+    c = ops.count_and_offsets(idx, cfg.experts, cfg.world)
+    o_counts = O.send_counts(o_idx, cfg.world, cfg.experts)
+    o_sizes, o_offs = O.dst_sizes_offsets(o_counts)
+    o_pos, o_rt = O.payload_positions(o_idx, cfg.experts)
+    assert_bits_equal(c.send_counts, o_counts, "send_counts")
+    assert_bits_equal(c.expert_offs, O.build_expert_offsets(o_counts), "expert_offs")
+    assert_bits_equal(c.dst_sizes, o_sizes, "dst_sizes")
+    assert_bits_equal(c.dst_offsets, o_offs, "dst_offsets")
+    assert_bits_equal(c.pos, o_pos, "pos")
+    assert_bits_equal(c.row_token, o_rt, "row_token")
+    caps = to_np(c.caps)
+    assert caps[0] == O.pair_capacity(o_sizes) and caps[1] == O.compute_capacity_from_pca(o_counts)
+
+    payload = ops.pack_payload(xd, c.row_token)
+    o_payload = O.send_payload(xn, o_rt)
+    assert_bits_equal(payload, o_payload, "send_payload")
+
+    M = int(caps[0]) + 3  # a few rows of mandatory zero padding everywhere
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    send = ops.pack_fixed_m(xd, c.row_token, c.dst_sizes, c.dst_offsets, M, status=status)
+    assert_bits_equal(send, O.pack_fixed_m(o_payload, o_offs, o_sizes, M), "send [W,M,H]")
+    assert int(status.item()) == 0
+
+
+def test_route_ties_prefer_lower_expert():
+    # identical router columns -> identical logits: every tie must resolve to the lower expert id
+    T, H, E, k = 130, 64, 40, 5
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(T, H, generator=g)
+    col = torch.randn(H, 4, generator=g)
+    w = col.repeat(1, E // 4)  # expert e has the same column as e % 4
+    idx, gate, logits = ops.route_topk(x.to(DEV), w.to(DEV).contiguous(), k)
+    o_idx, _, _ = O.route(x.numpy(), w.numpy(), k)
+    assert_bits_equal(idx, o_idx, "tied top-k")
+    # the best class appears with its k lowest ids (10 copies of each class, k = 5)
+    cls = o_idx % 4
+    assert (cls == cls[:, :1]).all() and (np.diff(o_idx, axis=1) == 4).all()
+
+
+@pytest.mark.parametrize("E,k,W", [(8, 8, 4), (512, 16, 64), (6, 1, 3), (60, 7, 1)])
+def test_route_edge_shapes(E, k, W):
+    T, H = 77, 72
+    g = torch.Generator().manual_seed(E * 31 + k)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    w = (torch.randn(H, E, generator=g) / 8).to(torch.bfloat16)
+    b = torch.randn(E, generator=g)
+    idx, gate, logits = ops.route_topk(x.to(DEV), w.to(DEV), k, b.to(DEV))
+    o_idx, o_gate, o_logits = O.route(to_np(x), to_np(w), k, b.numpy())
+    assert_bits_equal(logits, o_logits, "logits")
+    assert_bits_equal(idx, o_idx, "idx")
+    np.testing.assert_allclose(to_np(gate), o_gate, rtol=1e-5)
+    c = ops.count_and_offsets(idx, E, W)
+    assert_bits_equal(c.send_counts, O.send_counts(o_idx, W, E), "send_counts")
+    assert_bits_equal(c.pos, O.payload_positions(o_idx, E)[0], "pos")
+
+
+def test_zero_tokens_and_overflow_flag():
+    # zero routed tokens: all counts zero, capacities floor at 1 (reference utils.py:121,240-242)
+    idx = torch.empty((0, 2), dtype=torch.int32, device=DEV)
+    c = ops.count_and_offsets(idx, 8, 4)
+    assert to_np(c.send_counts).sum() == 0 and to_np(c.caps).tolist() == [1, 1]
+    # M smaller than a destination's rows -> status flag, rows beyond M dropped, no overrun
+    cfg = CONFIGS["plumbing"]
+    x, w, _ = _inputs(cfg)
+    xd = x.to(DEV)
+    idx, _, _ = ops.route_topk(xd, w.to(DEV), cfg.topk)
+    c = ops.count_and_offsets(idx, cfg.experts, cfg.world)
+    M = int(c.caps[0].item()) - 5
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    guard = torch.full((cfg.world * M + 4, cfg.hidden), 7.0, device=DEV)
+    ops.pack_fixed_m(xd, c.row_token, c.dst_sizes, c.dst_offsets, M, out=guard[:cfg.world * M].view(cfg.world, M, -1),
+                     status=status)
+    assert int(status.item()) == 1
+    assert (guard[cfg.world * M:] == 7.0).all()
+
+
+UNPACK_CASES = [("plumbing", None), ("small", None), ("mixtral", 1024), ("finegrained", 512), ("zipf_k4", 1024)]
+
+
+@pytest.mark.parametrize("name,tokens", UNPACK_CASES)
+def test_unpack_return_combine_bit_exact(name, tokens):
+    """All W shards routed on both sides; rank 0's receive buffer assembled; then token_buf, pca,
+    expert-major rows, return buffer and combine compared bit for bit."""
+    cfg = _cfg(name, tokens)
+    print(f"case {cfg}", flush=True)
+    w = gen_router(cfg)
+    b = gen_router_bias(cfg)
+    xs = [gen_shard_tokens(cfg, s) for s in range(cfg.world)]
+    xn = [to_np(x) for x in xs]
+    shards, M, CAP = oracle_world(cfg, xn, to_np(w), None if b is None else to_np(b))
+    o_recv, o_rc = oracle_recv(cfg, xn, shards, M, 0)
+
+    recv = torch.from_numpy(o_recv).to(cfg.torch_dtype).to(DEV)
+    rc = torch.from_numpy(o_rc).to(DEV)
+    S = int(o_rc.sum())
+
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    tb, pca = ops.unpack_token_buf(recv, rc, CAP, status=status)
+    o_tb, o_pca = O.recv_to_token_buf(o_recv, o_rc, CAP)
+    assert_bits_equal(tb, o_tb, "token_buf")
+    assert_bits_equal(pca, o_pca, "pca")
+    assert int(status.item()) == 0
+
+    sh, cnt = ops.shuffle_rows(tb, pca, S + 2)
+    o_sh = O.shuffle(o_tb, o_pca)
+    assert_bits_equal(sh[:S], o_sh, "shuffled")
+    assert (to_np(sh[S:]) == 0).all()
+    assert_bits_equal(cnt, O.expert_row_counts(o_pca), "expert_cnt")
+
+    sh2, cnt2 = ops.unpack_expert_major(recv, rc, S)
+    assert_bits_equal(sh2, O.unpack_expert_major(o_recv, o_rc), "unpack_expert_major")
+    assert_bits_equal(cnt2, O.expert_row_counts(o_pca), "expert_cnt (fused)")
+
+    # return path with a recognisable payload: y = -2 * shuffled (exact in every dtype)
+    y = (sh2 * -2).contiguous()
+    ret = ops.return_pack(y, rc, M)
+    o_ret = O.return_pack(o_sh * -2, o_rc, M)
+    assert_bits_equal(ret, o_ret, "return buffer")
+    # inverse property: the return buffer is -2 x the receive buffer, padding included
+    assert_bits_equal(ret, o_recv * -2, "return == -2 * recv")
+
+    # combine on rank 0 as a source: returned[d] is the slot dst d sends back = -2 * send_0[d]
+    s0 = shards[0]
+    o_send0 = O.pack_fixed_m(O.send_payload(xn[0], s0["row_token"]), s0["offs"], s0["sizes"], M)
+    returned = torch.from_numpy(o_send0 * -2).to(cfg.torch_dtype).to(DEV)
+    out = ops.combine(returned, torch.from_numpy(s0["idx"]).to(DEV), torch.from_numpy(s0["pos"]).to(DEV),
+                      torch.from_numpy(s0["gate"]).to(DEV), torch.from_numpy(s0["offs"]).to(DEV), cfg.e_local)
+    o_out = O.combine(o_send0 * -2, s0["idx"], s0["pos"], s0["gate"], s0["offs"], cfg.e_local, cfg.dtype)
+    assert_bits_equal(out, o_out, "combine")
+
+
+def test_capacity_overflow_flag_on_unpack():
+    rc = torch.tensor([[3, 1], [0, 2]], dtype=torch.int32, device=DEV)
+    recv = torch.arange(2 * 4 * 8, dtype=torch.float32, device=DEV).view(2, 4, 8)
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    tb, pca = ops.unpack_token_buf(recv, rc, 2, status=status)  # count 3 > CAP 2
+    assert int(status.item()) == 1
+    status.zero_()
+    tb, pca = ops.unpack_token_buf(recv, rc, 3, status=status)
+    assert int(status.item()) == 0
+    assert_bits_equal(tb, O.recv_to_token_buf(to_np(recv), to_np(rc), 3)[0], "token_buf")

@@ -1,0 +1,144 @@
+"""GPU parity, floating-point part of the path: grouped GEMM, expert MLP (GELU / SiLU / SwiGLU,
+fp32 / bf16 / fp8) and the end-to-end combine.  Tolerances are stated per test; max-abs and
+relative errors are printed."""
+import dataclasses
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import O, assert_bits_equal, err_stats, to_np
+
+pytestmark = pytest.mark.gpu
+
+from iris_testing_amd import ops  # noqa: E402
+from iris_testing_amd.layers.expert import ExpertWeights, expert_mlp  # noqa: E402
+
+DEV = "cuda"
+
+# bf16 outputs: the GPU and the oracle round the same fp32-accumulated value to bf16; they can differ
+# by accumulation order only, i.e. by at most one bf16 ulp (2^-8 relative) of the value plus the
+# propagated rounding of the hidden activation.  Bound used: |err| <= BF16_RTOL*|ref| + BF16_ATOL*rms(ref).
+BF16_RTOL, BF16_ATOL = 2.0 ** -6, 2.0 ** -6
+F32_RTOL, F32_ATOL = 1e-4, 1e-5
+# fp8: same quantised inputs on both sides (quantisation is part of the spec), error again only from
+# accumulation order and from re-quantising a hidden activation that differs in its last bf16 bit.
+FP8_RTOL, FP8_ATOL = 2.0 ** -4, 2.0 ** -5
+
+
+def _check(got, want, rtol, atol, what):
+    mx, mx_rms, rel = err_stats(got, want)
+    rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    print(f"{what}: max-abs {mx:.3e}  max-abs/rms {mx_rms:.3e}  max-rel(|ref|>rms/8) {rel:.3e}", flush=True)
+    bound = rtol * np.abs(want) + atol * rms
+    bad = np.abs(got.astype(np.float64) - want) > bound
+    assert not bad.any(), f"{what}: {bad.sum()} of {bad.size} outside tolerance (max-abs {mx}, rms {rms})"
+
+
+def _groups(rng, E_l, S_target, with_zero=True):
+    cnt = rng.multinomial(S_target, rng.dirichlet(np.ones(E_l))).astype(np.int32)
+    if with_zero and E_l > 2:
+        cnt[1] = 0
+    return cnt
+
+
+def _randn(rng, *shape, scale=1.0, dtype="bf16"):
+    a = (rng.standard_normal(shape) * scale).astype(np.float32)
+    return O.bf16_round(a) if dtype == "bf16" else a
+
+
+def _t(a, dtype):
+    return torch.from_numpy(a).to({"bf16": torch.bfloat16, "f32": torch.float32}[dtype]).to(DEV)
+
+
+@pytest.mark.parametrize("dtype,E_l,K,N,S", [("bf16", 2, 128, 256, 300), ("bf16", 5, 192, 328, 777),
+                                              ("bf16", 1, 4096, 512, 1500), ("bf16", 32, 256, 256, 3000),
+                                              ("f32", 2, 24, 48, 99), ("f32", 5, 128, 128, 333)])
+def test_grouped_gemm(dtype, E_l, K, N, S):
+    """expert(tokens, weights, cnt): one GEMM per group, the shapes the reference meant to test
+    ((2,24,48), (5,128,128), unit_tests.py:247-248) and MFMA-sized ones."""
+    rng = np.random.default_rng(E_l * 1000 + K)
+    cnt = _groups(rng, E_l, S)
+    S_tot = int(cnt.sum())
+    x = _randn(rng, S_tot + 3, K, dtype=dtype)
+    w = _randn(rng, E_l, K, N, scale=K ** -0.5, dtype=dtype)
+    out = ops.grouped_gemm(_t(x, dtype), _t(w, dtype), torch.from_numpy(cnt).to(DEV))
+    want = O.grouped_gemm(x, w, cnt, dtype)
+    r, a = (BF16_RTOL, BF16_ATOL) if dtype == "bf16" else (F32_RTOL, F32_ATOL)
+    _check(to_np(out)[:S_tot], want[:S_tot].astype(np.float64), r, a, f"grouped_gemm {dtype}")
+    assert (to_np(out)[S_tot:] == 0).all(), "rows past sum(cnt) must stay untouched"
+
+
+def test_grouped_gemm_identity_is_exact():
+    """Identity / one-hot weights: the GEMM must reproduce (permute) its input bit for bit."""
+    rng = np.random.default_rng(3)
+    E_l, K = 3, 256
+    cnt = np.array([130, 0, 259], dtype=np.int32)
+    x = _randn(rng, int(cnt.sum()), K)
+    perm = rng.permutation(K)
+    w = np.zeros((E_l, K, K), dtype=np.float32)
+    w[0] = np.eye(K)
+    w[1] = np.eye(K)
+    w[2][perm, np.arange(K)] = 1.0  # out[:, j] = x[:, perm[j]]
+    out = to_np(ops.grouped_gemm(_t(x, "bf16"), _t(w, "bf16"), torch.from_numpy(cnt).to(DEV)))
+    assert_bits_equal(out[:130], x[:130], "identity expert")
+    assert_bits_equal(out[130:], x[130:][:, perm], "permutation expert")
+
+
+MLP_CASES = [
+    # dtype, act, E_l, H, F, S
+    ("f32", "gelu", 2, 256, 512, 512),      # plumbing workload's expert
+    ("f32", "swiglu", 3, 64, 96, 200),
+    ("bf16", "silu", 2, 2048, 4096, 443),   # small workload's expert at its real shape
+    ("bf16", "gelu", 4, 256, 512, 900),
+    ("bf16", "swiglu", 1, 4096, 1792, 1300),  # Mixtral-style expert, F cut to 1/8 for CPU time
+    ("bf16", "swiglu", 32, 7168, 256, 2500),  # fine-grained: 32 small groups, F cut to 1/8
+    ("bf16", "swiglu", 15, 2048, 1408, 3000),
+]
+
+
+@pytest.mark.parametrize("dtype,act,E_l,H,F,S", MLP_CASES)
+def test_expert_mlp(dtype, act, E_l, H, F, S):
+    rng = np.random.default_rng(H + F + E_l)
+    cnt = _groups(rng, E_l, S)
+    S_tot = int(cnt.sum())
+    x = _randn(rng, S_tot, H, dtype=dtype)
+    w1 = _randn(rng, E_l, H, F, scale=H ** -0.5, dtype=dtype)
+    w2 = _randn(rng, E_l, F, H, scale=F ** -0.5, dtype=dtype)
+    wu = _randn(rng, E_l, H, F, scale=H ** -0.5, dtype=dtype) if act == "swiglu" else None
+    ew = ExpertWeights.prepare(act, _t(w1, dtype), _t(w2, dtype), None if wu is None else _t(wu, dtype))
+    out = to_np(expert_mlp(_t(x, dtype), ew, torch.from_numpy(cnt).to(DEV)))
+    want = O.expert_mlp(x, cnt, w1, w2, act, dtype, w_up=wu)
+    r, a = (BF16_RTOL, BF16_ATOL) if dtype == "bf16" else (F32_RTOL, F32_ATOL)
+    _check(out, want.astype(np.float64), r, a, f"expert_mlp {dtype} {act} E_l={E_l} H={H} F={F}")
+
+
+@pytest.mark.parametrize("R,C", [(5, 64), (300, 2048), (77, 1408)])
+def test_quantize_rows_fp8_bit_exact(R, C):
+    rng = np.random.default_rng(R)
+    x = _randn(rng, R, C, scale=3.0)
+    x[1] = 0.0  # an all-zero row -> scale 1, codes 0
+    q, s = ops.quantize_rows_fp8(_t(x, "bf16"))
+    oq, osc = O.quantize_rows_fp8(x)
+    assert_bits_equal(s, osc, "row scales")
+    assert_bits_equal(q, oq, "fp8 codes")
+
+
+@pytest.mark.parametrize("E_l,H,F,S", [(2, 256, 384, 400), (15, 2048, 1408, 2500)])
+def test_expert_mlp_fp8(E_l, H, F, S):
+    rng = np.random.default_rng(H + F)
+    cnt = _groups(rng, E_l, S)
+    S_tot = int(cnt.sum())
+    x = _randn(rng, S_tot, H)
+    wg = _randn(rng, E_l, H, F, scale=H ** -0.5)
+    wu = _randn(rng, E_l, H, F, scale=H ** -0.5)
+    wd = _randn(rng, E_l, F, H, scale=F ** -0.5)
+    (gq, gs), (uq, us), (dq, ds) = (O.quantize_cols_fp8(w) for w in (wg, wu, wd))
+    tq = lambda a: torch.from_numpy(a).to(DEV)  # noqa: E731
+    ew = ExpertWeights.prepare_fp8(tq(gq), tq(gs), tq(uq), tq(us), tq(dq), tq(ds))
+    out = to_np(expert_mlp(_t(x, "bf16"), ew, torch.from_numpy(cnt).to(DEV)))
+    want = O.expert_mlp_fp8(x, cnt, gq, gs, uq, us, dq, ds)
+    _check(out, want.astype(np.float64), FP8_RTOL, FP8_ATOL, f"expert_mlp_fp8 E_l={E_l} H={H} F={F}")
+    # and against the unquantised fp32 MLP, to show what the quantisation itself costs (reported only)
+    ref = O.expert_mlp(x, cnt, wg, wd, "swiglu", "f32", w_up=wu)
+    print("fp8 vs unquantised fp32 MLP:", err_stats(out, ref.astype(np.float64)), flush=True)
