@@ -161,21 +161,21 @@ def test_unpack_return_combine_bit_exact(name, tokens):
     assert_bits_equal(sh2, O.unpack_expert_major(o_recv, o_rc), "unpack_expert_major")
     assert_bits_equal(cnt2, O.expert_row_counts(o_pca), "expert_cnt (fused)")
 
-    # return path with a recognisable payload: y = -2 * shuffled (exact in every dtype)
-    y = (sh2 * -2).contiguous()
+    # return path with a recognisable payload: y = 2 * shuffled (exact in every dtype, keeps +0 padding)
+    y = (sh2 * 2).contiguous()
     ret = ops.return_pack(y, rc, M)
-    o_ret = O.return_pack(o_sh * -2, o_rc, M)
+    o_ret = O.return_pack(o_sh * 2, o_rc, M)
     assert_bits_equal(ret, o_ret, "return buffer")
-    # inverse property: the return buffer is -2 x the receive buffer, padding included
-    assert_bits_equal(ret, o_recv * -2, "return == -2 * recv")
+    # inverse property: the return buffer is 2 x the receive buffer, padding included
+    assert_bits_equal(ret, o_recv * 2, "return == 2 * recv")
 
-    # combine on rank 0 as a source: returned[d] is the slot dst d sends back = -2 * send_0[d]
+    # combine on rank 0 as a source: returned[d] is the slot dst d sends back = 2 * send_0[d]
     s0 = shards[0]
     o_send0 = O.pack_fixed_m(O.send_payload(xn[0], s0["row_token"]), s0["offs"], s0["sizes"], M)
-    returned = torch.from_numpy(o_send0 * -2).to(cfg.torch_dtype).to(DEV)
+    returned = torch.from_numpy(o_send0 * 2).to(cfg.torch_dtype).to(DEV)
     out = ops.combine(returned, torch.from_numpy(s0["idx"]).to(DEV), torch.from_numpy(s0["pos"]).to(DEV),
                       torch.from_numpy(s0["gate"]).to(DEV), torch.from_numpy(s0["offs"]).to(DEV), cfg.e_local)
-    o_out = O.combine(o_send0 * -2, s0["idx"], s0["pos"], s0["gate"], s0["offs"], cfg.e_local, cfg.dtype)
+    o_out = O.combine(o_send0 * 2, s0["idx"], s0["pos"], s0["gate"], s0["offs"], cfg.e_local, cfg.dtype)
     assert_bits_equal(out, o_out, "combine")
 
 

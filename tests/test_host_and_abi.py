@@ -1,0 +1,77 @@
+"""CPU-side checks of the product: the C-ABI library loads and exports every symbol the header
+declares, the host layer rejects CPU tensors the way the reference does, and nothing in the
+package reaches for the oracle."""
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "moe_gfx950.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(moe_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from iris_testing_amd import _lib as L
+    lib = L.lib()
+    declared = _declared()
+    assert len(declared) >= 20
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in include/moe_gfx950.h but not exported"
+    assert sorted(L.exported_symbols()) == declared, "ctypes table and header disagree"
+    assert lib.moe_abi_version() == 1
+    assert lib.moe_last_error() == b""
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    # calls that fail validation before any HIP call
+    from iris_testing_amd import _lib as L
+    lib = L.lib()
+    rc = lib.moe_count_and_offsets(None, 4, 2, 9, 4, None, None, None, None, None, None, None, None, 0, None)
+    assert rc == -1 and b"divisible" in lib.moe_last_error()
+    rc = lib.moe_route_topk(None, None, None, 0, 4, 64, 8, 9, None, None, None, None)
+    assert rc == -1 and b"topk" in lib.moe_last_error()
+    rc = lib.moe_route_topk(None, None, None, 1, 4, 60, 8, 2, None, None, None, None)
+    assert rc == -1 and b"16-byte" in lib.moe_last_error()
+    with pytest.raises(L.MoeLibraryError):
+        L.check(lib.moe_pack(None, 7, 1, 64, None, None, None, 4, 4, None, None, None, None))
+    assert lib.moe_count_workspace_bytes(1000, 2, 8) == 4 * (2 * 8 * 16 + 2 * 8 + 1)
+
+
+def test_host_layer_rejects_cpu_tensors_like_the_reference():
+    from iris_testing_amd import utils
+    from iris_testing_amd.baseline import reorder_flat_to_token_buf
+    with pytest.raises(AssertionError, match="Expect CUDA tokens"):  # reference utils.py:193
+        utils.route_and_pack_padding_free(torch.zeros(4, 8), torch.zeros(8, 4), 1, 2, 4)
+    with pytest.raises(AssertionError, match="must be CUDA"):  # reference utils.py:16
+        utils.build_expert_offsets(torch.zeros((2, 2), dtype=torch.int32))
+    with pytest.raises(ValueError, match="CUDA"):  # reference baseline.py:10-12
+        reorder_flat_to_token_buf(torch.zeros(2, 4), torch.zeros((1, 1), dtype=torch.int32), 2, torch.zeros(1, 1, 2, 4))
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "iris_testing_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.lower() or f == "harness.py" and "moe_oracle" not in text, \
+                    f"{f} mentions the oracle"
+
+
+def test_configs_and_generators_are_deterministic():
+    from iris_testing_amd.configs import CONFIGS, gen_router, gen_router_bias, gen_shard_tokens
+    cfg = CONFIGS["plumbing"]
+    a, b = gen_shard_tokens(cfg, 1), gen_shard_tokens(cfg, 1)
+    assert torch.equal(a, b) and not torch.equal(a, gen_shard_tokens(cfg, 2))
+    assert gen_router(cfg).shape == (256, 8)
+    z = gen_router_bias(CONFIGS["zipf_k2"])
+    assert z.shape == (60,) and torch.all(z[:-1] > z[1:])  # expert 0 hottest
+    assert abs(float(torch.exp(z).sum()) - 1) < 1e-5
+    for name, c in CONFIGS.items():
+        assert c.experts % c.world == 0 and c.topk <= c.experts, name

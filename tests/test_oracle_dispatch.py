@@ -1,0 +1,183 @@
+"""Pins the oracle's integer/layout functions (a2-a10, a13) against a literal pure-Python restatement
+of the reference's bucket loop (utils.py:204-246), brute force, round trips and the reference's own
+uniform placement pattern (unit_tests.py:137-150,211-218).  CPU only."""
+import numpy as np
+import pytest
+
+from helpers import O
+
+
+def reference_bucket_loop(x, top_idxs, world_size, num_experts_total):
+    """The reference's host algorithm, line by line (utils.py:204-246), on numpy arrays."""
+    e_local = num_experts_total // world_size
+    buckets = [[[] for _ in range(e_local)] for _ in range(world_size)]
+    for ti in range(x.shape[0]):
+        for kk in range(top_idxs.shape[1]):
+            ex = int(top_idxs[ti, kk])
+            dst = ex // e_local
+            el = ex - dst * e_local
+            buckets[dst][el].append(x[ti])
+    send_counts = np.zeros((world_size, e_local), np.int32)
+    chunks, dst_offsets, dst_sizes, running = [], np.zeros(world_size, np.int32), np.zeros(world_size, np.int32), 0
+    for dst in range(world_size):
+        dst_offsets[dst] = running
+        rows = 0
+        for el in range(e_local):
+            n = len(buckets[dst][el])
+            send_counts[dst, el] = n
+            if n:
+                chunks.append(np.stack(buckets[dst][el]))
+            rows += n
+        dst_sizes[dst] = rows
+        running += rows
+    payload = np.concatenate(chunks) if running else np.empty((0, x.shape[1]), x.dtype)
+    return payload, send_counts, dst_offsets, dst_sizes
+
+
+def coded_rows(T, H):
+    """x[t,h] = t*H + h in fp32: every row identifiable (the reference's bf16 codes collide)."""
+    return (np.arange(T)[:, None] * H + np.arange(H)[None, :]).astype(np.float32)
+
+
+@pytest.mark.parametrize("T,E,k,W,seed", [(37, 8, 2, 4, 0), (64, 16, 1, 8, 1), (50, 12, 4, 3, 2), (9, 6, 6, 2, 3),
+                                          (0, 8, 2, 4, 4)])
+def test_counts_offsets_payload_against_bucket_loop(T, E, k, W, seed):
+    rng = np.random.default_rng(seed)
+    H = 5
+    x = coded_rows(T, H)
+    idx = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32) if T else np.zeros((0, k), np.int32)
+    payload, counts, offs, sizes = reference_bucket_loop(x, idx, W, E)
+    o_counts = O.send_counts(idx, W, E)
+    o_sizes, o_offs = O.dst_sizes_offsets(o_counts)
+    pos, row_token = O.payload_positions(idx, E)
+    assert np.array_equal(o_counts, counts) and o_counts.dtype == np.int32
+    assert np.array_equal(o_sizes, sizes) and np.array_equal(o_offs, offs)
+    assert np.array_equal(O.send_payload(x, row_token), payload)
+    # brute-force count cube and invariants
+    cube = np.zeros(E, np.int64)
+    np.add.at(cube, idx.reshape(-1), 1)
+    assert np.array_equal(cube.reshape(W, E // W), counts)
+    assert counts.sum() == T * k and (o_offs[-1] + o_sizes[-1] == T * k)
+    eo = O.build_expert_offsets(counts)
+    for d in range(W):
+        for e in range(E // W):
+            assert eo[d, e] == counts[d, :e].sum()
+    # pos is the inverse of row_token and points at the token's own row
+    for t in range(T):
+        for kk in range(k):
+            assert row_token[pos[t, kk]] == t
+    # capacities, floor of 1 (utils.py:121)
+    assert O.compute_capacity_from_pca(counts) == max(1, counts.max(initial=0))
+    assert O.pair_capacity(sizes) == max(1, sizes.max(initial=0))
+
+
+def test_route_and_pack_padding_free_end_to_end():
+    rng = np.random.default_rng(5)
+    T, H, E, k, W = 70, 32, 8, 2, 4
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    w = rng.standard_normal((H, E)).astype(np.float32)
+    payload, counts, offs, sizes = O.route_and_pack_padding_free(x, w, k, W, E)
+    idx = O.route(x, w, k)[0]
+    p2, c2, o2, s2 = reference_bucket_loop(x, idx, W, E)
+    assert np.array_equal(payload, p2) and np.array_equal(counts, c2) and np.array_equal(offs, o2) and np.array_equal(sizes, s2)
+    with pytest.raises(AssertionError):
+        O.send_counts(idx, 3, E)  # utils.py:197
+
+
+def test_fixed_m_layout_and_receive_side_round_trip():
+    rng = np.random.default_rng(6)
+    W, E_l, T, k, H = 4, 3, 45, 3, 6
+    E = W * E_l
+    xs = [coded_rows(T, H) + s * 10000 for s in range(W)]
+    routes = []
+    for s in range(W):
+        idx = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+        counts = O.send_counts(idx, W, E)
+        sizes, offs = O.dst_sizes_offsets(counts)
+        pos, rt = O.payload_positions(idx, E)
+        routes.append(dict(idx=idx, counts=counts, sizes=sizes, offs=offs, pos=pos, rt=rt))
+    M = O.pair_capacity(np.stack([r["sizes"] for r in routes]))
+    CAP = max(O.compute_capacity_from_pca(r["counts"]) for r in routes)
+    sends = [O.pack_fixed_m(O.send_payload(x, r["rt"]), r["offs"], r["sizes"], M) for x, r in zip(xs, routes)]
+    for s, (send, r) in enumerate(zip(sends, routes)):
+        assert send.shape == (W, M, H)
+        for d in range(W):
+            n = r["sizes"][d]
+            assert (send[d, n:] == 0).all()  # padding rows are all-zero
+            # rows of dst d are the stable sort by local expert of the tokens routed there
+            want = [xs[s][t] for el in range(E_l) for t in range(T) if (r["idx"][t] == d * E_l + el).any()]
+            assert np.array_equal(send[d, :n], np.stack(want) if want else np.empty((0, H), np.float32))
+    with pytest.raises(ValueError):
+        O.pack_fixed_m(O.send_payload(xs[0], routes[0]["rt"]), routes[0]["offs"], routes[0]["sizes"], M - 1 if
+                       routes[0]["sizes"].max() == M else routes[0]["sizes"].max() - 1)
+    for d in range(W):
+        recv = np.stack([sends[s][d] for s in range(W)])
+        rc = np.stack([routes[s]["counts"][d] for s in range(W)])
+        tb, pca = O.recv_to_token_buf(recv, rc, CAP)
+        assert np.array_equal(pca, rc.T)
+        # same placement as the reference's reorder loop fed with the padding-free concatenation
+        flat = np.concatenate([recv[s, :rc[s].sum()] for s in range(W)])
+        tb2 = O.reorder_flat_to_token_buf(flat, rc, CAP, np.full((E_l, W, CAP, H), 9.0, np.float32))
+        assert np.array_equal(tb, tb2)
+        sh = O.shuffle(tb, pca)
+        assert np.array_equal(sh, O.unpack_expert_major(recv, rc))
+        # every routed row arrives exactly once, grouped by expert, in (src, token) order
+        want = [xs[s][t] for el in range(E_l) for s in range(W) for t in range(T)
+                if (routes[s]["idx"][t] == d * E_l + el).any()]
+        assert np.array_equal(sh, np.stack(want))
+        assert np.array_equal(O.expert_row_counts(pca), [sum((routes[s]["idx"] == d * E_l + el).sum() for s in range(W))
+                                                         for el in range(E_l)])
+        # return path inverts the unpack exactly
+        assert np.array_equal(O.return_pack(sh, rc, M), recv)
+
+
+def test_reorder_error_cases():
+    rc = np.array([[2, 1], [0, 3]], np.int32)
+    flat = np.zeros((6, 4), np.float32)
+    with pytest.raises(ValueError):
+        O.reorder_flat_to_token_buf(flat, rc, 3, np.zeros((2, 2, 4, 4), np.float32))  # wrong shape (baseline.py:199-201)
+    with pytest.raises(ValueError):
+        O.reorder_flat_to_token_buf(flat, rc, 2, np.zeros((2, 2, 2, 4), np.float32))  # count > capacity (:215-216)
+    with pytest.raises(RuntimeError):
+        O.reorder_flat_to_token_buf(np.zeros((7, 4), np.float32), rc, 3, np.zeros((2, 2, 3, 4), np.float32))  # rows consumed (:220-221)
+
+
+def test_uniform_pattern_of_the_reference_unit_test():
+    # every src sends exactly cap rows to every (dst, expert): dst_offsets = arange(W)*E_l*cap (unit_tests.py:138-139)
+    W, E_l, cap, H = 8, 2, 32, 4
+    counts = np.full((W, E_l), cap, np.int32)
+    sizes, offs = O.dst_sizes_offsets(counts)
+    assert np.array_equal(offs, np.arange(W) * E_l * cap) and (sizes == E_l * cap).all()
+    assert np.array_equal(O.build_expert_offsets(counts), np.tile(np.arange(E_l) * cap, (W, 1)))
+    rank = 5
+    payloads = [(s * 1_000_000 + np.arange(W * E_l * cap))[:, None].repeat(H, 1).astype(np.float32) for s in range(W)]
+    flat = np.concatenate([p[offs[rank]:offs[rank] + sizes[rank]] for p in payloads])
+    tb = O.reorder_flat_to_token_buf(flat, counts, cap, np.empty((E_l, W, cap, H), np.float32))
+    for e in range(E_l):
+        for s in range(W):
+            start = offs[rank] + e * cap
+            assert np.array_equal(tb[e, s], payloads[s][start:start + cap])  # unit_tests.py:211-218
+
+
+def test_combine_closed_forms():
+    rng = np.random.default_rng(8)
+    T, H, E, k, W = 30, 8, 8, 3, 4
+    E_l = E // W
+    x = O.bf16_round(rng.standard_normal((T, H)).astype(np.float32))
+    w = rng.standard_normal((H, E)).astype(np.float32)
+    idx, gate, _ = O.route(x, w, k)
+    counts = O.send_counts(idx, W, E)
+    sizes, offs = O.dst_sizes_offsets(counts)
+    pos, rt = O.payload_positions(idx, E)
+    M = O.pair_capacity(sizes)
+    send = O.pack_fixed_m(O.send_payload(x, rt), offs, sizes, M)
+    # identity experts: out[t] = (sum_kk gate) * x[t]
+    out = O.combine(send, idx, pos, gate, offs, E_l, "f32")
+    np.testing.assert_allclose(out, gate.sum(1, keepdims=True) * x, rtol=1e-6, atol=1e-7)
+    # brute force per token
+    for t in range(T):
+        acc = np.zeros(H, np.float32)
+        for kk in range(k):
+            d = idx[t, kk] // E_l
+            acc = acc + gate[t, kk] * send[d, pos[t, kk] - offs[d]]
+        assert np.array_equal(O.combine(send, idx, pos, gate, offs, E_l, "bf16")[t], O.bf16_round(acc))
