@@ -140,6 +140,12 @@ int moe_grouped_gemm(const void* tokens, const void* weights, const int32_t* exp
 int moe_prepack_weights(const void* w, const void* w_up, int dtype, int E_l, int K, int N, void* packed,
                         moe_stream_t stream);
 
+/* One bf16 grouped GEMM on pre-packed weights with a fused epilogue: out [S_rows,N] =
+ * act(tokens [S_rows,K] @ W[g]) per group; for MOE_ACT_SWIGLU `packed` holds (Wg,Wu) interleaved and
+ * out = silu(x Wg) * (x Wu).  K % 64 == 0, N % 8 == 0.  (The two halves of moe_grouped_mlp.) */
+int moe_grouped_gemm_packed(const void* tokens, const void* packed, const int32_t* expert_cnt, int S_rows, int K,
+                            int N, int E_l, int act, void* out, moe_stream_t stream);
+
 /* ---- a12: expert MLP (not in the reference; shapes from the workload descriptions) ------------
  * act GELU/SILU: y = act(x W1) W2;  SWIGLU: y = (silu(x Wg) * (x Wu)) Wd.
  * MOE_BF16: w1 = moe_prepack_weights(W1 or (Wg,Wu)) with K=H, N=F; w2 = moe_prepack_weights(W2)

@@ -47,6 +47,7 @@ _SIGNATURES = {
     "moe_prepack_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "moe_prepack_weights": (c_int, [P, P, c_int, c_int, c_int, c_int, P, P]),
     "moe_grouped_gemm": (c_int, [P, P, P, c_int, c_int, c_int, c_int, c_int, P, P, c_size_t, P]),
+    "moe_grouped_gemm_packed": (c_int, [P, P, P, c_int, c_int, c_int, c_int, c_int, P, P]),
     "moe_grouped_mlp": (c_int, [P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, P, P, P, P, P]),
     "moe_prepack_weights_fp8": (c_int, [P, P, c_int, c_int, c_int, P, P]),
     "moe_quantize_rows_fp8": (c_int, [P, c_int, c_int, P, P, P, P]),

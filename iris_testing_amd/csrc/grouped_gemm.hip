@@ -583,6 +583,20 @@ extern "C" int moe_grouped_gemm(const void* tokens, const void* weights, const i
     return launch_gemm<false>(p, EPI_NONE, s);
 }
 
+extern "C" int moe_grouped_gemm_packed(const void* tokens, const void* packed, const int32_t* expert_cnt, int S_rows, int K,
+                                       int N, int E_l, int act, void* out, moe_stream_t stream) {
+    MOE_REQUIRE(S_rows >= 0 && K > 0 && N > 0 && E_l > 0 && E_l <= GG_MAXG, MOE_ERR_INVALID, "grouped_gemm_packed: bad shape");
+    MOE_REQUIRE(act >= EPI_NONE && act <= EPI_SWIGLU, MOE_ERR_INVALID, "grouped_gemm_packed: activation %d", act);
+    MOE_REQUIRE(K % 64 == 0 && N % 8 == 0, MOE_ERR_UNSUPPORTED, "grouped_gemm_packed: needs K %% 64 == 0 and N %% 8 == 0 (K=%d N=%d)", K, N);
+    if (S_rows == 0) return MOE_OK;
+    MOE_REQUIRE(tokens && packed && expert_cnt && out, MOE_ERR_INVALID, "grouped_gemm_packed: null pointer");
+    GemmParams p{};
+    p.A = (const uint8_t*)tokens; p.B = (const uint8_t*)packed; p.C = out; p.cnt = expert_cnt;
+    p.E_l = E_l; p.K = K; p.N = N; p.ldc = N; p.S_rows = S_rows;
+    p.Npad = round_up(act == EPI_SWIGLU ? 2 * N : N, GG_BN);
+    return launch_gemm<false>(p, act, (hipStream_t)stream);
+}
+
 extern "C" int moe_grouped_mlp(const void* tokens, const int32_t* expert_cnt, int dtype, int S_rows, int H, int F, int E_l,
                                int act, const void* w1, const void* w_up, const void* w2, void* hidden_ws, void* out,
                                moe_stream_t stream) {

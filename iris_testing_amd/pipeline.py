@@ -1,0 +1,156 @@
+"""The whole hot path of one step on rank 0, with every buffer allocated once up front.
+
+A step = what rank 0 does for one batch:
+  as a source       route + top-k  ->  counts / offsets / positions  ->  pack into [W,M,H]
+  as a destination  expert-major unpack of its receive buffer  ->  grouped expert MLP  ->  return pack
+  as a source       top-k-weighted combine of the returned buffer into token order
+The two transfers in between are not part of a one-GPU build: the receive buffer and the returned
+buffer are assembled beforehand (harness.build_world) and stay fixed.  Each stage is one C-ABI call
+on the current stream; no stage synchronises or allocates.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from . import _lib as L
+from .harness import World
+from .layers.expert import ExpertWeights
+
+STAGES = ["route", "count", "pack", "unpack", "mlp_up", "mlp_down", "return_pack", "combine"]
+
+
+class DispatchPipeline:
+    def __init__(self, world: World, weights: ExpertWeights, returned: Optional[torch.Tensor] = None):
+        cfg = world.cfg
+        self.world, self.cfg, self.weights = world, cfg, weights
+        dev = world.x0.device
+        T, H, E, k, W, E_l, F = cfg.tokens, cfg.hidden, cfg.experts, cfg.topk, cfg.world, cfg.e_local, cfg.ffn
+        M, S = world.M, world.S
+        self.S = S
+        dt = cfg.torch_dtype
+        i32 = lambda *s: torch.empty(s, dtype=torch.int32, device=dev)  # noqa: E731
+        lib = L.lib()
+        self.code = L.dtype_code(dt)
+        # source side
+        self.logits = torch.empty((T, E), dtype=torch.float32, device=dev)
+        self.idx, self.gate = i32(T, k), torch.empty((T, k), dtype=torch.float32, device=dev)
+        self.send_counts, self.expert_offs = i32(W, E_l), i32(W, E_l)
+        self.dst_sizes, self.dst_offsets, self.caps = i32(W), i32(W), i32(2)
+        self.pos, self.row_token = i32(T, k), i32(T * k)
+        self.count_ws_bytes = lib.moe_count_workspace_bytes(T, k, E)
+        self.count_ws = torch.empty(self.count_ws_bytes, dtype=torch.uint8, device=dev)
+        self.send = torch.empty((W, M, H), dtype=dt, device=dev)
+        self.send_map = i32(W * M)
+        self.status = torch.zeros(1, dtype=torch.int32, device=dev)
+        # destination side
+        self.rows = torch.empty((S, H), dtype=dt, device=dev)
+        self.expert_cnt = i32(E_l)
+        self.unpack_map = i32(lib.moe_recv_map_ints(W, E_l, S))
+        self.hidden = torch.empty((S, F), dtype=dt, device=dev)
+        self.y = torch.zeros((S, H), dtype=dt, device=dev)
+        self.ret = torch.empty((W, M, H), dtype=dt, device=dev)
+        self.ret_map = i32(lib.moe_recv_map_ints(W, E_l, W * M))
+        if weights.dtype == torch.uint8:
+            self.xq = torch.empty((S, H), dtype=torch.uint8, device=dev)
+            self.xs = torch.empty((S,), dtype=torch.float32, device=dev)
+            self.hq = torch.empty((S, F), dtype=torch.uint8, device=dev)
+            self.hs = torch.empty((S,), dtype=torch.float32, device=dev)
+        # source side again: what comes back ([W,M,H], same slots as `send`) and the combined output
+        self.returned = returned if returned is not None else torch.zeros((W, M, H), dtype=dt, device=dev)
+        self.out = torch.empty((T, H), dtype=dt, device=dev)
+        self._p = L.ptr
+
+    # each stage is a closure-free method so that callers can time them one by one
+    def route(self, s):
+        c, w = self.cfg, self.world
+        L.check(L.lib().moe_route_topk(self._p(w.x0), self._p(w.router), self._p(w.bias), self.code, c.tokens, c.hidden,
+                                       c.experts, c.topk, self._p(self.logits), self._p(self.idx), self._p(self.gate), s))
+
+    def count(self, s):
+        c = self.cfg
+        L.check(L.lib().moe_count_and_offsets(self._p(self.idx), c.tokens, c.topk, c.experts, c.world,
+                                              self._p(self.send_counts), self._p(self.expert_offs), self._p(self.dst_sizes),
+                                              self._p(self.dst_offsets), self._p(self.caps), self._p(self.pos),
+                                              self._p(self.row_token), self._p(self.count_ws), self.count_ws_bytes, s))
+
+    def pack(self, s):
+        c, w = self.cfg, self.world
+        L.check(L.lib().moe_pack(self._p(w.x0), self.code, c.tokens, c.hidden, self._p(self.row_token),
+                                 self._p(self.dst_sizes), self._p(self.dst_offsets), c.world, w.M, self._p(self.send),
+                                 self._p(self.send_map), self._p(self.status), s))
+
+    def unpack(self, s):
+        c, w = self.cfg, self.world
+        L.check(L.lib().moe_unpack_expert_major(self._p(w.recv), self.code, c.world, w.M, c.hidden, self._p(w.recv_counts),
+                                                c.e_local, self._p(self.rows), self.S, self._p(self.expert_cnt),
+                                                self._p(self.unpack_map), s))
+
+    def mlp_up(self, s):
+        c, ew = self.cfg, self.weights
+        lib = L.lib()
+        if ew.dtype == torch.uint8:
+            sg, su, sd = ew.scales
+            # the fp8 entry point runs quantise + gate/up + quantise + down in one call
+            L.check(lib.moe_grouped_mlp_fp8(self._p(self.rows), self._p(self.expert_cnt), self.S, c.hidden, c.ffn, c.e_local,
+                                            self._p(ew.w1), self._p(sg), self._p(su), self._p(ew.w2), self._p(sd),
+                                            self._p(self.xq), self._p(self.xs), self._p(self.hidden), self._p(self.hq),
+                                            self._p(self.hs), self._p(self.y), s))
+        elif ew.dtype == torch.float32:
+            L.check(lib.moe_grouped_mlp(self._p(self.rows), self._p(self.expert_cnt), self.code, self.S, c.hidden, c.ffn,
+                                        c.e_local, L.ACT[ew.act], self._p(ew.w1), self._p(ew.w_up), self._p(ew.w2),
+                                        self._p(self.hidden), self._p(self.y), s))
+        else:
+            L.check(lib.moe_grouped_gemm_packed(self._p(self.rows), self._p(ew.w1), self._p(self.expert_cnt), self.S, c.hidden,
+                                                c.ffn, c.e_local, L.ACT[ew.act], self._p(self.hidden), s))
+
+    def mlp_down(self, s):
+        c, ew = self.cfg, self.weights
+        if ew.dtype == torch.bfloat16:
+            L.check(L.lib().moe_grouped_gemm_packed(self._p(self.hidden), self._p(ew.w2), self._p(self.expert_cnt), self.S,
+                                                    c.ffn, c.hidden, c.e_local, 0, self._p(self.y), s))
+
+    def return_pack(self, s):
+        c, w = self.cfg, self.world
+        L.check(L.lib().moe_return_pack(self._p(self.y), self.code, self.S, c.hidden, self._p(w.recv_counts), c.world,
+                                        c.e_local, w.M, self._p(self.ret), self._p(self.ret_map), s))
+
+    def combine(self, s):
+        c, w = self.cfg, self.world
+        L.check(L.lib().moe_combine(self._p(self.returned), self.code, c.world, w.M, c.hidden, self._p(self.idx),
+                                    self._p(self.pos), self._p(self.gate), self._p(self.dst_offsets), c.tokens, c.topk,
+                                    c.e_local, self._p(self.out), s))
+
+    def step(self, events: Optional[List[Dict[str, tuple]]] = None):
+        """One pass of the hot path.  With ``events`` (a list), per-stage (start, end) torch.cuda.Event
+        pairs of this step are appended to it."""
+        s = L.stream_ptr()
+        rec = {} if events is not None else None
+        for name in STAGES:
+            if rec is not None:
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+            getattr(self, name)(s)
+            if rec is not None:
+                b.record()
+                rec[name] = (a, b)
+        if events is not None:
+            events.append(rec)
+
+    # ---- algorithmic work per stage (bytes for the HBM-bound ones, flops for the GEMMs) ---------
+    def work(self) -> Dict[str, dict]:
+        c, w = self.cfg, self.world
+        T, H, E, k, W, F = c.tokens, c.hidden, c.experts, c.topk, c.world, c.ffn
+        B = 4 if c.dtype == "f32" else 2
+        S, M = self.S, w.M
+        up_mats = 2 if c.act == "swiglu" else 1
+        return {
+            "route": dict(bound="hbm", amount=T * H * B + H * E * B + T * k * 8),
+            "pack": dict(bound="hbm", amount=T * H * B + W * M * H * B),
+            "unpack": dict(bound="hbm", amount=2 * S * H * B),
+            "mlp_up": dict(bound="mfma", amount=2 * S * H * F * up_mats),
+            "mlp_down": dict(bound="mfma", amount=2 * S * F * H),
+            "return_pack": dict(bound="hbm", amount=S * H * B + W * M * H * B),
+            "combine": dict(bound="hbm", amount=T * k * H * B + T * H * B + T * k * 8),
+        }

@@ -508,14 +508,13 @@ def expert_mlp(tokens, cnt, w1, w2, act: str, dtype: str = "bf16", w_up=None):
     return round_to(y, dtype)
 
 
-def expert_mlp_fp8(tokens, cnt, wg_q, wg_s, wu_q, wu_s, wd_q, wd_s):
-    """fp8 SwiGLU expert: bf16 activations quantised per token to e4m3, e4m3 weights with
-    per-output-channel fp32 scales, fp32 accumulation, epilogue acc * s_tok[m] * s_ch[n];
-    the hidden activation is rounded to bf16, re-quantised per row, and the output is bf16.
-    """
+def expert_up_fp8(tokens, cnt, wg_q, wg_s, wu_q, wu_s):
+    """First half of the fp8 SwiGLU expert: bf16 rows quantised per token to e4m3, e4m3 weights with
+    per-output-channel fp32 scales, fp32 accumulation, epilogue acc * s_tok[m] * s_ch[n], then
+    h = silu(g) * u rounded to bf16.  [S,H] -> [S,F]."""
     S, H = tokens.shape
     E_l = wg_q.shape[0]
-    y = np.zeros((S, wd_q.shape[2]), dtype=np.float32)
+    h = np.zeros((S, wg_q.shape[2]), dtype=np.float32)
     xq, xs = quantize_rows_fp8(tokens)
     xf = fp8_e4m3_decode(xq)
     r = 0
@@ -526,12 +525,30 @@ def expert_mlp_fp8(tokens, cnt, wg_q, wg_s, wu_q, wu_s, wd_q, wd_s):
             sx = xs[r:r + c, None]
             g = ((xe @ fp8_e4m3_decode(wg_q[e])) * sx).astype(np.float32) * wg_s[e][None, :]
             u = ((xe @ fp8_e4m3_decode(wu_q[e])) * sx).astype(np.float32) * wu_s[e][None, :]
-            h = bf16_round((act_silu(g.astype(np.float32)) * u.astype(np.float32)).astype(np.float32))
-            hq, hs = quantize_rows_fp8(h)
-            o = ((fp8_e4m3_decode(hq) @ fp8_e4m3_decode(wd_q[e])) * hs[:, None]).astype(np.float32) * wd_s[e][None, :]
-            y[r:r + c] = o
+            h[r:r + c] = (act_silu(g.astype(np.float32)) * u.astype(np.float32)).astype(np.float32)
+        r += c
+    return bf16_round(h)
+
+
+def expert_down_fp8(h, cnt, wd_q, wd_s):
+    """Second half: the bf16 hidden activation is re-quantised per row, multiplied by the e4m3 down
+    projection, scaled, and rounded to bf16.  [S,F] -> [S,H]."""
+    E_l = wd_q.shape[0]
+    y = np.zeros((h.shape[0], wd_q.shape[2]), dtype=np.float32)
+    hq, hs = quantize_rows_fp8(h)
+    hf = fp8_e4m3_decode(hq)
+    r = 0
+    for e in range(E_l):
+        c = int(cnt[e])
+        if c:
+            y[r:r + c] = ((hf[r:r + c] @ fp8_e4m3_decode(wd_q[e])) * hs[r:r + c, None]).astype(np.float32) * wd_s[e][None, :]
         r += c
     return bf16_round(y)
+
+
+def expert_mlp_fp8(tokens, cnt, wg_q, wg_s, wu_q, wu_s, wd_q, wd_s):
+    """fp8 SwiGLU expert = expert_down_fp8(expert_up_fp8(x)).  Not in the reference."""
+    return expert_down_fp8(expert_up_fp8(tokens, cnt, wg_q, wg_s, wu_q, wu_s), cnt, wd_q, wd_s)
 
 
 # --------------------------------------------------------------------------------------

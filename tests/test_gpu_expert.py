@@ -21,9 +21,9 @@ DEV = "cuda"
 # propagated rounding of the hidden activation.  Bound used: |err| <= BF16_RTOL*|ref| + BF16_ATOL*rms(ref).
 BF16_RTOL, BF16_ATOL = 2.0 ** -6, 2.0 ** -6
 F32_RTOL, F32_ATOL = 1e-4, 1e-5
-# fp8: same quantised inputs on both sides (quantisation is part of the spec), error again only from
-# accumulation order and from re-quantising a hidden activation that differs in its last bf16 bit.
-FP8_RTOL, FP8_ATOL = 2.0 ** -4, 2.0 ** -5
+# fp8 end to end (see test_expert_mlp_fp8): a one-bit difference in a hidden row's amax re-codes a few
+# per cent of that row in fp8 (steps of 2^-3 relative), so single outputs may move by ~0.1 rms.
+FP8_RTOL, FP8_ATOL = 2.0 ** -4, 2.0 ** -3
 
 
 def _check(got, want, rtol, atol, what):
@@ -126,6 +126,10 @@ def test_quantize_rows_fp8_bit_exact(R, C):
 
 @pytest.mark.parametrize("E_l,H,F,S", [(2, 256, 384, 400), (15, 2048, 1408, 2500)])
 def test_expert_mlp_fp8(E_l, H, F, S):
+    """The two GEMMs are checked separately with tight bounds (the second one against the oracle fed
+    with the GPU's own hidden activation).  End to end the bound is loose on purpose: re-quantising
+    a hidden row whose amax differs in its last bf16 bit moves a few per cent of that row's fp8 codes
+    by one step, which is a property of the two-stage quantisation, not of the kernels."""
     rng = np.random.default_rng(H + F)
     cnt = _groups(rng, E_l, S)
     S_tot = int(cnt.sum())
@@ -136,9 +140,20 @@ def test_expert_mlp_fp8(E_l, H, F, S):
     (gq, gs), (uq, us), (dq, ds) = (O.quantize_cols_fp8(w) for w in (wg, wu, wd))
     tq = lambda a: torch.from_numpy(a).to(DEV)  # noqa: E731
     ew = ExpertWeights.prepare_fp8(tq(gq), tq(gs), tq(uq), tq(us), tq(dq), tq(ds))
-    out = to_np(expert_mlp(_t(x, "bf16"), ew, torch.from_numpy(cnt).to(DEV)))
+    ws = ops.fp8_workspace(S_tot, H, F, DEV)
+    sg, su, sd = ew.scales
+    out = to_np(ops.grouped_mlp_fp8(_t(x, "bf16"), torch.from_numpy(cnt).to(DEV), F, ew.w1, sg, su, ew.w2, sd, ws=ws))
+    h_gpu = to_np(ws["h"])
+    h_want = O.expert_up_fp8(x, cnt, gq, gs, uq, us)
+    _check(h_gpu, h_want.astype(np.float64), BF16_RTOL, BF16_ATOL, f"fp8 gate/up GEMM + SwiGLU E_l={E_l} H={H} F={F}")
+    y_from_gpu_h = O.expert_down_fp8(h_gpu, cnt, dq, ds)
+    _check(out, y_from_gpu_h.astype(np.float64), BF16_RTOL, BF16_ATOL, f"fp8 down GEMM E_l={E_l} H={H} F={F}")
     want = O.expert_mlp_fp8(x, cnt, gq, gs, uq, us, dq, ds)
-    _check(out, want.astype(np.float64), FP8_RTOL, FP8_ATOL, f"expert_mlp_fp8 E_l={E_l} H={H} F={F}")
-    # and against the unquantised fp32 MLP, to show what the quantisation itself costs (reported only)
+    _check(out, want.astype(np.float64), FP8_RTOL, FP8_ATOL, f"expert_mlp_fp8 end to end E_l={E_l} H={H} F={F}")
+    rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
+    tight = np.abs(out - want) <= BF16_RTOL * np.abs(want) + BF16_ATOL * rms
+    print(f"fraction of outputs within the bf16 bound end to end: {tight.mean():.6f}", flush=True)
+    assert tight.mean() > 0.99
+    # against the unquantised fp32 MLP, to show what the quantisation itself costs (reported only)
     ref = O.expert_mlp(x, cnt, wg, wd, "swiglu", "f32", w_up=wu)
     print("fp8 vs unquantised fp32 MLP:", err_stats(out, ref.astype(np.float64)), flush=True)
