@@ -98,15 +98,17 @@ __device__ __forceinline__ void gg_mmas(floatx16 (&acc)[TM][TN], const uint4 (&a
         for (int j = 0; j < TN; ++j) mma<FP8>(acc[i][j], b[j], a[i]);
 }
 
+// s_waitcnt through the builtin (not inline asm) so that the compiler's own wait-count bookkeeping
+// sees it.  gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14.
+template <int VM, int LGKM>
+__device__ __forceinline__ void gg_wait() {
+    static_assert(VM >= 0 && VM <= 63 && LGKM >= 0 && LGKM <= 15, "wait counts");
+    __builtin_amdgcn_s_waitcnt((VM & 15) | (7 << 4) | (LGKM << 8) | ((VM >> 4) << 14));
+}
 template <int N>
 __device__ __forceinline__ void gg_wait_vm() {
-    if constexpr (N == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    else if constexpr (N == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    else if constexpr (N == 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-    else if constexpr (N == 16) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    else static_assert(N == 0, "add the wait count");
+    gg_wait<N, 15>();
 }
-
 
 // acc(i,j) holds the TRANSPOSED 32x32 product (weights as the MFMA A operand, activations as B):
 // lane l owns token row l%32 and output columns 8*(v/4) + 4*(l/32) + v%4, v = 0..15, i.e. four runs
@@ -187,13 +189,15 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         if (rv <= 0) continue;
 
         const uint8_t* Ab = p.A + (size_t)row0 * p.K * ES;
-        const uint8_t* Bb = p.B + ((size_t)g * p.Npad + (size_t)nt * BN) * p.K * ES;
+        // packed weights are slab-major: [group][K slab of ROWB bytes][Npad rows][ROWB bytes]
+        const uint8_t* Bb = p.B + (size_t)g * p.Npad * p.K * ES + (size_t)nt * BN * ROWB;
+        const size_t b_slab = (size_t)p.Npad * ROWB;
         const uint32_t ldk = (uint32_t)(p.K * ES);
         uint32_t a_off[RA];
 #pragma unroll
         for (int r = 0; r < RA; ++r) a_off[r] = (uint32_t)min(r * LR + lrow, rv - 1) * ldk + lchunk * 16;
-        const uint32_t b_off0 = (uint32_t)lrow * ldk + lchunk * 16;
-        const uint32_t b_step = (uint32_t)LR * ldk;
+        const uint32_t b_off0 = (uint32_t)lrow * ROWB + lchunk * 16;
+        const uint32_t b_step = (uint32_t)LR * ROWB;
 
         floatx16 acc[TM][TN];
 #pragma unroll
@@ -204,6 +208,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
         uint4 a0[TM], b0[TN], a1[TM], b1[TN];
+        constexpr int NMMA = TM * TN * (FP8 ? 2 : 1);  // MFMA instructions per fragment step
         const int pos0 = (0 + khalf) ^ fswz, pos1 = (2 + khalf) ^ fswz, pos2 = (4 + khalf) ^ fswz, pos3 = (6 + khalf) ^ fswz;
         static_assert(NKK == 4, "GG_STAGE is written for four fragment steps");
 
@@ -211,20 +216,27 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         // the stage hand-over (loads landed + barrier + refill of the buffer just drained) sits before
         // the last MFMA block so that its latency hides behind that block.
 #define GG_ISSUE(sA, sB, ks) \
-    gg_issue<RA, RB, LR>(sA, sB, Ab + (size_t)(ks) * ROWB, Bb + (size_t)(ks) * ROWB, a_off, b_off0, b_step, wave)
+    gg_issue<RA, RB, LR>(sA, sB, Ab + (size_t)(ks) * ROWB, Bb + (size_t)(ks) * b_slab, a_off, b_off0, b_step, wave)
+#define GG_ORDER()                                                          \
+    do {                                                                    \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                  \
+        __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);            \
+        __builtin_amdgcn_sched_group_barrier(0x008, NMMA - 1, 0);           \
+        __builtin_amdgcn_sched_barrier(0);                                  \
+    } while (0)
 #define GG_STAGE(fa, fb, na, nb, curA, curB, ks)                           \
     do {                                                                   \
         gg_frags<TM, TN>(fa, fb, pos1, a1, b1);                            \
         gg_mmas<TM, TN, FP8>(acc, a0, b0);                                 \
-        __builtin_amdgcn_sched_barrier(0);                                 \
+        GG_ORDER();                                                        \
         gg_frags<TM, TN>(fa, fb, pos2, a0, b0);                            \
         gg_mmas<TM, TN, FP8>(acc, a1, b1);                                 \
-        __builtin_amdgcn_sched_barrier(0);                                 \
+        GG_ORDER();                                                        \
         gg_frags<TM, TN>(fa, fb, pos3, a1, b1);                            \
         gg_mmas<TM, TN, FP8>(acc, a0, b0);                                 \
-        __builtin_amdgcn_sched_barrier(0);                                 \
+        GG_ORDER();                                                        \
         if ((ks) + 1 < nk) {                                               \
-            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");    \
+            gg_wait<0, 0>();                                               \
             __syncthreads();                                               \
             if ((ks) + 2 < nk) GG_ISSUE(curA, curB, (ks) + 2);             \
             gg_frags<TM, TN>(na, nb, pos0, a0, b0);                        \
@@ -249,6 +261,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             if (ks + 1 < nk) GG_STAGE(fa1, fb1, fa0, fb0, sA1, sB1, ks + 1);
         }
 #undef GG_STAGE
+#undef GG_ORDER
 #undef GG_ISSUE
 
         // ---- epilogue: acc -> (scales) -> activation -> bf16 -> C
@@ -316,7 +329,8 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     }
 }
 
-// ---- one-time weight re-tiling: w [E_l,K,N] (N contiguous) -> out [E_l,Npad,K] (K contiguous) -------
+// ---- one-time weight re-tiling: w [E_l,K,N] (N contiguous) -> out [E_l][K/SK][Npad][SK], SK = one LDS
+// stage of K (ROWB bytes): the B tile of a stage is one contiguous 32 KB block -----------------------
 // With w_up, gate and up columns are interleaved in groups of 32: packed col = (n/32)*64 + {0,32} + n%32.
 template <typename T>
 __global__ __launch_bounds__(256) void prepack_kernel(const T* __restrict__ w, const T* __restrict__ w_up, T* __restrict__ out,
@@ -327,6 +341,7 @@ __global__ __launch_bounds__(256) void prepack_kernel(const T* __restrict__ w, c
     const T* src = w + (size_t)e * K * N;
     const T* src2 = w_up ? w_up + (size_t)e * K * N : nullptr;
     T* dst = out + (size_t)e * Npad * K;
+    constexpr int SK = ROWB / (int)sizeof(T);  // K elements per slab
     for (int pass = 0; pass < (src2 ? 2 : 1); ++pass) {
         const T* s = pass ? src2 : src;
         for (int i = threadIdx.x; i < 64 * 64; i += 256) {
@@ -339,7 +354,8 @@ __global__ __launch_bounds__(256) void prepack_kernel(const T* __restrict__ w, c
             const int n = n0 + nn;
             if (n < N && k0 + kk < K) {
                 const int np = src2 ? ((n >> 5) * 64 + pass * 32 + (n & 31)) : n;
-                dst[(size_t)np * K + k0 + kk] = tile[kk][nn];
+                const int k = k0 + kk;
+                dst[((size_t)(k / SK) * Npad + np) * SK + (k % SK)] = tile[kk][nn];
             }
         }
         __syncthreads();
@@ -348,11 +364,16 @@ __global__ __launch_bounds__(256) void prepack_kernel(const T* __restrict__ w, c
 
 template <typename T>
 __global__ void zero_pad_rows_kernel(T* __restrict__ out, int K, int Nreal, int Npad) {
-    // rows [Nreal, Npad) of every expert's packed matrix
+    // rows [Nreal, Npad) of every K slab of every expert's packed matrix
+    constexpr int SK = ROWB / (int)sizeof(T);
     const int e = blockIdx.y;
-    const size_t n = (size_t)(Npad - Nreal) * K;
-    T* dst = out + ((size_t)e * Npad + Nreal) * K;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) dst[i] = (T)0;
+    const size_t per_slab = (size_t)(Npad - Nreal) * SK;
+    const size_t n = per_slab * (size_t)(K / SK);
+    T* dst = out + (size_t)e * Npad * K;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t slab = i / per_slab, r = i % per_slab;
+        dst[(slab * Npad + Nreal) * SK + r] = (T)0;
+    }
 }
 
 // ---- fp32 path: plain tiled FMA kernel, weights in the reference layout ------------------------------
