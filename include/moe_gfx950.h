@@ -87,8 +87,8 @@ int moe_pack_payload(const void* x, int dtype, int T, int H, const int32_t* row_
 
 /* ---- a8: fixed [W,M,H] send layout (reference README.md:5-7) ----------------------------------
  * send[dst,m,:] = x[row_token[dst_offsets[dst]+m],:] for m < dst_sizes[dst], else zeros.
- * map_ws: int32 [W*M] scratch.  status (nullable): set to 1 if some dst_sizes[dst] > M (rows beyond
- * M are dropped). */
+ * map_ws: unused (kept for ABI stability; may be NULL).  status (nullable): set to 1 if some
+ * dst_sizes[dst] > M (rows beyond M are dropped). */
 int moe_pack(const void* x, int dtype, int T, int H, const int32_t* row_token, const int32_t* dst_sizes,
              const int32_t* dst_offsets, int W, int M, void* send_buf, int32_t* map_ws, int32_t* status,
              moe_stream_t stream);
@@ -99,7 +99,8 @@ int moe_pack(const void* x, int dtype, int T, int H, const int32_t* row_token, c
  * token_buf[e,s,j,:] = recv[s, expert_offs_s[e]+j, :] for j < recv_counts[s,e], else zeros;
  * pca[e,s] = recv_counts[s,e].  status (nullable): 1 on count > CAP.
  * map_ws (here and in every entry point below that takes one): int32 scratch of
- * moe_recv_map_ints(W, E_l, n_out) elements, n_out = rows of the output buffer. */
+ * moe_recv_map_ints(W, E_l, n_out) elements (prefix tables over the counts; n_out = rows of the
+ * output buffer, which no longer enters the size). */
 size_t moe_recv_map_ints(int W, int E_l, int n_out);
 int moe_unpack_token_buf(const void* recv, int dtype, int W, int M, int H, const int32_t* recv_counts, int E_l,
                          int CAP, void* token_buf, int32_t* pca, int32_t* map_ws, int32_t* status,
@@ -133,8 +134,9 @@ size_t moe_prepack_bytes(int dtype, int E_l, int K, int N);
 int moe_grouped_gemm(const void* tokens, const void* weights, const int32_t* expert_cnt, int dtype, int S_rows,
                      int K, int N, int E_l, void* out, void* ws, size_t ws_bytes, moe_stream_t stream);
 
-/* One-time weight re-tiling for the MFMA kernels: [E_l,K,N] (N contiguous) -> [E_l,Npad,K]
- * (K contiguous, Npad = N rounded up to the kernel's N tile).  With w_up != NULL the two
+/* One-time weight re-tiling for the MFMA kernels: [E_l,K,N] (N contiguous) -> K-contiguous rows grouped
+ * in K slabs ([E_l][K/slab][Npad][slab], Npad = N rounded up to the kernel's N tile; the layout is
+ * private to the kernels).  With w_up != NULL the two
  * matrices are interleaved in 32-column groups (gate, up, gate, up, ...) so one kernel computes
  * silu(x Wg) * (x Wu); the packed matrix then has 2N columns. */
 int moe_prepack_weights(const void* w, const void* w_up, int dtype, int E_l, int K, int N, void* packed,

@@ -150,18 +150,6 @@ __global__ void max_floor1_kernel(const int32_t* __restrict__ v, int n, int32_t*
     if (threadIdx.x == 0) out[0] = red[0];
 }
 
-// send map: map[d*M+m] = token for m < dst_sizes[d], else -1
-__global__ void send_map_kernel(const int32_t* __restrict__ row_token, const int32_t* __restrict__ dst_sizes,
-                                const int32_t* __restrict__ dst_offsets, int W, int M, int32_t* __restrict__ map,
-                                int32_t* __restrict__ status) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= W * M) return;
-    const int d = i / M, m = i % M;
-    const int n = dst_sizes[d];
-    if (m == 0 && n > M && status) *status = 1;
-    map[i] = m < n ? row_token[dst_offsets[d] + m] : -1;
-}
-
 // Tables derived from recv_counts [W,E_l] (one block):
 //   src_off[s*E_l+e] = exclusive prefix over e of recv_counts[s,:]   (row inside slot s)
 //   row_off[e*W+s]   = exclusive prefix over flattened (e,s) of recv_counts[s,e]  (+ total at [E_l*W])
@@ -224,73 +212,102 @@ __global__ __launch_bounds__(WAVE) void expert_offsets_kernel(const int32_t* __r
     }
 }
 
-__device__ __forceinline__ int upper_seg(const int32_t* off, int n, int r) {
-    // largest i in [0,n) with off[i] <= r   (off ascending, off[0] = 0)
-    int lo = 0, hi = n;
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (off[mid] <= r) lo = mid; else hi = mid;
+// ---- row movement: dst[r,:] = src[source_row(r),:], or zeros when the row has no source ---------------
+// One wave per output row, 16 bytes per lane.  The source row is resolved inside the kernel (no map
+// buffer, no extra launch); every quantity involved is wave-uniform.
+enum {
+    SRC_MAP = 0,      // map[r]                                  (padding-free payload)
+    SRC_PACK = 1,     // send slot (d,m) -> token                (fixed [W,M,H] pack)
+    SRC_UNPACK = 2,   // expert-major row r -> recv row          (recv [W,M,H] -> [S,H])
+    SRC_TOKBUF = 3,   // token_buf row (e,s,j) -> recv row       (recv [W,M,H] -> [E_l,W,CAP,H])
+    SRC_RETURN = 4,   // return slot (s,m) -> expert-major row   ([S,H] -> [W,M,H])
+    SRC_REORDER = 5,  // token_buf row (e,s,j) -> flat row       (flat payload -> [E_l,W,CAP,H])
+    SRC_SHUFFLE = 6   // expert-major row r -> token_buf row     ([E_l,W,CAP,H] -> [S,H])
+};
+
+struct RowSource {
+    int mode;
+    const int32_t* map;                                   // SRC_MAP / SRC_PACK: row_token
+    const int32_t *dst_sizes, *dst_offsets;               // SRC_PACK
+    const int32_t *rc, *src_off, *row_off, *flat_off;     // recv-driven modes
+    int W, E_l, M, CAP;
+    int32_t* status;
+};
+
+// largest i in [0,n) with off[i] <= r (off ascending, off[0] = 0): the whole wave looks at 64 entries
+// at a time and counts them with a ballot.  Equal offsets mark empty segments; the last of a run of
+// equal offsets is the segment that owns the row.
+__device__ __forceinline__ int wave_seg(const int32_t* __restrict__ off, int n, int r) {
+    int total = 0;
+    for (int base = 0; base < n; base += WAVE) {
+        const int i = base + lane_id();
+        const bool le = i < n && off[i] <= r;
+        total += __popcll(__ballot(le));
     }
-    return lo;
+    return total - 1;
 }
 
-// mode 0: shuffled row r -> recv row (s*M + src_off[s,e] + j)
-// mode 1: token_buf row (e,s,j) -> recv row, or -1
-// mode 2: return slot (s,m) -> shuffled row off[e,s]+j, or -1
-// mode 3: token_buf row (e,s,j) -> flat payload row flat_off[s,e]+j, or -1
-// mode 4: shuffled row r -> token_buf row ((e*W+s)*CAP + j)
-__global__ void recv_map_kernel(int mode, const int32_t* __restrict__ rc, const int32_t* __restrict__ src_off,
-                                const int32_t* __restrict__ row_off, const int32_t* __restrict__ flat_off, int W,
-                                int E_l, int M, int CAP, int n_out, int32_t* __restrict__ map,
-                                int32_t* __restrict__ status) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n_out) return;
-    const int n = W * E_l;
-    int out = -1;
-    if (mode == 0 || mode == 4) {
-        const int S = row_off[n];
-        if (i < S) {
-            const int seg = upper_seg(row_off, n + 1, i);  // seg = e*W+s, skips empty segments by construction
-            const int e = seg / W, s = seg % W, j = i - row_off[seg];
-            out = mode == 0 ? s * M + src_off[s * E_l + e] + j : (e * W + s) * CAP + j;
+__device__ __forceinline__ int source_row(const RowSource& a, int r) {
+    const int n = a.W * a.E_l;
+    switch (a.mode) {
+        case SRC_MAP: return a.map[r];
+        case SRC_PACK: {
+            const int d = r / a.M, m = r % a.M;
+            const int cnt = a.dst_sizes[d];
+            if (m == 0 && cnt > a.M && a.status && lane_id() == 0) *a.status = 1;
+            return m < cnt ? a.map[a.dst_offsets[d] + m] : -1;
         }
-    } else if (mode == 1 || mode == 3) {
-        const int j = i % CAP, s = (i / CAP) % W, e = i / (CAP * W);
-        const int c = rc[s * E_l + e];
-        if (j == 0 && c > CAP && status) *status = 1;
-        if (j < c) out = mode == 1 ? s * M + src_off[s * E_l + e] + j : flat_off[s * E_l + e] + j;
-    } else {  // mode 2
-        const int s = i / M, m = i % M;
-        const int tot = src_off[s * E_l + E_l - 1] + rc[s * E_l + E_l - 1];
-        if (m < tot) {
-            const int e = upper_seg(src_off + s * E_l, E_l, m);
-            // upper_seg returns the LAST expert whose offset <= m, which is the non-empty one owning m
-            out = row_off[e * W + s] + (m - src_off[s * E_l + e]);
+        case SRC_UNPACK:
+        case SRC_SHUFFLE: {
+            if (r >= a.row_off[n]) return -1;
+            const int seg = wave_seg(a.row_off, n + 1, r);  // seg = e*W + s
+            const int e = seg / a.W, s = seg % a.W, j = r - a.row_off[seg];
+            return a.mode == SRC_UNPACK ? s * a.M + a.src_off[s * a.E_l + e] + j : (e * a.W + s) * a.CAP + j;
+        }
+        case SRC_TOKBUF:
+        case SRC_REORDER: {
+            const int j = r % a.CAP, s = (r / a.CAP) % a.W, e = r / (a.CAP * a.W);
+            const int c = a.rc[s * a.E_l + e];
+            if (j == 0 && c > a.CAP && a.status && lane_id() == 0) *a.status = 1;
+            if (j >= c) return -1;
+            return a.mode == SRC_TOKBUF ? s * a.M + a.src_off[s * a.E_l + e] + j : a.flat_off[s * a.E_l + e] + j;
+        }
+        default: {  // SRC_RETURN
+            const int s = r / a.M, m = r % a.M;
+            const int32_t* so = a.src_off + s * a.E_l;
+            const int tot = so[a.E_l - 1] + a.rc[s * a.E_l + a.E_l - 1];
+            if (m >= tot) return -1;
+            const int e = wave_seg(so, a.E_l, m);
+            return a.row_off[e * a.W + s] + (m - so[e]);
         }
     }
-    map[i] = out;
 }
 
-// ---- row gather: dst[r,:] = map[r] >= 0 ? src[map[r],:] : 0 ; one wave per row, 16-byte lanes ----
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
 template <int WPB>
-__global__ __launch_bounds__(WPB * WAVE) void gather_rows_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
-                                                                  const int32_t* __restrict__ map, int n_rows,
+__global__ __launch_bounds__(WPB * WAVE) void gather_rows_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst,
+                                                                  const RowSource a, int n_rows,
                                                                   int row_vec /* 16-byte units per row */) {
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     for (int r = blockIdx.x * WPB + wave; r < n_rows; r += gridDim.x * WPB) {
-        const int m = map[r];
-        uint4* d = dst + (size_t)r * row_vec;
+        const int m = source_row(a, r);
+        u32x4* d = dst + (size_t)r * row_vec;
         if (m >= 0) {
-            const uint4* s = src + (size_t)m * row_vec;
+            // streaming copy: every byte is touched once, so loads and stores bypass cache retention
+            const u32x4* s = src + (size_t)m * row_vec;
             int c = lane;
-            for (; c + 3 * WAVE < row_vec; c += 4 * WAVE) {
-                const uint4 a0 = s[c], a1 = s[c + WAVE], a2 = s[c + 2 * WAVE], a3 = s[c + 3 * WAVE];
-                d[c] = a0; d[c + WAVE] = a1; d[c + 2 * WAVE] = a2; d[c + 3 * WAVE] = a3;
+            for (; c + 7 * WAVE < row_vec; c += 8 * WAVE) {
+                u32x4 v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(s + c + u * WAVE);
+#pragma unroll
+                for (int u = 0; u < 8; ++u) __builtin_nontemporal_store(v[u], d + c + u * WAVE);
             }
-            for (; c < row_vec; c += WAVE) d[c] = s[c];
+            for (; c < row_vec; c += WAVE) __builtin_nontemporal_store(__builtin_nontemporal_load(s + c), d + c);
         } else {
-            const uint4 z = make_uint4(0, 0, 0, 0);
-            for (int c = lane; c < row_vec; c += WAVE) d[c] = z;
+            const u32x4 z = {0u, 0u, 0u, 0u};
+            for (int c = lane; c < row_vec; c += WAVE) __builtin_nontemporal_store(z, d + c);
         }
     }
 }
@@ -324,33 +341,42 @@ struct Vec16<float> {
     }
 };
 
-template <typename XT, int WPB>
+// KT = compile-time top-k (1,2,4,8) or 0 for a run-time k up to MOE_MAX_TOPK.  All k row reads of a
+// 16-byte column are issued before the first is used.
+template <typename XT, int KT, int WPB>
 __global__ __launch_bounds__(WPB * WAVE) void combine_kernel(const uint4* __restrict__ ret, const int32_t* __restrict__ idx,
                                                               const int32_t* __restrict__ pos, const float* __restrict__ gate,
-                                                              const int32_t* __restrict__ dst_offsets, int T, int k, int E_l,
+                                                              const int32_t* __restrict__ dst_offsets, int T, int k_rt, int E_l,
                                                               int M, int row_vec, uint4* __restrict__ out) {
     constexpr int N = Vec16<XT>::N;
+    constexpr int KMAX = KT ? KT : MOE_MAX_TOPK;
+    const int k = KT ? KT : k_rt;
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     for (int t = blockIdx.x * WPB + wave; t < T; t += gridDim.x * WPB) {
-        size_t rows[MOE_MAX_TOPK];
-        float g[MOE_MAX_TOPK];
+        size_t rows[KMAX];
+        float g[KMAX];
 #pragma unroll
-        for (int j = 0; j < MOE_MAX_TOPK; ++j) {
+        for (int j = 0; j < KMAX; ++j) {
             if (j < k) {
                 const int d = idx[(size_t)t * k + j] / E_l;
                 rows[j] = ((size_t)d * M + (pos[(size_t)t * k + j] - dst_offsets[d])) * row_vec;
                 g[j] = gate[(size_t)t * k + j];
             }
         }
+#pragma unroll 2
         for (int c = lane; c < row_vec; c += WAVE) {
+            uint4 v[KMAX];
+#pragma unroll
+            for (int j = 0; j < KMAX; ++j)
+                if (j < k) v[j] = ret[rows[j] + c];
             float acc[N];
 #pragma unroll
             for (int i = 0; i < N; ++i) acc[i] = 0.f;
 #pragma unroll
-            for (int j = 0; j < MOE_MAX_TOPK; ++j) {
+            for (int j = 0; j < KMAX; ++j) {
                 if (j < k) {
                     float f[N];
-                    Vec16<XT>::unpack(ret[rows[j] + c], f);
+                    Vec16<XT>::unpack(v[j], f);
 #pragma unroll
                     for (int i = 0; i < N; ++i) acc[i] = __fadd_rn(acc[i], __fmul_rn(g[j], f[i]));
                 }
@@ -360,10 +386,27 @@ __global__ __launch_bounds__(WPB * WAVE) void combine_kernel(const uint4* __rest
     }
 }
 
-int gather_rows(const void* src, void* dst, const int32_t* map, int n_rows, int row_bytes, hipStream_t s) {
+template <typename XT>
+int launch_combine(const void* ret, const int32_t* idx, const int32_t* pos, const float* gate, const int32_t* dst_offsets, int T,
+                   int k, int E_l, int M, int row_vec, void* out, hipStream_t s) {
+    const int blocks = min(ceil_div(T, 4), 65535 * 8);
+#define MOE_COMBINE(KT) \
+    combine_kernel<XT, KT, 4><<<blocks, 4 * WAVE, 0, s>>>((const uint4*)ret, idx, pos, gate, dst_offsets, T, k, E_l, M, row_vec, (uint4*)out)
+    switch (k) {
+        case 1: MOE_COMBINE(1); break;
+        case 2: MOE_COMBINE(2); break;
+        case 4: MOE_COMBINE(4); break;
+        case 8: MOE_COMBINE(8); break;
+        default: MOE_COMBINE(0); break;
+    }
+#undef MOE_COMBINE
+    return moe_check_launch("combine");
+}
+
+int gather_rows(const void* src, void* dst, const RowSource& a, int n_rows, int row_bytes, hipStream_t s) {
     if (n_rows == 0) return MOE_OK;
     const int blocks = min(ceil_div(n_rows, 4), 65535 * 8);
-    gather_rows_kernel<4><<<blocks, 4 * WAVE, 0, s>>>((const uint4*)src, (uint4*)dst, map, n_rows, row_bytes / 16);
+    gather_rows_kernel<4><<<blocks, 4 * WAVE, 0, s>>>((const u32x4*)src, (u32x4*)dst, a, n_rows, row_bytes / 16);
     return moe_check_launch("gather_rows");
 }
 
@@ -435,7 +478,10 @@ extern "C" int moe_pack_payload(const void* x, int dtype, int T, int H, const in
     MOE_REQUIRE(R >= 0 && T >= 0, MOE_ERR_INVALID, "pack_payload: bad shape");
     if (R == 0) return MOE_OK;
     MOE_REQUIRE(x && row_token && payload, MOE_ERR_INVALID, "pack_payload: null pointer");
-    return gather_rows(x, payload, row_token, R, H * dtype_size(dtype), (hipStream_t)stream);
+    RowSource a{};
+    a.mode = SRC_MAP;
+    a.map = row_token;
+    return gather_rows(x, payload, a, R, H * dtype_size(dtype), (hipStream_t)stream);
 }
 
 extern "C" int moe_pack(const void* x, int dtype, int T, int H, const int32_t* row_token, const int32_t* dst_sizes,
@@ -446,10 +492,16 @@ extern "C" int moe_pack(const void* x, int dtype, int T, int H, const int32_t* r
     if (rc) return rc;
     MOE_REQUIRE(W > 0 && M >= 1 && T >= 0, MOE_ERR_INVALID, "pack: bad shape W=%d M=%d", W, M);
     MOE_REQUIRE((long long)W * M < (1ll << 31), MOE_ERR_UNSUPPORTED, "pack: W*M too large");
-    MOE_REQUIRE(send_buf && map_ws && dst_sizes && dst_offsets, MOE_ERR_INVALID, "pack: null pointer");
-    const int n = W * M;
-    send_map_kernel<<<ceil_div(n, 256), 256, 0, s>>>(row_token, dst_sizes, dst_offsets, W, M, map_ws, status);
-    return gather_rows(x, send_buf, map_ws, n, H * dtype_size(dtype), s);
+    MOE_REQUIRE(send_buf && dst_sizes && dst_offsets, MOE_ERR_INVALID, "pack: null pointer");
+    (void)map_ws;
+    RowSource a{};
+    a.mode = SRC_PACK;
+    a.map = row_token;
+    a.dst_sizes = dst_sizes;
+    a.dst_offsets = dst_offsets;
+    a.M = M;
+    a.status = status;
+    return gather_rows(x, send_buf, a, W * M, H * dtype_size(dtype), s);
 }
 
 static int recv_driven(const char* who, int mode, const void* src, void* dst, int dtype, int H, const int32_t* rc_dev,
@@ -459,27 +511,33 @@ static int recv_driven(const char* who, int mode, const void* src, void* dst, in
     if (rc) return rc;
     MOE_REQUIRE(W > 0 && E_l > 0 && W * E_l <= MOE_MAX_EXPERTS, MOE_ERR_INVALID, "%s: bad W=%d E_l=%d", who, W, E_l);
     MOE_REQUIRE(n_out >= 0 && rc_dev && map_ws, MOE_ERR_INVALID, "%s: bad arguments", who);
-    int32_t* tables = map_ws + n_out;
+    int32_t* tables = map_ws;
     const int n = W * E_l;
     int32_t* src_off = tables;
     int32_t* row_off = tables + (n + 1);
     int32_t* flat_off = tables + 2 * (n + 1);
     recv_tables_kernel<<<1, WAVE, 0, s>>>(rc_dev, W, E_l, src_off, row_off, flat_off, pca, expert_cnt);
     if (n_out == 0) return moe_check_launch(who);
-    MOE_REQUIRE(dst && (src || mode == 3), MOE_ERR_INVALID, "%s: null pointer", who);  // an empty flat payload has no storage
-    recv_map_kernel<<<ceil_div(n_out, 256), 256, 0, s>>>(mode, rc_dev, src_off, row_off, flat_off, W, E_l, M, CAP, n_out,
-                                                        map_ws, status);
-    return gather_rows(src, dst, map_ws, n_out, H * dtype_size(dtype), s);
+    MOE_REQUIRE(dst && (src || mode == SRC_REORDER), MOE_ERR_INVALID, "%s: null pointer", who);  // an empty flat payload has no storage
+    RowSource a{};
+    a.mode = mode;
+    a.rc = rc_dev; a.src_off = src_off; a.row_off = row_off; a.flat_off = flat_off;
+    a.W = W; a.E_l = E_l; a.M = M; a.CAP = CAP;
+    a.status = status;
+    return gather_rows(src, dst, a, n_out, H * dtype_size(dtype), s);
 }
 
-extern "C" size_t moe_recv_map_ints(int W, int E_l, int n_out) { return (size_t)n_out + recv_tables_ints(W, E_l); }
+extern "C" size_t moe_recv_map_ints(int W, int E_l, int n_out) {
+    (void)n_out;  // the per-row map of earlier versions is gone: rows are resolved inside the gather kernel
+    return recv_tables_ints(W, E_l);
+}
 
 extern "C" int moe_unpack_token_buf(const void* recv, int dtype, int W, int M, int H, const int32_t* recv_counts,
                                     int E_l, int CAP, void* token_buf, int32_t* pca, int32_t* map_ws, int32_t* status,
                                     moe_stream_t stream) {
     MOE_REQUIRE(M >= 1 && CAP >= 1, MOE_ERR_INVALID, "unpack_token_buf: M=%d CAP=%d", M, CAP);
     MOE_REQUIRE((long long)E_l * W * CAP < (1ll << 31), MOE_ERR_UNSUPPORTED, "unpack_token_buf: too many rows");
-    return recv_driven("unpack_token_buf", 1, recv, token_buf, dtype, H, recv_counts, W, E_l, M, CAP, E_l * W * CAP, pca,
+    return recv_driven("unpack_token_buf", SRC_TOKBUF, recv, token_buf, dtype, H, recv_counts, W, E_l, M, CAP, E_l * W * CAP, pca,
                        nullptr, map_ws, status, (hipStream_t)stream);
 }
 
@@ -489,7 +547,7 @@ extern "C" int moe_reorder_flat_to_token_buf(const void* flat, int dtype, int R,
     (void)R;
     MOE_REQUIRE(CAP >= 1, MOE_ERR_INVALID, "reorder: CAP=%d", CAP);
     MOE_REQUIRE((long long)E_l * W * CAP < (1ll << 31), MOE_ERR_UNSUPPORTED, "reorder: too many rows");
-    return recv_driven("reorder_flat_to_token_buf", 3, flat, token_buf, dtype, H, recv_counts, W, E_l, 1, CAP,
+    return recv_driven("reorder_flat_to_token_buf", SRC_REORDER, flat, token_buf, dtype, H, recv_counts, W, E_l, 1, CAP,
                        E_l * W * CAP, nullptr, nullptr, map_ws, status, (hipStream_t)stream);
 }
 
@@ -497,7 +555,7 @@ extern "C" int moe_unpack_expert_major(const void* recv, int dtype, int W, int M
                                        int E_l, void* shuffled, int S_rows, int32_t* expert_cnt, int32_t* map_ws,
                                        moe_stream_t stream) {
     MOE_REQUIRE(M >= 1, MOE_ERR_INVALID, "unpack_expert_major: M=%d", M);
-    return recv_driven("unpack_expert_major", 0, recv, shuffled, dtype, H, recv_counts, W, E_l, M, 1, S_rows, nullptr,
+    return recv_driven("unpack_expert_major", SRC_UNPACK, recv, shuffled, dtype, H, recv_counts, W, E_l, M, 1, S_rows, nullptr,
                        expert_cnt, map_ws, nullptr, (hipStream_t)stream);
 }
 
@@ -513,9 +571,9 @@ extern "C" int moe_shuffle(const void* token_buf, int dtype, int E_l, int W, int
     MOE_REQUIRE(W > 0 && E_l > 0 && W * E_l <= MOE_MAX_EXPERTS && CAP >= 1 && S_rows >= 0 && pca && map_ws,
                 MOE_ERR_INVALID, "shuffle: bad arguments");
     // recv_counts[s,e] = pca[e,s], kept behind the tables in map_ws
-    int32_t* rc_t = map_ws + S_rows + recv_tables_ints(W, E_l);
+    int32_t* rc_t = map_ws + 3 * (W * E_l + 1);
     transpose_counts_kernel<<<ceil_div(W * E_l, 256), 256, 0, s>>>(pca, E_l, W, rc_t);
-    return recv_driven("shuffle", 4, token_buf, shuffled, dtype, H, rc_t, W, E_l, 1, CAP, S_rows, nullptr, expert_cnt,
+    return recv_driven("shuffle", SRC_SHUFFLE, token_buf, shuffled, dtype, H, rc_t, W, E_l, 1, CAP, S_rows, nullptr, expert_cnt,
                        map_ws, nullptr, s);
 }
 
@@ -524,7 +582,7 @@ extern "C" int moe_return_pack(const void* y, int dtype, int S_rows, int H, cons
     (void)S_rows;
     MOE_REQUIRE(M >= 1, MOE_ERR_INVALID, "return_pack: M=%d", M);
     MOE_REQUIRE((long long)W * M < (1ll << 31), MOE_ERR_UNSUPPORTED, "return_pack: W*M too large");
-    return recv_driven("return_pack", 2, y, ret, dtype, H, recv_counts, W, E_l, M, 1, W * M, nullptr, nullptr, map_ws,
+    return recv_driven("return_pack", SRC_RETURN, y, ret, dtype, H, recv_counts, W, E_l, M, 1, W * M, nullptr, nullptr, map_ws,
                        nullptr, (hipStream_t)stream);
 }
 
@@ -539,12 +597,6 @@ extern "C" int moe_combine(const void* ret, int dtype, int W, int M, int H, cons
     if (T == 0) return MOE_OK;
     MOE_REQUIRE(ret && topk_idx && pos && gate && dst_offsets && out, MOE_ERR_INVALID, "combine: null pointer");
     const int row_vec = H * dtype_size(dtype) / 16;
-    const int blocks = min(ceil_div(T, 4), 65535 * 8);
-    if (dtype == MOE_F32)
-        combine_kernel<float, 4><<<blocks, 4 * WAVE, 0, s>>>((const uint4*)ret, topk_idx, pos, gate, dst_offsets, T, k, E_l,
-                                                            M, row_vec, (uint4*)out);
-    else
-        combine_kernel<bf16_t, 4><<<blocks, 4 * WAVE, 0, s>>>((const uint4*)ret, topk_idx, pos, gate, dst_offsets, T, k,
-                                                             E_l, M, row_vec, (uint4*)out);
-    return moe_check_launch("combine");
+    if (dtype == MOE_F32) return launch_combine<float>(ret, topk_idx, pos, gate, dst_offsets, T, k, E_l, M, row_vec, out, s);
+    return launch_combine<bf16_t>(ret, topk_idx, pos, gate, dst_offsets, T, k, E_l, M, row_vec, out, s);
 }

@@ -129,6 +129,96 @@ __global__ __launch_bounds__(RT_THREADS) void route_logits_kernel(const XT* __re
     }
 }
 
+// Few experts (E <= 16): one thread per (token, EE experts).  Lane = token (64 tokens per block), wave w
+// owns experts [w*EE, w*EE+EE).  x goes through LDS in its storage type (the lane reads its own row 16
+// bytes at a time); the router slab is converted to fp32 once per slab and read back with broadcast
+// 128-bit LDS reads.  The next slab is fetched into registers while the current one is consumed.
+// Same reduction order as above: one fmaf chain per (t,e), ascending h.
+constexpr int RS_KC = 128;
+
+template <typename XT, int EE>
+__global__ __launch_bounds__(RT_THREADS) void route_logits_small_kernel(const XT* __restrict__ x, const XT* __restrict__ w,
+                                                                         const float* __restrict__ bias,
+                                                                         float* __restrict__ logits, int T, int H, int E) {
+    constexpr int VN = VecLoad<XT>::N;          // elements per 16 bytes
+    constexpr int XS = RS_KC + VN;              // padded row (16 bytes of padding: conflict-free b128 rows)
+    constexpr int XCH = RT_TB * (RS_KC / VN);   // 16-byte chunks of an x slab
+    constexpr int XPT = XCH / RT_THREADS;       // per thread
+    constexpr int WPT = 16 * RS_KC / RT_THREADS;  // router elements per thread per slab (16 expert rows)
+    __shared__ __align__(16) XT xs[RT_TB][XS];
+    __shared__ __align__(16) float wsT[16][RS_KC + 4];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int t0 = blockIdx.x * RT_TB;
+    const int e0 = wave * EE;
+    float acc[EE];
+#pragma unroll
+    for (int j = 0; j < EE; ++j) acc[j] = 0.f;
+
+    uint4 xr[XPT];
+    float wr[WPT];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < XPT; ++i) {
+            const int c = tid + i * RT_THREADS;
+            const int row = c / (RS_KC / VN), col = (c % (RS_KC / VN)) * VN;
+            const int t = t0 + row;
+            xr[i] = (t < T && k0 + col < H) ? *reinterpret_cast<const uint4*>(x + (size_t)t * H + k0 + col) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < WPT; ++i) {
+            const int c = tid + i * RT_THREADS;
+            const int kk = c / 16, e = c % 16;
+            wr[i] = (k0 + kk < H && e < E) ? load_f32<XT>(w + (size_t)(k0 + kk) * E + e) : 0.f;
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int i = 0; i < XPT; ++i) {
+            const int c = tid + i * RT_THREADS;
+            const int row = c / (RS_KC / VN), col = (c % (RS_KC / VN)) * VN;
+            *reinterpret_cast<uint4*>(&xs[row][col]) = xr[i];
+        }
+#pragma unroll
+        for (int i = 0; i < WPT; ++i) {
+            const int c = tid + i * RT_THREADS;
+            wsT[c % 16][c / 16] = wr[i];
+        }
+    };
+
+    fetch(0);
+    for (int k0 = 0; k0 < H; k0 += RS_KC) {
+        stash();
+        __syncthreads();
+        if (k0 + RS_KC < H) fetch(k0 + RS_KC);
+        const int kmax = min(RS_KC, H - k0);
+        for (int kk = 0; kk < kmax; kk += VN) {
+            float xv[VN];
+            VecLoad<XT>::load(&xs[lane][kk], xv);
+#pragma unroll
+            for (int q = 0; q < VN; q += 4) {
+#pragma unroll
+                for (int j = 0; j < EE; ++j) {
+                    const float4 wv = *reinterpret_cast<const float4*>(&wsT[e0 + j][kk + q]);
+                    acc[j] = fmaf(xv[q + 0], wv.x, acc[j]);
+                    acc[j] = fmaf(xv[q + 1], wv.y, acc[j]);
+                    acc[j] = fmaf(xv[q + 2], wv.z, acc[j]);
+                    acc[j] = fmaf(xv[q + 3], wv.w, acc[j]);
+                }
+            }
+        }
+        __syncthreads();
+    }
+    const int t = t0 + lane;
+    if (t < T) {
+#pragma unroll
+        for (int j = 0; j < EE; ++j) {
+            const int e = e0 + j;
+            if (e < E) logits[(size_t)t * E + e] = bias ? __fadd_rn(acc[j], bias[e]) : acc[j];
+        }
+    }
+}
+
 // Softmax gates + top-k.  G lanes cooperate on one token (G = 8,16,32,64); lane gl holds experts
 // gl, gl+G, gl+2G, ...  Selection key: (logit descending, expert id ascending).
 constexpr int TK_MAXV = 8;  // values per lane -> E <= 8*G
@@ -204,10 +294,14 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict_
 template <typename XT>
 int launch_logits(const XT* x, const XT* w, const float* bias, float* logits, int T, int H, int E, hipStream_t s) {
     const int gx = ceil_div(T, RT_TB);
-    if (E <= 8) {
-        route_logits_kernel<XT, 1, 2, 4><<<dim3(gx, ceil_div(E, 8)), RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
+    if (E <= 4) {
+        route_logits_small_kernel<XT, 1><<<gx, RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
+    } else if (E <= 8) {
+        route_logits_small_kernel<XT, 2><<<gx, RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
+    } else if (E <= 12) {
+        route_logits_small_kernel<XT, 3><<<gx, RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
     } else if (E <= 16) {
-        route_logits_kernel<XT, 1, 4, 4><<<dim3(gx, 1), RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
+        route_logits_small_kernel<XT, 4><<<gx, RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
     } else if (E <= 32) {
         route_logits_kernel<XT, 2, 4, 8><<<dim3(gx, 1), RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
     } else {

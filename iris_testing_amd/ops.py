@@ -111,8 +111,6 @@ def pack_fixed_m(x: torch.Tensor, row_token: torch.Tensor, dst_sizes: torch.Tens
     if out is None:
         out = torch.empty((W, M, H), dtype=x.dtype, device=x.device)
     assert out.shape == (W, M, H) and out.dtype == x.dtype and out.is_contiguous()
-    if map_ws is None:
-        map_ws = _i32((W * M,), x.device)
     L.check(L.lib().moe_pack(L.ptr(x), L.dtype_code(x.dtype), T, H, L.ptr(row_token), L.ptr(dst_sizes),
                              L.ptr(dst_offsets), W, M, L.ptr(out), L.ptr(map_ws), L.ptr(status), L.stream_ptr()))
     return out

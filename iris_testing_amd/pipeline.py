@@ -42,7 +42,6 @@ class DispatchPipeline:
         self.count_ws_bytes = lib.moe_count_workspace_bytes(T, k, E)
         self.count_ws = torch.empty(self.count_ws_bytes, dtype=torch.uint8, device=dev)
         self.send = torch.empty((W, M, H), dtype=dt, device=dev)
-        self.send_map = i32(W * M)
         self.status = torch.zeros(1, dtype=torch.int32, device=dev)
         # destination side
         self.rows = torch.empty((S, H), dtype=dt, device=dev)
@@ -79,7 +78,7 @@ class DispatchPipeline:
         c, w = self.cfg, self.world
         L.check(L.lib().moe_pack(self._p(w.x0), self.code, c.tokens, c.hidden, self._p(self.row_token),
                                  self._p(self.dst_sizes), self._p(self.dst_offsets), c.world, w.M, self._p(self.send),
-                                 self._p(self.send_map), self._p(self.status), s))
+                                 None, self._p(self.status), s))
 
     def unpack(self, s):
         c, w = self.cfg, self.world
