@@ -22,8 +22,8 @@ struct VecLoad;
 template <>
 struct VecLoad<bf16_t> {
     static constexpr int N = 8;
-    __device__ static void load(const bf16_t* p, float* out) {
-        uint4 v = *reinterpret_cast<const uint4*>(p);
+    __device__ static void load(const bf16_t* p, float* out) { unpack(*reinterpret_cast<const uint4*>(p), out); }
+    __device__ static void unpack(const uint4& v, float* out) {
         uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -35,9 +35,9 @@ struct VecLoad<bf16_t> {
 template <>
 struct VecLoad<float> {
     static constexpr int N = 4;
-    __device__ static void load(const float* p, float* out) {
-        float4 v = *reinterpret_cast<const float4*>(p);
-        out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+    __device__ static void load(const float* p, float* out) { unpack(*reinterpret_cast<const uint4*>(p), out); }
+    __device__ static void unpack(const uint4& v, float* out) {
+        out[0] = __uint_as_float(v.x); out[1] = __uint_as_float(v.y); out[2] = __uint_as_float(v.z); out[3] = __uint_as_float(v.w);
     }
 };
 
@@ -155,55 +155,88 @@ __global__ __launch_bounds__(RT_THREADS) void route_logits_small_kernel(const XT
 #pragma unroll
     for (int j = 0; j < EE; ++j) acc[j] = 0.f;
 
+    // raw slab data held in registers while the previous slab is consumed; masking and conversion
+    // happen when it is written to LDS, so nothing waits on these loads until then
     uint4 xr[XPT];
-    float wr[WPT];
+    XT wr[WPT];
     auto fetch = [&](int k0) {
 #pragma unroll
         for (int i = 0; i < XPT; ++i) {
             const int c = tid + i * RT_THREADS;
             const int row = c / (RS_KC / VN), col = (c % (RS_KC / VN)) * VN;
-            const int t = t0 + row;
-            xr[i] = (t < T && k0 + col < H) ? *reinterpret_cast<const uint4*>(x + (size_t)t * H + k0 + col) : make_uint4(0, 0, 0, 0);
+            // clamped (always valid) address: no divergent branch, all loads of a slab in flight together
+            xr[i] = *reinterpret_cast<const uint4*>(x + (size_t)min(t0 + row, T - 1) * H + min(k0 + col, H - VN));
         }
 #pragma unroll
         for (int i = 0; i < WPT; ++i) {
             const int c = tid + i * RT_THREADS;
-            const int kk = c / 16, e = c % 16;
-            wr[i] = (k0 + kk < H && e < E) ? load_f32<XT>(w + (size_t)(k0 + kk) * E + e) : 0.f;
+            wr[i] = w[(size_t)min(k0 + c / 16, H - 1) * E + min(c % 16, E - 1)];
         }
     };
-    auto stash = [&]() {
+    auto stash = [&](int k0) {
 #pragma unroll
         for (int i = 0; i < XPT; ++i) {
             const int c = tid + i * RT_THREADS;
             const int row = c / (RS_KC / VN), col = (c % (RS_KC / VN)) * VN;
-            *reinterpret_cast<uint4*>(&xs[row][col]) = xr[i];
+            const bool ok = t0 + row < T && k0 + col < H;
+            *reinterpret_cast<uint4*>(&xs[row][col]) =
+                make_uint4(ok ? xr[i].x : 0u, ok ? xr[i].y : 0u, ok ? xr[i].z : 0u, ok ? xr[i].w : 0u);
         }
 #pragma unroll
         for (int i = 0; i < WPT; ++i) {
             const int c = tid + i * RT_THREADS;
-            wsT[c % 16][c / 16] = wr[i];
+            const bool ok = k0 + c / 16 < H && c % 16 < E;
+            wsT[c % 16][c / 16] = ok ? load_f32<XT>(&wr[i]) : 0.f;
         }
     };
 
+    constexpr int UN = 4;  // 16-byte x chunks consumed per inner step
     fetch(0);
     for (int k0 = 0; k0 < H; k0 += RS_KC) {
-        stash();
+        stash(k0);
         __syncthreads();
         if (k0 + RS_KC < H) fetch(k0 + RS_KC);
         const int kmax = min(RS_KC, H - k0);
-        for (int kk = 0; kk < kmax; kk += VN) {
+        int kk = 0;
+        for (; kk + UN * VN <= kmax; kk += UN * VN) {
+            // all LDS reads of the step first, then the fmaf chains in ascending h
+            uint4 xraw[UN];
+            float4 wv[EE][UN * VN / 4];
+#pragma unroll
+            for (int u = 0; u < UN; ++u) xraw[u] = *reinterpret_cast<const uint4*>(&xs[lane][kk + u * VN]);
+#pragma unroll
+            for (int j = 0; j < EE; ++j)
+#pragma unroll
+                for (int q = 0; q < UN * VN / 4; ++q) wv[j][q] = *reinterpret_cast<const float4*>(&wsT[e0 + j][kk + 4 * q]);
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+                float xv[VN];
+                VecLoad<XT>::unpack(xraw[u], xv);
+#pragma unroll
+                for (int q = 0; q < VN; q += 4) {
+#pragma unroll
+                    for (int j = 0; j < EE; ++j) {
+                        const float4 wq = wv[j][(u * VN + q) / 4];
+                        acc[j] = fmaf(xv[q + 0], wq.x, acc[j]);
+                        acc[j] = fmaf(xv[q + 1], wq.y, acc[j]);
+                        acc[j] = fmaf(xv[q + 2], wq.z, acc[j]);
+                        acc[j] = fmaf(xv[q + 3], wq.w, acc[j]);
+                    }
+                }
+            }
+        }
+        for (; kk < kmax; kk += VN) {
             float xv[VN];
             VecLoad<XT>::load(&xs[lane][kk], xv);
 #pragma unroll
             for (int q = 0; q < VN; q += 4) {
 #pragma unroll
                 for (int j = 0; j < EE; ++j) {
-                    const float4 wv = *reinterpret_cast<const float4*>(&wsT[e0 + j][kk + q]);
-                    acc[j] = fmaf(xv[q + 0], wv.x, acc[j]);
-                    acc[j] = fmaf(xv[q + 1], wv.y, acc[j]);
-                    acc[j] = fmaf(xv[q + 2], wv.z, acc[j]);
-                    acc[j] = fmaf(xv[q + 3], wv.w, acc[j]);
+                    const float4 wq = *reinterpret_cast<const float4*>(&wsT[e0 + j][kk + q]);
+                    acc[j] = fmaf(xv[q + 0], wq.x, acc[j]);
+                    acc[j] = fmaf(xv[q + 1], wq.y, acc[j]);
+                    acc[j] = fmaf(xv[q + 2], wq.z, acc[j]);
+                    acc[j] = fmaf(xv[q + 3], wq.w, acc[j]);
                 }
             }
         }
