@@ -69,16 +69,31 @@ enum { EPI_NONE = 0, EPI_GELU = 1, EPI_SILU = 2, EPI_SWIGLU = 3 };
 
 // ---- pieces of the main loop ---------------------------------------------------------------------
 // HBM -> LDS, 16 bytes per lane, no register staging.  One instruction moves 8 tile rows (64 lanes x
-// 16 B); wave w of a round moves rows [w*8, w*8+8) of that round.
+// 16 B); wave w of a round moves rows [w*8, w*8+8) of that round.  Written as inline assembly to get the
+// scalar-base + 32-bit-lane-offset form (the builtin expands to a 64-bit per-lane address); M0 holds
+// the LDS byte address of the wave's 1 KB destination.
+__device__ __forceinline__ void gg_dma16(const uint8_t* sbase, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0" : : "s"(sbase), "v"(voff), "s"(lds_addr) : "memory");
+}
+
+// a wave-uniform value forced into scalar registers
+__device__ __forceinline__ const uint8_t* gg_uniform(const uint8_t* p) {
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const uint8_t*)(((uint64_t)hi << 32) | lo);
+}
+
 template <int RA, int RB, int LR>
 __device__ __forceinline__ void gg_issue(uint4* sA, uint4* sB, const uint8_t* ap, const uint8_t* bp,
                                          const uint32_t* a_off, uint32_t b_off0, uint32_t b_step, int wave) {
+    ap = gg_uniform(ap);
+    bp = gg_uniform(bp);
+    const uint32_t la = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(sA + wave * 8 * CHUNKS));
+    const uint32_t lb = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(sB + wave * 8 * CHUNKS));
 #pragma unroll
-    for (int r = 0; r < RA; ++r)
-        __builtin_amdgcn_global_load_lds(ap + a_off[r], (lds_ptr_t)(sA + (r * LR + wave * 8) * CHUNKS), 16, 0, 0);
+    for (int r = 0; r < RA; ++r) gg_dma16(ap, a_off[r], la + r * LR * CHUNKS * 16);
 #pragma unroll
-    for (int r = 0; r < RB; ++r)
-        __builtin_amdgcn_global_load_lds(bp + b_off0 + r * b_step, (lds_ptr_t)(sB + (r * LR + wave * 8) * CHUNKS), 16, 0, 0);
+    for (int r = 0; r < RB; ++r) gg_dma16(bp + (size_t)r * b_step, b_off0, lb + r * LR * CHUNKS * 16);
 }
 
 template <int TM, int TN>
@@ -209,6 +224,8 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 
         uint4 a0[TM], b0[TN], a1[TM], b1[TN];
         constexpr int NMMA = TM * TN * (FP8 ? 2 : 1);  // MFMA instructions per fragment step
+        constexpr int LPS = RA + RB;                   // HBM->LDS loads per lane per stage
+        static_assert(LPS == 8 || LPS == 12, "load interleave is written for 8 or 12 loads per stage");
         const int pos0 = (0 + khalf) ^ fswz, pos1 = (2 + khalf) ^ fswz, pos2 = (4 + khalf) ^ fswz, pos3 = (6 + khalf) ^ fswz;
         static_assert(NKK == 4, "GG_STAGE is written for four fragment steps");
 
@@ -224,6 +241,23 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         __builtin_amdgcn_sched_group_barrier(0x008, NMMA - 1, 0);           \
         __builtin_amdgcn_sched_barrier(0);                                  \
     } while (0)
+        static_assert(TM * TN == 8, "GG_MD is unrolled for eight MFMA tiles per wave");
+        /* I-th MFMA of the block, then its share of the stage's loads (constant indices only) */
+#define GG_LD(d)                                                                                         \
+    do {                                                                                                 \
+        if constexpr ((d) < RA) gg_dma16(ap_, a_off[(d) < RA ? (d) : 0], la_ + (d) * LR * CHUNKS * 16);     \
+        else if constexpr ((d) < LPS) gg_dma16(bp_ + (size_t)((d) - RA) * b_step, b_off0, lb_ + ((d) - RA) * LR * CHUNKS * 16); \
+    } while (0)
+#define GG_MD(I)                                                                                         \
+    do {                                                                                                 \
+        mma<FP8>(acc[(I) / TN][(I) % TN], b1[(I) % TN], a1[(I) / TN]);                                   \
+        __builtin_amdgcn_sched_barrier(0);                                                               \
+        if (more_) {                                                                                     \
+            if constexpr (LPS == 8) { GG_LD(I); }                                                        \
+            else { GG_LD(((I) * 3) / 2); if constexpr ((I) % 2 == 1) GG_LD(((I) * 3) / 2 + 1); }         \
+        }                                                                                                \
+        __builtin_amdgcn_sched_barrier(0);                                                               \
+    } while (0)
 #define GG_STAGE(fa, fb, na, nb, curA, curB, ks)                           \
     do {                                                                   \
         gg_frags<TM, TN>(fa, fb, pos1, a1, b1);                            \
@@ -238,11 +272,19 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         if ((ks) + 1 < nk) {                                               \
             gg_wait<0, 0>();                                               \
             __syncthreads();                                               \
-            if ((ks) + 2 < nk) GG_ISSUE(curA, curB, (ks) + 2);             \
             gg_frags<TM, TN>(na, nb, pos0, a0, b0);                        \
+            __builtin_amdgcn_sched_barrier(0);                             \
         }                                                                  \
-        __builtin_amdgcn_sched_barrier(0);                                 \
-        gg_mmas<TM, TN, FP8>(acc, a1, b1);                                 \
+        {                                                                  \
+            /* last MFMA block of the stage with the refill loads spread between its MFMAs: each load  \
+               is issued in the shadow of the MFMA before it, so the matrix pipe does not drain */     \
+            const bool more_ = (ks) + 2 < nk;                                                            \
+            const uint8_t* ap_ = gg_uniform(Ab + (size_t)((ks) + 2) * ROWB);                             \
+            const uint8_t* bp_ = gg_uniform(Bb + (size_t)((ks) + 2) * b_slab);                           \
+            const uint32_t la_ = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)((curA) + wave * 8 * CHUNKS)); \
+            const uint32_t lb_ = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)((curB) + wave * 8 * CHUNKS)); \
+            GG_MD(0); GG_MD(1); GG_MD(2); GG_MD(3); GG_MD(4); GG_MD(5); GG_MD(6); GG_MD(7);              \
+        }                                                                  \
         __builtin_amdgcn_sched_barrier(0);                                 \
     } while (0)
 
@@ -261,6 +303,8 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             if (ks + 1 < nk) GG_STAGE(fa1, fb1, fa0, fb0, sA1, sB1, ks + 1);
         }
 #undef GG_STAGE
+#undef GG_MD
+#undef GG_LD
 #undef GG_ORDER
 #undef GG_ISSUE
 
