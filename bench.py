@@ -131,10 +131,19 @@ def main():
             unit = "TFLOP/s"
         stages[n] = {"ms": round(ms, 4), "bound": wk["bound"], "achieved": round(ach, 2), "peak": peak, "unit": unit,
                      "frac": round(ach / peak, 4)}
+    # HBM traffic per launch of the dominant kernel, from the FETCH_SIZE / WRITE_SIZE runs summarised in
+    # profiles/mixtral_hbm_traffic.txt (bytes; only measured for the default workload)
+    measured_traffic = {"mixtral": 12.44e9}
     dom = "mlp_up"  # the gate/up grouped GEMM: most of the flops of a step
-    roofline = {"kernel": "grouped_gemm_kernel (gate/up + SwiGLU epilogue)" if cfg.act == "swiglu" else "grouped_gemm_kernel (up)",
+    if cfg.quant == "fp8":
+        kname = "moe_grouped_mlp_fp8 (row quantisation + gate/up GEMM + SwiGLU + re-quantisation + down GEMM)"
+    elif cfg.dtype == "f32":
+        kname = "moe_grouped_mlp fp32 (both GEMMs)"
+    else:
+        kname = "grouped_gemm_kernel (gate/up + SwiGLU epilogue)" if cfg.act == "swiglu" else "grouped_gemm_kernel (up + activation)"
+    roofline = {"kernel": kname,
                 "bound": "mfma", "achieved": stages[dom]["achieved"], "peak": stages[dom]["peak"], "unit": "TFLOP/s",
-                "frac": stages[dom]["frac"], "traffic": None, "avg_launch_ms": stages[dom]["ms"],
+                "frac": stages[dom]["frac"], "traffic": measured_traffic.get(cfg.name), "avg_launch_ms": stages[dom]["ms"],
                 "flops_per_launch": work[dom]["amount"]}
 
     out = {

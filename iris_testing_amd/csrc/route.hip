@@ -68,52 +68,75 @@ __global__ __launch_bounds__(RT_THREADS) void route_logits_kernel(const XT* __re
     constexpr int VN = VecLoad<XT>::N;
     constexpr int CH_PER_TOK = RT_KC / VN;
     constexpr int X_CHUNKS = TB * CH_PER_TOK;
+    constexpr int XPT = (X_CHUNKS + RT_THREADS - 1) / RT_THREADS;
+    constexpr int WPT = RT_KC * EB / RT_THREADS;
+    static_assert(X_CHUNKS % RT_THREADS == 0 && (RT_KC * EB) % RT_THREADS == 0, "staging split");
 
-    for (int k0 = 0; k0 < H; k0 += RT_KC) {
-        const int kmax = min(RT_KC, H - k0);
-        // stage x tile [TB tokens][KC] -> xs[k][token] as fp32
-        for (int c = tid; c < X_CHUNKS; c += RT_THREADS) {
+    // The next slab is fetched into registers (from clamped, always valid addresses) while the current one
+    // is consumed; masking and conversion to fp32 happen when it is written to LDS.
+    uint4 xr[XPT];
+    XT wr[WPT];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < XPT; ++i) {
+            const int c = tid + i * RT_THREADS;
             const int tt = c / CH_PER_TOK, kc = (c % CH_PER_TOK) * VN;
-            const int t = t0 + tt;
+            xr[i] = *reinterpret_cast<const uint4*>(x + (size_t)min(t0 + tt, T - 1) * H + min(k0 + kc, H - VN));
+        }
+#pragma unroll
+        for (int i = 0; i < WPT; ++i) {
+            const int c = tid + i * RT_THREADS;
+            wr[i] = w[(size_t)min(k0 + c / EB, H - 1) * E + min(e0 + c % EB, E - 1)];
+        }
+    };
+    auto stash = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < XPT; ++i) {
+            const int c = tid + i * RT_THREADS;
+            const int tt = c / CH_PER_TOK, kc = (c % CH_PER_TOK) * VN;
+            const bool ok = t0 + tt < T && k0 + kc < H;
             float v[VN];
-            if (t < T && k0 + kc + VN <= H) {
-                VecLoad<XT>::load(x + (size_t)t * H + k0 + kc, v);
-            } else {
+            VecLoad<XT>::unpack(xr[i], v);
 #pragma unroll
-                for (int j = 0; j < VN; ++j)
-                    v[j] = (t < T && k0 + kc + j < H) ? load_f32<XT>(x + (size_t)t * H + k0 + kc + j) : 0.0f;
-            }
+            for (int j = 0; j < VN; ++j) xs[kc + j][tt] = ok ? v[j] : 0.0f;
+        }
 #pragma unroll
-            for (int j = 0; j < VN; ++j) xs[kc + j][tt] = v[j];
+        for (int i = 0; i < WPT; ++i) {
+            const int c = tid + i * RT_THREADS;
+            const bool ok = k0 + c / EB < H && e0 + c % EB < E;
+            ws[c / EB][c % EB] = ok ? load_f32<XT>(&wr[i]) : 0.0f;
         }
-        // stage router tile [KC][EB]
-        for (int c = tid; c < RT_KC * EB; c += RT_THREADS) {
-            const int kk = c / EB, ee = c % EB;
-            const int e = e0 + ee;
-            ws[kk][ee] = (kk < kmax && e < E) ? load_f32<XT>(w + (size_t)(k0 + kk) * E + e) : 0.0f;
-        }
+    };
+
+    constexpr int UK = 8;  // h per inner step: all LDS reads of the step are issued before its fmaf chains
+    fetch(0);
+    for (int k0 = 0; k0 < H; k0 += RT_KC) {
+        stash(k0);
         __syncthreads();
-        if (kmax == RT_KC) {
-#pragma unroll 8
-            for (int kk = 0; kk < RT_KC; ++kk) {
-                float xv[TT], wv[EE];
+        if (k0 + RT_KC < H) fetch(k0 + RT_KC);
+        const int kmax = min(RT_KC, H - k0);
+        int kk = 0;
+        for (; kk + UK <= kmax; kk += UK) {
+            float xv[UK][TT], wv[UK][EE];
 #pragma unroll
-                for (int i = 0; i < TT; ++i) xv[i] = xs[kk][ty * TT + i];
+            for (int u = 0; u < UK; ++u) {
 #pragma unroll
-                for (int j = 0; j < EE; ++j) wv[j] = ws[kk][tx * EE + j];
+                for (int i = 0; i < TT; ++i) xv[u][i] = xs[kk + u][ty * TT + i];
+#pragma unroll
+                for (int j = 0; j < EE; ++j) wv[u][j] = ws[kk + u][tx * EE + j];
+            }
+#pragma unroll
+            for (int u = 0; u < UK; ++u)
 #pragma unroll
                 for (int i = 0; i < TT; ++i)
 #pragma unroll
-                    for (int j = 0; j < EE; ++j) acc[i][j] = fmaf(xv[i], wv[j], acc[i][j]);
-            }
-        } else {
-            for (int kk = 0; kk < kmax; ++kk) {
+                    for (int j = 0; j < EE; ++j) acc[i][j] = fmaf(xv[u][i], wv[u][j], acc[i][j]);
+        }
+        for (; kk < kmax; ++kk) {
 #pragma unroll
-                for (int i = 0; i < TT; ++i)
+            for (int i = 0; i < TT; ++i)
 #pragma unroll
-                    for (int j = 0; j < EE; ++j)
-                        acc[i][j] = fmaf(xs[kk][ty * TT + i], ws[kk][tx * EE + j], acc[i][j]);
-            }
+                for (int j = 0; j < EE; ++j) acc[i][j] = fmaf(xs[kk][ty * TT + i], ws[kk][tx * EE + j], acc[i][j]);
         }
         __syncthreads();
     }

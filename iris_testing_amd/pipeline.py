@@ -144,12 +144,17 @@ class DispatchPipeline:
         B = 4 if c.dtype == "f32" else 2
         S, M = self.S, w.M
         up_mats = 2 if c.act == "swiglu" else 1
+        if self.weights.dtype != torch.bfloat16:
+            # fp8 and fp32 run both GEMMs (and the fp8 quantisation passes) inside one entry point
+            mlp = {"mlp_up": dict(bound="mfma", amount=2 * S * H * F * (up_mats + 1))}
+        else:
+            mlp = {"mlp_up": dict(bound="mfma", amount=2 * S * H * F * up_mats),
+                   "mlp_down": dict(bound="mfma", amount=2 * S * F * H)}
         return {
             "route": dict(bound="hbm", amount=T * H * B + H * E * B + T * k * 8),
             "pack": dict(bound="hbm", amount=T * H * B + W * M * H * B),
             "unpack": dict(bound="hbm", amount=2 * S * H * B),
-            "mlp_up": dict(bound="mfma", amount=2 * S * H * F * up_mats),
-            "mlp_down": dict(bound="mfma", amount=2 * S * F * H),
+            **mlp,
             "return_pack": dict(bound="hbm", amount=S * H * B + W * M * H * B),
             "combine": dict(bound="hbm", amount=T * k * H * B + T * H * B + T * k * 8),
         }
