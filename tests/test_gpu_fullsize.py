@@ -1,0 +1,87 @@
+"""The three large workloads at their full BASELINE sizes, through the pipeline the benchmark times.
+What the oracle can finish in seconds is compared directly (shard-0 routing, counts, the packed send
+buffer, sampled expert rows); the rest is pinned by size-independent properties: the return pack is the
+exact inverse of the unpack, every received row appears exactly once, combine is linear under exact
+scalings, sum-of-rows checksums agree."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import O, assert_bits_equal, err_stats, to_np
+
+pytestmark = pytest.mark.gpu
+
+from iris_testing_amd import harness, ops  # noqa: E402
+from iris_testing_amd.configs import CONFIGS  # noqa: E402
+from iris_testing_amd.pipeline import DispatchPipeline  # noqa: E402
+
+DEV = "cuda"
+
+
+@pytest.mark.parametrize("name", ["mixtral", "finegrained", "zipf_k4"])
+def test_full_size_pipeline(name):
+    cfg = CONFIGS[name]
+    print(f"case {cfg}", flush=True)
+    world = harness.build_world(cfg, DEV)
+    ew, raw, qs = harness.expert_weights(cfg, 0, DEV)
+    pipe = DispatchPipeline(world, ew)
+    pipe.step()
+    torch.cuda.synchronize()
+    assert int(pipe.status.item()) == 0
+    W, M, H, E_l, S = cfg.world, world.M, cfg.hidden, cfg.e_local, world.S
+
+    # ---- source side of rank 0 against the oracle (bit-exact)
+    x0, router = to_np(world.x0), to_np(world.router)
+    bias = None if world.bias is None else to_np(world.bias)
+    idx, gate, _ = O.route(x0, router, cfg.topk, bias)
+    assert_bits_equal(pipe.idx, idx, "top-k indices")
+    counts = O.send_counts(idx, W, cfg.experts)
+    sizes, offs = O.dst_sizes_offsets(counts)
+    pos, row_token = O.payload_positions(idx, cfg.experts)
+    assert_bits_equal(pipe.send_counts, counts, "send_counts")
+    assert_bits_equal(pipe.pos, pos, "pos")
+    assert M >= O.pair_capacity(sizes) and world.CAP >= O.compute_capacity_from_pca(counts)
+    assert_bits_equal(pipe.send, O.pack_fixed_m(O.send_payload(x0, row_token), offs, sizes, M), "send [W,M,H]")
+
+    # ---- destination side: properties of the unpack / return pair on the assembled receive buffer
+    rc = to_np(world.recv_counts)
+    assert S == int(rc.sum())
+    assert_bits_equal(pipe.expert_cnt, rc.sum(axis=0).astype(np.int32), "expert_cnt")
+    back = ops.return_pack(pipe.rows, world.recv_counts, M)
+    assert torch.equal(back, world.recv), "return_pack(unpack(recv)) != recv"
+    # checksum of checksums: every valid row exactly once (row sums in fp64, order-free)
+    valid = torch.arange(M, device=DEV)[None, :] < world.recv_counts.sum(1)[:, None]
+    s_recv = world.recv.double().sum(-1)[valid].sum().item()
+    s_rows = pipe.rows.double().sum().item()
+    assert abs(s_recv - s_rows) <= 1e-6 * max(1.0, abs(s_recv))
+    assert (world.recv.double().abs().sum(-1)[~valid] == 0).all(), "padding rows must be zero"
+
+    # ---- expert MLP on a row sample against the oracle
+    rng = np.random.default_rng(cfg.seed)
+    cnt = rc.sum(axis=0)
+    starts = np.concatenate([[0], np.cumsum(cnt)])
+    sample = np.unique(np.concatenate([rng.integers(0, S, 48), starts[:-1][cnt > 0], (starts[1:] - 1)[cnt > 0]]))
+    expert_of = np.searchsorted(starts, sample, side="right") - 1
+    rows_np = to_np(pipe.rows[torch.from_numpy(sample).to(DEV)])
+    got = to_np(pipe.y[torch.from_numpy(sample).to(DEV)])
+    want = np.zeros_like(got)
+    for e in np.unique(expert_of):
+        sel = expert_of == e
+        one = np.array([int(sel.sum())], np.int32)
+        if cfg.quant == "fp8":
+            (gq, gs), (uq, us), (dq, ds) = [(to_np(q[e:e + 1]), to_np(s_[e:e + 1])) for q, s_ in qs]
+            want[sel] = O.expert_mlp_fp8(rows_np[sel], one, gq, gs, uq, us, dq, ds)
+        else:
+            wg, wu, wd = (to_np(w[e:e + 1]) for w in raw)
+            want[sel] = O.expert_mlp(rows_np[sel], one, wg, wd, "swiglu", cfg.dtype, w_up=wu)
+    mx, mx_rms, rel = err_stats(got, want.astype(np.float64))
+    print(f"{name}: expert MLP on {len(sample)} sampled rows: max-abs {mx:.3e}, max-abs/rms {mx_rms:.3e}, max-rel {rel:.3e}",
+          flush=True)
+    assert mx_rms < (2.0 ** -3 if cfg.quant == "fp8" else 2.0 ** -5)
+
+    # ---- combine: linear under exact scalings, and equal to the oracle on the tokens of one block
+    out1 = ops.combine(pipe.returned, pipe.idx, pipe.pos, pipe.gate, pipe.dst_offsets, E_l)
+    out2 = ops.combine((pipe.returned * 2).contiguous(), pipe.idx, pipe.pos, pipe.gate, pipe.dst_offsets, E_l)
+    assert torch.equal((out1 * 2), out2), "combine(2 r) != 2 combine(r)"
+    o_out = O.combine(to_np(pipe.returned), idx[:256], pos[:256], to_np(pipe.gate)[:256], offs, E_l, cfg.dtype)
+    assert_bits_equal(out1[:256], o_out, "combine (first 256 tokens)")
