@@ -67,6 +67,50 @@ __device__ __forceinline__ int seg_of(const int* off, int n, int r) {
 
 enum { EPI_NONE = 0, EPI_GELU = 1, EPI_SILU = 2, EPI_SWIGLU = 3 };
 
+// One output tile of the walk: group g, n tile nt, first row row0, rv valid rows (rv <= 0: none).
+struct GgTile {
+    int g, nt, row0, rv;
+};
+
+// lin -> tile: group-major, 16-row bands, 16-column super-columns (see the XCD-aware walk above)
+template <int BM>
+__device__ __forceinline__ GgTile gg_decode(const int* g_tile_start, const int* g_row_start, int E_l, int Nt, int S_rows, int lin) {
+    const int g = seg_of(g_tile_start, E_l + 1, lin);
+    const int cnt_g = g_row_start[g + 1] - g_row_start[g];
+    const int Mt = (cnt_g + BM - 1) / BM;
+    const int idx = lin - g_tile_start[g];
+    const int band = idx / (SUP * Nt), rem = idx % (SUP * Nt);
+    const int hr = min(SUP, Mt - band * SUP);
+    const int sc = rem / (hr * SUP), rem2 = rem % (hr * SUP);
+    const int wc = min(SUP, Nt - sc * SUP);
+    const int mt = band * SUP + rem2 / wc;
+    GgTile t;
+    t.g = g;
+    t.nt = sc * SUP + rem2 % wc;
+    t.row0 = g_row_start[g] + mt * BM;
+    t.rv = min(min(BM, cnt_g - mt * BM), S_rows - t.row0);
+    return t;
+}
+
+// next non-empty tile of this workgroup at or after round `base` (base is advanced past it)
+template <int BM>
+__device__ __forceinline__ GgTile gg_next_tile(const int* g_tile_start, const int* g_row_start, int E_l, int Nt, int S_rows,
+                                               int total, int my, int stride, int& base) {
+    GgTile t;
+    t.g = t.nt = t.row0 = 0;
+    t.rv = 0;
+    while (base < total) {
+        const int lin = base + my;
+        base += stride;
+        if (lin < total) {
+            t = gg_decode<BM>(g_tile_start, g_row_start, E_l, Nt, S_rows, lin);
+            if (t.rv > 0) break;
+        }
+    }
+    return t;
+}
+
+
 // ---- pieces of the main loop ---------------------------------------------------------------------
 // HBM -> LDS, 16 bytes per lane, no register staging.  One instruction moves 8 tile rows (64 lanes x
 // 16 B); wave w of a round moves rows [w*8, w*8+8) of that round.  Written as inline assembly to get the
@@ -185,34 +229,36 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     const uint4* fb0 = sB0 + (wn * (BN / 2) + (lane & 31)) * CHUNKS;
     const uint4* fb1 = sB1 + (wn * (BN / 2) + (lane & 31)) * CHUNKS;
 
-    for (int base = 0; base < total; base += gridDim.x) {
-        const int lin = base + my;
-        if (lin >= total) continue;  // uniform over the workgroup
-        // ---- decode lin -> (group, m tile, n tile): group-major, 16-row bands, 16-col super-columns
-        const int g = seg_of(g_tile_start, p.E_l + 1, lin);
-        const int cnt_g = g_row_start[g + 1] - g_row_start[g];
-        const int Mt = (cnt_g + BM - 1) / BM;
-        const int idx = lin - g_tile_start[g];
-        const int band = idx / (SUP * Nt), rem = idx % (SUP * Nt);
-        const int hr = min(SUP, Mt - band * SUP);
-        const int sc = rem / (hr * SUP), rem2 = rem % (hr * SUP);
-        const int wc = min(SUP, Nt - sc * SUP);
-        const int mt = band * SUP + rem2 / wc, nt = sc * SUP + rem2 % wc;
+    // Tiles are software-pipelined: the first two K stages of the next tile are requested before the
+    // epilogue of the current one, so the stores of one tile overlap the first loads of the next.
+    const uint32_t ldk = (uint32_t)(p.K * ES);
+    const size_t b_slab = (size_t)p.Npad * ROWB;  // packed weights are slab-major: [group][K slab][Npad rows][ROWB bytes]
+    const uint32_t b_off0 = (uint32_t)lrow * ROWB + lchunk * 16;
+    const uint32_t b_step = (uint32_t)LR * ROWB;
+#define GG_TILE_PTRS(t, Ab_, Bb_, aoff_)                                                                   \
+    const uint8_t* Ab_ = p.A + (size_t)(t).row0 * p.K * ES;                                                 \
+    const uint8_t* Bb_ = p.B + (size_t)(t).g * p.Npad * p.K * ES + (size_t)(t).nt * BN * ROWB;               \
+    uint32_t aoff_[RA];                                                                                     \
+    _Pragma("unroll") for (int r = 0; r < RA; ++r) aoff_[r] = (uint32_t)min(r * LR + lrow, (t).rv - 1) * ldk + lchunk * 16;
+#define GG_ISSUE_T(sA, sB, Ab_, Bb_, aoff_, ks) \
+    gg_issue<RA, RB, LR>(sA, sB, Ab_ + (size_t)(ks) * ROWB, Bb_ + (size_t)(ks) * b_slab, aoff_, b_off0, b_step, wave)
 
-        const int row0 = g_row_start[g] + mt * BM;
-        const int rv = min(min(BM, cnt_g - mt * BM), p.S_rows - row0);  // valid rows of this tile
-        if (rv <= 0) continue;
-
-        const uint8_t* Ab = p.A + (size_t)row0 * p.K * ES;
-        // packed weights are slab-major: [group][K slab of ROWB bytes][Npad rows][ROWB bytes]
-        const uint8_t* Bb = p.B + (size_t)g * p.Npad * p.K * ES + (size_t)nt * BN * ROWB;
-        const size_t b_slab = (size_t)p.Npad * ROWB;
-        const uint32_t ldk = (uint32_t)(p.K * ES);
-        uint32_t a_off[RA];
+    int base = 0;
+    GgTile cur = gg_next_tile<BM>(g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, total, my, gridDim.x, base);
+    uint32_t a_off[RA];
+    const uint8_t *Ab = p.A, *Bb = p.B;
+    if (cur.rv > 0) {
+        GG_TILE_PTRS(cur, Ab0, Bb0, a_off0);
+        Ab = Ab0;
+        Bb = Bb0;
 #pragma unroll
-        for (int r = 0; r < RA; ++r) a_off[r] = (uint32_t)min(r * LR + lrow, rv - 1) * ldk + lchunk * 16;
-        const uint32_t b_off0 = (uint32_t)lrow * ROWB + lchunk * 16;
-        const uint32_t b_step = (uint32_t)LR * ROWB;
+        for (int r = 0; r < RA; ++r) a_off[r] = a_off0[r];
+        GG_ISSUE_T(sA0, sB0, Ab, Bb, a_off, 0);
+        if (nk > 1) GG_ISSUE_T(sA1, sB1, Ab, Bb, a_off, 1);
+    }
+    while (cur.rv > 0) {
+        const int g = __builtin_amdgcn_readfirstlane(cur.g), nt = __builtin_amdgcn_readfirstlane(cur.nt);
+        const int row0 = __builtin_amdgcn_readfirstlane(cur.row0), rv = __builtin_amdgcn_readfirstlane(cur.rv);
 
         floatx16 acc[TM][TN];
 #pragma unroll
@@ -288,14 +334,9 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         __builtin_amdgcn_sched_barrier(0);                                 \
     } while (0)
 
-        __syncthreads();  // every wave is done with LDS of the previous tile
-        GG_ISSUE(sA0, sB0, 0);
-        if (nk > 1) {
-            GG_ISSUE(sA1, sB1, 1);
-            gg_wait_vm<RA + RB>();
-        } else {
-            gg_wait_vm<0>();
-        }
+        // stages 0 and 1 of this tile were requested before the previous tile's epilogue (or above, for the
+        // first tile); the epilogue's stores sit behind them in the same counter, so wait for everything
+        gg_wait_vm<0>();
         __syncthreads();
         gg_frags<TM, TN>(fa0, fb0, pos0, a0, b0);
         for (int ks = 0; ks < nk; ks += 2) {
@@ -307,6 +348,16 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 #undef GG_LD
 #undef GG_ORDER
 #undef GG_ISSUE
+
+        // ---- next tile: decode it and request its first two stages now (both LDS buffers are free once
+        // every wave has passed the barrier: the last fragments of this tile are already in registers)
+        const GgTile nxt = gg_next_tile<BM>(g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, total, my, gridDim.x, base);
+        GG_TILE_PTRS(nxt, Ab_n, Bb_n, a_off_n);
+        if (nxt.rv > 0) {
+            __syncthreads();
+            GG_ISSUE_T(sA0, sB0, Ab_n, Bb_n, a_off_n, 0);
+            if (nk > 1) GG_ISSUE_T(sA1, sB1, Ab_n, Bb_n, a_off_n, 1);
+        }
 
         // ---- epilogue: acc -> (scales) -> activation -> bf16 -> C
         bf16_t* C = (bf16_t*)p.C;
@@ -370,7 +421,14 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                 }
             }
         }
+        cur = nxt;
+        Ab = Ab_n;
+        Bb = Bb_n;
+#pragma unroll
+        for (int r = 0; r < RA; ++r) a_off[r] = a_off_n[r];
     }
+#undef GG_TILE_PTRS
+#undef GG_ISSUE_T
 }
 
 // ---- one-time weight re-tiling: w [E_l,K,N] (N contiguous) -> out [E_l][K/SK][Npad][SK], SK = one LDS
