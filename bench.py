@@ -67,6 +67,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="mixtral")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay timing")
     ap.add_argument("--cpu-sample-tokens", type=int, default=0, help="0 = sized for roughly 10-30 s")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -116,6 +117,27 @@ def main():
     ms_total = t_start.elapsed_time(t_end)
     ms_per_step = ms_total / args.steps
 
+    # the same K steps replayed as one HIP graph per step (launch overhead removed); the headline value is
+    # the faster of the two ways of launching, and says which
+    launch = "stream"
+    if not args.no_graph:
+        graph = pipe.capture()
+        for _ in range(args.warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        g0.record()
+        for _ in range(args.steps):
+            graph.replay()
+        g1.record()
+        torch.cuda.synchronize()
+        ms_graph = g0.elapsed_time(g1) / args.steps
+        stream_ms_per_step = ms_per_step
+        if ms_graph < ms_per_step:
+            ms_per_step, launch = ms_graph, "hipGraph"
+    else:
+        ms_graph, stream_ms_per_step = None, ms_per_step
+
     stage_ms = {n: sum(e[n][0].elapsed_time(e[n][1]) for e in events) / len(events) for n in STAGES}
     work = pipe.work()
     stages = {}
@@ -160,6 +182,9 @@ def main():
                    "rows_received": world.S},
         "routed_rows_per_s": round(cfg.tokens * cfg.topk / (ms_per_step * 1e-3), 1),
         "host_wall_ms_per_step": round(wall * 1e3 / args.steps, 4),
+        "launch": launch,
+        "ms_per_step_stream": round(stream_ms_per_step, 4),
+        "ms_per_step_graph": None if ms_graph is None else round(ms_graph, 4),
         "roofline": roofline,
         "stages": stages,
     }

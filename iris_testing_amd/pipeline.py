@@ -137,6 +137,17 @@ class DispatchPipeline:
         if events is not None:
             events.append(rec)
 
+    def capture(self):
+        """The whole step as one HIP graph (every stage only enqueues kernels: no allocation, no memset,
+        no synchronisation, so the capture is a plain kernel chain).  Returns a torch.cuda.CUDAGraph whose
+        replay() runs one step on the capturing stream's successor."""
+        self.step()  # warm every kernel before capture
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self.step()
+        return g
+
     # ---- algorithmic work per stage (bytes for the HBM-bound ones, flops for the GEMMs) ---------
     def work(self) -> Dict[str, dict]:
         c, w = self.cfg, self.world

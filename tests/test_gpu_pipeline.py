@@ -57,3 +57,30 @@ def test_dispatch_expert_combine_matches_dense(name):
     print(f"{name}: end-to-end max-abs {mx:.3e}, max-abs/rms {mx_rms:.3e}, max-rel {rel:.3e}", flush=True)
     tol = 2.0 ** -6 if cfg.dtype == "bf16" else 1e-4
     assert mx_rms < tol * 4, f"end-to-end error {mx_rms} of rms"
+
+
+@pytest.mark.parametrize("name", ["small", "zipf_k1"])
+def test_graph_replay_equals_eager(name):
+    """The whole step captured as one HIP graph: every replay (with eager work and synchronisation in
+    between, and outputs cleared before each replay) must reproduce the eager step bit for bit."""
+    from iris_testing_amd.pipeline import DispatchPipeline
+    cfg = CONFIGS[name]
+    world = harness.build_world(cfg, DEV)
+    ew, _, _ = harness.expert_weights(cfg, 0, DEV)
+    pipe = DispatchPipeline(world, ew)
+    pipe.returned.copy_(torch.randn(pipe.returned.shape, device=DEV).to(pipe.returned.dtype))
+    pipe.step()
+    torch.cuda.synchronize()
+    names = ["idx", "gate", "send_counts", "pos", "send", "rows", "y", "ret", "out"]
+    eager = {n: getattr(pipe, n).clone() for n in names}
+    graph = pipe.capture()
+    for rep in range(3):
+        for n in names:
+            getattr(pipe, n).zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for n in names:
+            assert torch.equal(getattr(pipe, n), eager[n]), f"replay {rep}: {n} differs from the eager step"
+        pipe.step()  # eager work between replays
+        torch.cuda.synchronize()
