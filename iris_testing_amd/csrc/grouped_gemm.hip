@@ -4,10 +4,13 @@
 // Replaces the reference's intended expert layer (layers/expert.py:31-60) and grouped_gemm kernel
 // (kernels.py:240-289): out[rows of group g] = tokens[rows of g] @ weights[g], fp32 accumulate,
 // persistent grid walking a tile list that spans all groups.  Differences in kind, not a port:
-//   * tiles are 256(or 128) x 256 x 128 bytes of K, four wave64s each owning a 128(64) x 128 block of
-//     32x32x16 MFMAs;
-//   * operands go HBM -> LDS directly (global_load_lds, 16 bytes per lane), double buffered, with
-//     an XOR swizzle of the 16-byte chunks so that MFMA fragment reads are bank-conflict free;
+//   * tiles are 256 (or 128) x 256, four wave64s each owning a 128 (64) x 128 block of 32x32x16 MFMAs
+//     with the accumulators in the accumulation registers;
+//   * operands go HBM -> LDS directly (global_load_lds, 16 bytes per lane) through a ring of four
+//     64-byte K stages, the loads of a stage spread over two MFMA blocks and issued two stages ahead;
+//     an XOR swizzle of the 16-byte chunks keeps MFMA fragment reads bank-conflict free;
+//   * fragment reads are interleaved one by one between the MFMAs of the previous K step, and the
+//     products of a step are taken in the order in which their operands arrive;
 //   * weights are re-tiled once into a K-contiguous layout (gate/up interleaved for SwiGLU) so both
 //     MFMA operands are read as 128-bit fragments;
 //   * ragged group tails are masked (the reference assumes full tiles, kernels.py:270,282);
@@ -21,11 +24,16 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int ROWB = 128;  // bytes of K per tile row per stage
+constexpr int ROWB = 64;   // bytes of K per tile row per LDS ring stage
 constexpr int CHUNKS = ROWB / 16;
+constexpr int NRING = 4;   // LDS ring stages
+constexpr int WROWS = 64 / CHUNKS;  // tile rows moved by one wave-wide 16-byte-per-lane load
 constexpr int SUP = 16;  // super-tile edge, in tiles
 constexpr int GG_MAXG = MOE_MAX_EXPERTS;
 constexpr int GG_BN = 256;
+#ifndef GG_BIG_NWM
+#define GG_BIG_NWM 2  // waves along M of the 256-row tile (x 2 along N)
+#endif
 
 struct GemmParams {
     const uint8_t* A;         // [S_rows, K] activations (bf16 or fp8)
@@ -38,6 +46,16 @@ struct GemmParams {
     int E_l, K, N, Npad, ldc, S_rows, ncs;
 };
 
+// x * sigmoid(x) with the hardware reciprocal (1 ulp) instead of an IEEE division: the SwiGLU epilogue of a
+// 128 x 128 wave tile evaluates this 8192 times per lane-row, and the division was most of its cost
+// two fp32 -> packed bf16 (round to nearest even) in one hardware conversion
+typedef __bf16 gg_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float gg_f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t gg_pack_bf16(float lo, float hi) {
+    const gg_f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, gg_bf16x2));
+}
+__device__ __forceinline__ float act_silu_fast(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 __device__ __forceinline__ float act_silu(float x) { return x / (1.0f + __expf(-x)); }
 __device__ __forceinline__ float act_gelu(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }
 
@@ -112,10 +130,10 @@ __device__ __forceinline__ GgTile gg_next_tile(const int* g_tile_start, const in
 
 
 // ---- pieces of the main loop ---------------------------------------------------------------------
-// HBM -> LDS, 16 bytes per lane, no register staging.  One instruction moves 8 tile rows (64 lanes x
-// 16 B); wave w of a round moves rows [w*8, w*8+8) of that round.  Written as inline assembly to get the
-// scalar-base + 32-bit-lane-offset form (the builtin expands to a 64-bit per-lane address); M0 holds
-// the LDS byte address of the wave's 1 KB destination.
+// HBM -> LDS, 16 bytes per lane, no register staging.  One instruction moves 16 tile rows of one ring
+// stage (64 lanes x 16 B = 16 rows x 64 B); wave w of a round moves rows [w*16, w*16+16) of that round.
+// Written as inline assembly to get the scalar-base + 32-bit-lane-offset form (the builtin expands to a
+// 64-bit per-lane address); M0 holds the LDS byte address of the wave's 1 KB destination.
 __device__ __forceinline__ void gg_dma16(const uint8_t* sbase, uint32_t voff, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0" : : "s"(sbase), "v"(voff), "s"(lds_addr) : "memory");
 }
@@ -127,19 +145,6 @@ __device__ __forceinline__ const uint8_t* gg_uniform(const uint8_t* p) {
     return (const uint8_t*)(((uint64_t)hi << 32) | lo);
 }
 
-template <int RA, int RB, int LR>
-__device__ __forceinline__ void gg_issue(uint4* sA, uint4* sB, const uint8_t* ap, const uint8_t* bp,
-                                         const uint32_t* a_off, uint32_t b_off0, uint32_t b_step, int wave) {
-    ap = gg_uniform(ap);
-    bp = gg_uniform(bp);
-    const uint32_t la = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(sA + wave * 8 * CHUNKS));
-    const uint32_t lb = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(sB + wave * 8 * CHUNKS));
-#pragma unroll
-    for (int r = 0; r < RA; ++r) gg_dma16(ap, a_off[r], la + r * LR * CHUNKS * 16);
-#pragma unroll
-    for (int r = 0; r < RB; ++r) gg_dma16(bp + (size_t)r * b_step, b_off0, lb + r * LR * CHUNKS * 16);
-}
-
 template <int TM, int TN>
 __device__ __forceinline__ void gg_frags(const uint4* fa, const uint4* fb, int pos, uint4 (&a)[TM], uint4 (&b)[TN]) {
 #pragma unroll
@@ -148,14 +153,42 @@ __device__ __forceinline__ void gg_frags(const uint4* fa, const uint4* fb, int p
     for (int j = 0; j < TN; ++j) b[j] = fb[j * 32 * CHUNKS + pos];
 }
 
-// weights are the MFMA A operand and activations the B operand, so acc holds the transposed product
-template <int TM, int TN, bool FP8>
-__device__ __forceinline__ void gg_mmas(floatx16 (&acc)[TM][TN], const uint4 (&a)[TM], const uint4 (&b)[TN]) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) mma<FP8>(acc[i][j], b[j], a[i]);
-}
+// Order of the TM x TN products of one MFMA block and of the TM + TN fragment reads that feed the
+// next block: fragments are read a0, b0, a1, b1, ... and the products are taken in the order in which
+// their operands arrive ((0,0); then everything that needs a1; then everything that needs b1; ...), so
+// a read issued late in one block is not needed before late in the next.
+template <int TM, int TN>
+struct GgOrder {
+    static constexpr int NT = TM * TN, NR = TM + TN, D = TM > TN ? TM : TN;
+    // I-th product -> (a index, b index)
+    static constexpr int prod(int I, bool want_a) {
+        int n = 0;
+        for (int d = 0; d < D; ++d) {
+            if (d < TM)
+                for (int j = 0; j < (d < TN ? d : TN); ++j, ++n)
+                    if (n == I) return want_a ? d : j;
+            if (d < TN)
+                for (int i = 0; i <= (d < TM ? d : TM - 1); ++i, ++n)
+                    if (n == I) return want_a ? i : d;
+        }
+        return 0;
+    }
+    // R-th read -> operand (true: a) and index
+    static constexpr int read(int R, bool want_is_a) {
+        int n = 0;
+        for (int d = 0; d < D; ++d) {
+            if (d < TM) { if (n == R) return want_is_a ? 1 : d; ++n; }
+            if (d < TN) { if (n == R) return want_is_a ? 0 : d; ++n; }
+        }
+        return 0;
+    }
+    // the read issued behind product I (-1: none): reads are spread evenly over the block
+    static constexpr int read_at(int I) {
+        for (int R = 0; R < NR; ++R)
+            if ((R * NT) / NR == I) return R;
+        return -1;
+    }
+};
 
 // s_waitcnt through the builtin (not inline asm) so that the compiler's own wait-count bookkeeping
 // sees it.  gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14.
@@ -164,37 +197,40 @@ __device__ __forceinline__ void gg_wait() {
     static_assert(VM >= 0 && VM <= 63 && LGKM >= 0 && LGKM <= 15, "wait counts");
     __builtin_amdgcn_s_waitcnt((VM & 15) | (7 << 4) | (LGKM << 8) | ((VM >> 4) << 14));
 }
-template <int N>
-__device__ __forceinline__ void gg_wait_vm() {
-    gg_wait<N, 15>();
-}
 
 // acc(i,j) holds the TRANSPOSED 32x32 product (weights as the MFMA A operand, activations as B):
 // lane l owns token row l%32 and output columns 8*(v/4) + 4*(l/32) + v%4, v = 0..15, i.e. four runs
 // of four consecutive columns -> 8-byte bf16 stores.
 // NWM x 2 wave64s per workgroup; every wave owns a (BM/NWM) x 128 block of the tile.
+//
+// K moves through LDS in a ring of NRING stages of ROWB bytes per tile row.  A stage is two MFMA
+// blocks (one per 32 bytes of K).  The loads of stage s+4 go into the slot of stage s as soon as every
+// wave holds the last fragments of stage s in registers, and are spread over the two MFMA blocks that
+// follow, so the load pipe sees a steady stream instead of a burst and every load has two full stages
+// of MFMA work to land.
 template <int BM, int NWM, int EPI, bool FP8>
 __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const GemmParams p) {
     constexpr int BN = GG_BN;
     constexpr int ES = FP8 ? 1 : 2;
-    constexpr int BK = ROWB / ES;
-    constexpr int NW = NWM * 2;                       // waves per workgroup
+    constexpr int NW = NWM * 2;                        // waves per workgroup
     constexpr int TM = BM / (NWM * 32), TN = BN / 64;  // 32x32 MFMA tiles per wave
-    constexpr int LR = NW * 8;                        // rows fetched per load round (8 per wave)
-    constexpr int RA = BM / LR, RB = BN / LR;         // load rounds per stage
-    constexpr int NKK = CHUNKS / 2;            // fragment steps per stage (4)
+    constexpr int NT = TM * TN;
+    constexpr int LR = NW * WROWS;                     // rows fetched per load round (16 per wave)
+    constexpr int RA = BM / LR, RB = BN / LR;          // load rounds per stage
+    constexpr int LPS = RA + RB;                       // HBM->LDS loads per lane per stage
+    constexpr int LH = LPS / 2;                        // ... per MFMA block
+    constexpr int ASLOT = BM * CHUNKS, BSLOT = BN * CHUNKS;  // uint4 per ring slot
+    static_assert(TM * 32 * NWM == BM && BM % LR == 0 && BN % LR == 0 && LPS % 2 == 0 && LH <= NT, "tile shape");
+    static_assert(CHUNKS == 4 && NRING == 4, "the stage schedule below is written for two MFMA blocks per stage and four slots");
 
-    __shared__ __align__(1024) uint4 sA0[BM * CHUNKS];
-    __shared__ __align__(1024) uint4 sB0[BN * CHUNKS];
-    __shared__ __align__(1024) uint4 sA1[BM * CHUNKS];
-    __shared__ __align__(1024) uint4 sB1[BN * CHUNKS];
+    __shared__ __align__(1024) uint4 sA[NRING * ASLOT];
+    __shared__ __align__(1024) uint4 sB[NRING * BSLOT];
     __shared__ int g_tile_start[GG_MAXG + 1];
     __shared__ int g_row_start[GG_MAXG + 1];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int Nt = p.Npad / BN;
-    static_assert(TM * 32 * NWM == BM && LR % 16 == 0, "tile shape");
 
     if (tid == 0) {
         int ts = 0, rs = 0;
@@ -210,7 +246,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     }
     __syncthreads();
     const int total = g_tile_start[p.E_l];
-    const int nk = p.K / BK;
+    const int nk = (p.K * ES) / ROWB;  // ring stages per tile; even (K * ES is a multiple of 2 * ROWB)
 
     // XCD-aware position inside a round of gridDim.x tiles: workgroups b, b+8, b+16, ... share an L2.
     int my = blockIdx.x;
@@ -219,29 +255,61 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         my = (((xcd >> 1) * 4 + (l >> 3)) * SUP) + ((xcd & 1) * 8 + (l & 7));
     }
 
-    // lane-constant pieces of the addressing
-    const int lrow = wave * 8 + (lane >> 3);            // row inside a load round
-    const int lchunk = (lane & 7) ^ ((lrow >> 1) & 7);  // global 16-byte chunk this lane fetches
-    const int fswz = (lane >> 1) & 7;                   // swizzle of the fragment row (row % 16 = lane % 16)
+    // lane-constant pieces of the addressing.  A tile row is 4 chunks of 16 bytes; row r keeps logical
+    // chunk c at position c ^ ((r >> 2) & 3), which makes both the 16-rows-per-instruction DMA writes
+    // and the 128-bit fragment reads (rows = lane % 32) bank-conflict free.
+    const int lrow = wave * WROWS + (lane >> 2);         // row inside a load round
+    const int lchunk = (lane & 3) ^ ((lane >> 4) & 3);   // global 16-byte chunk this lane fetches
+    const int fswz = (lane >> 2) & 3;                    // swizzle of the fragment row
     const int khalf = lane >> 5;
-    const uint4* fa0 = sA0 + (wm * (BM / NWM) + (lane & 31)) * CHUNKS;
-    const uint4* fa1 = sA1 + (wm * (BM / NWM) + (lane & 31)) * CHUNKS;
-    const uint4* fb0 = sB0 + (wn * (BN / 2) + (lane & 31)) * CHUNKS;
-    const uint4* fb1 = sB1 + (wn * (BN / 2) + (lane & 31)) * CHUNKS;
+    const int pos0 = (0 + khalf) ^ fswz, pos1 = (2 + khalf) ^ fswz;
+    const uint4* fa = sA + (wm * (BM / NWM) + (lane & 31)) * CHUNKS;
+    const uint4* fb = sB + (wn * (BN / 2) + (lane & 31)) * CHUNKS;
+    const uint32_t la0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(sA + wave * WROWS * CHUNKS));
+    const uint32_t lb0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(sB + wave * WROWS * CHUNKS));
 
-    // Tiles are software-pipelined: the first two K stages of the next tile are requested before the
-    // epilogue of the current one, so the stores of one tile overlap the first loads of the next.
     const uint32_t ldk = (uint32_t)(p.K * ES);
     const size_t b_slab = (size_t)p.Npad * ROWB;  // packed weights are slab-major: [group][K slab][Npad rows][ROWB bytes]
     const uint32_t b_off0 = (uint32_t)lrow * ROWB + lchunk * 16;
-    const uint32_t b_step = (uint32_t)LR * ROWB;
+
 #define GG_TILE_PTRS(t, Ab_, Bb_, aoff_)                                                                   \
     const uint8_t* Ab_ = p.A + (size_t)(t).row0 * p.K * ES;                                                 \
     const uint8_t* Bb_ = p.B + (size_t)(t).g * p.Npad * p.K * ES + (size_t)(t).nt * BN * ROWB;               \
     uint32_t aoff_[RA];                                                                                     \
     _Pragma("unroll") for (int r = 0; r < RA; ++r) aoff_[r] = (uint32_t)min(r * LR + lrow, (t).rv - 1) * ldk + lchunk * 16;
-#define GG_ISSUE_T(sA, sB, Ab_, Bb_, aoff_, ks) \
-    gg_issue<RA, RB, LR>(sA, sB, Ab_ + (size_t)(ks) * ROWB, Bb_ + (size_t)(ks) * b_slab, aoff_, b_off0, b_step, wave)
+    // load d (0 .. LPS-1) of one stage: A rounds first, then B rounds
+#define GG_LD(d, ap_, bp_, aoff_, slot)                                                                       \
+    do {                                                                                                      \
+        if constexpr ((d) < RA) gg_dma16(ap_, aoff_[(d) < RA ? (d) : 0], la0 + ((slot) * ASLOT + (d) * LR * CHUNKS) * 16); \
+        else gg_dma16(bp_ + (size_t)((d) - RA) * (LR * ROWB), b_off0, lb0 + ((slot) * BSLOT + ((d) - RA) * LR * CHUNKS) * 16); \
+    } while (0)
+    // loads [first, first + count) of stage `st` (clamped to the last stage: the ring never holds data
+    // of another tile, and a repeated load of the last stage lands in a slot nobody reads again)
+#define GG_STAGE_PTRS(Ab_, Bb_, st, ap_, bp_)                                                  \
+    const int st_ = min((st), nk - 1);                                                         \
+    const uint8_t* ap_ = gg_uniform(Ab_ + (size_t)st_ * ROWB);                                 \
+    const uint8_t* bp_ = gg_uniform(Bb_ + (size_t)st_ * b_slab);
+#define GG_ISSUE_RANGE(Ab_, Bb_, aoff_, st, slot, first, count)                                \
+    do {                                                                                       \
+        GG_STAGE_PTRS(Ab_, Bb_, st, ap_i, bp_i)                                                \
+        if constexpr ((first) + 0 < (first) + (count)) GG_LD((first) + 0 < LPS ? (first) + 0 : 0, ap_i, bp_i, aoff_, slot); \
+        if constexpr ((first) + 1 < (first) + (count)) GG_LD((first) + 1 < LPS ? (first) + 1 : 0, ap_i, bp_i, aoff_, slot); \
+        if constexpr ((first) + 2 < (first) + (count)) GG_LD((first) + 2 < LPS ? (first) + 2 : 0, ap_i, bp_i, aoff_, slot); \
+        if constexpr ((first) + 3 < (first) + (count)) GG_LD((first) + 3 < LPS ? (first) + 3 : 0, ap_i, bp_i, aoff_, slot); \
+        if constexpr ((first) + 4 < (first) + (count)) GG_LD((first) + 4 < LPS ? (first) + 4 : 0, ap_i, bp_i, aoff_, slot); \
+        if constexpr ((first) + 5 < (first) + (count)) GG_LD((first) + 5 < LPS ? (first) + 5 : 0, ap_i, bp_i, aoff_, slot); \
+        if constexpr ((first) + 6 < (first) + (count)) GG_LD((first) + 6 < LPS ? (first) + 6 : 0, ap_i, bp_i, aoff_, slot); \
+        if constexpr ((first) + 7 < (first) + (count)) GG_LD((first) + 7 < LPS ? (first) + 7 : 0, ap_i, bp_i, aoff_, slot); \
+        static_assert((count) <= 8, "GG_ISSUE_RANGE is unrolled for eight loads");             \
+    } while (0)
+    // what a tile has in flight before its first MFMA: stages 0, 1, 2 and the first half of stage 3
+#define GG_PROLOGUE(Ab_, Bb_, aoff_)                          \
+    do {                                                      \
+        GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 0, 0, 0, LPS);        \
+        GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 1, 1, 0, LPS);        \
+        GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 2, 2, 0, LPS);        \
+        GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 3, 3, 0, LH);         \
+    } while (0)
 
     int base = 0;
     GgTile cur = gg_next_tile<BM>(g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, total, my, gridDim.x, base);
@@ -253,8 +321,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         Bb = Bb0;
 #pragma unroll
         for (int r = 0; r < RA; ++r) a_off[r] = a_off0[r];
-        GG_ISSUE_T(sA0, sB0, Ab, Bb, a_off, 0);
-        if (nk > 1) GG_ISSUE_T(sA1, sB1, Ab, Bb, a_off, 1);
+        GG_PROLOGUE(Ab, Bb, a_off);
     }
     while (cur.rv > 0) {
         const int g = __builtin_amdgcn_readfirstlane(cur.g), nt = __builtin_amdgcn_readfirstlane(cur.nt);
@@ -269,94 +336,103 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
         uint4 a0[TM], b0[TN], a1[TM], b1[TN];
-        constexpr int NMMA = TM * TN * (FP8 ? 2 : 1);  // MFMA instructions per fragment step
-        constexpr int LPS = RA + RB;                   // HBM->LDS loads per lane per stage
-        static_assert(LPS == 8 || LPS == 12, "load interleave is written for 8 or 12 loads per stage");
-        const int pos0 = (0 + khalf) ^ fswz, pos1 = (2 + khalf) ^ fswz, pos2 = (4 + khalf) ^ fswz, pos3 = (6 + khalf) ^ fswz;
-        static_assert(NKK == 4, "GG_STAGE is written for four fragment steps");
+        static_assert(NT == 8 || NT == 16, "GG_BLOCK is unrolled for 8 or 16 MFMA tiles per wave");
 
-        // One K stage: fragments of step kk+1 are requested before the MFMAs of step kk are issued;
-        // the stage hand-over (loads landed + barrier + refill of the buffer just drained) sits before
-        // the last MFMA block so that its latency hides behind that block.
-#define GG_ISSUE(sA, sB, ks) \
-    gg_issue<RA, RB, LR>(sA, sB, Ab + (size_t)(ks) * ROWB, Bb + (size_t)(ks) * b_slab, a_off, b_off0, b_step, wave)
-#define GG_ORDER()                                                          \
-    do {                                                                    \
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                  \
-        __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);            \
-        __builtin_amdgcn_sched_group_barrier(0x008, NMMA - 1, 0);           \
-        __builtin_amdgcn_sched_barrier(0);                                  \
-    } while (0)
-        static_assert(TM * TN == 8, "GG_MD is unrolled for eight MFMA tiles per wave");
-        /* I-th MFMA of the block, then its share of the stage's loads (constant indices only) */
-#define GG_LD(d)                                                                                         \
+        // One MFMA block: the NT products of one 32-byte K step, with (a) the fragment reads of the next
+        // step right behind the first MFMA and (b) LH loads of a later stage spread between the MFMAs.
+        // Everything is pinned by scheduling fences: each load is issued in the shadow of an MFMA.
+        using Ord = GgOrder<TM, TN>;
+#define GG_MM(I, FA_, FB_)                                                                               \
     do {                                                                                                 \
-        if constexpr ((d) < RA) gg_dma16(ap_, a_off[(d) < RA ? (d) : 0], la_ + (d) * LR * CHUNKS * 16);     \
-        else if constexpr ((d) < LPS) gg_dma16(bp_ + (size_t)((d) - RA) * b_step, b_off0, lb_ + ((d) - RA) * LR * CHUNKS * 16); \
+        constexpr int pa_ = Ord::prod(I, true), pb_ = Ord::prod(I, false);                               \
+        mma<FP8>(acc[pa_][pb_], FB_[pb_], FA_[pa_]);                                                     \
     } while (0)
-#define GG_MD(I)                                                                                         \
+        // fragment read R of the next step, from slot-relative bases nfa_/nfb_ at chunk position npos_
+#define GG_RD(R, NA_, NB_)                                                                               \
     do {                                                                                                 \
-        mma<FP8>(acc[(I) / TN][(I) % TN], b1[(I) % TN], a1[(I) / TN]);                                   \
-        __builtin_amdgcn_sched_barrier(0);                                                               \
-        if (more_) {                                                                                     \
-            if constexpr (LPS == 8) { GG_LD(I); }                                                        \
-            else { GG_LD(((I) * 3) / 2); if constexpr ((I) % 2 == 1) GG_LD(((I) * 3) / 2 + 1); }         \
+        constexpr bool ra_ = Ord::read(R, true) != 0;                                                    \
+        constexpr int ri_ = Ord::read(R, false);                                                         \
+        if constexpr (ra_) NA_[ri_] = nfa_[ri_ * 32 * CHUNKS + npos_];                                   \
+        else NB_[ri_] = nfb_[ri_ * 32 * CHUNKS + npos_];                                                 \
+    } while (0)
+#define GG_ML(I, FA_, FB_, NA_, NB_, aoff_, slot, half)                                                  \
+    do {                                                                                                 \
+        if constexpr ((I) < NT) {                                                                        \
+            GG_MM(I, FA_, FB_);                                                                          \
+            __builtin_amdgcn_sched_barrier(0);                                                           \
+            constexpr int rd_ = Ord::read_at(I);                                                         \
+            if constexpr (rd_ >= 0) GG_RD((rd_ >= 0 ? rd_ : 0), NA_, NB_);                               \
+            if constexpr (((I) + 1) * LH / NT > (I) * LH / NT) GG_LD((half) * LH + (I) * LH / NT, ap_, bp_, aoff_, slot); \
+            __builtin_amdgcn_sched_barrier(0);                                                           \
         }                                                                                                \
+    } while (0)
+        // One MFMA block: the NT products of one 32-byte K step (FA_, FB_), with the fragment reads of the
+        // next step (into NA_, NB_) and LH loads of a later stage spread between them.  Everything is
+        // pinned by scheduling fences: each read and each load is issued in the shadow of an MFMA.
+#define GG_BLOCK(FA_, FB_, NA_, NB_, nslot, npos, st, slot, half)                                        \
+    do {                                                                                                 \
+        GG_STAGE_PTRS(Ab, Bb, st, ap_, bp_)                                                              \
+        const uint4* nfa_ = fa + (nslot) * ASLOT;                                                        \
+        const uint4* nfb_ = fb + (nslot) * BSLOT;                                                        \
+        const int npos_ = (npos);                                                                        \
         __builtin_amdgcn_sched_barrier(0);                                                               \
+        GG_ML(0, FA_, FB_, NA_, NB_, a_off, slot, half); GG_ML(1, FA_, FB_, NA_, NB_, a_off, slot, half);   \
+        GG_ML(2, FA_, FB_, NA_, NB_, a_off, slot, half); GG_ML(3, FA_, FB_, NA_, NB_, a_off, slot, half);   \
+        GG_ML(4, FA_, FB_, NA_, NB_, a_off, slot, half); GG_ML(5, FA_, FB_, NA_, NB_, a_off, slot, half);   \
+        GG_ML(6, FA_, FB_, NA_, NB_, a_off, slot, half); GG_ML(7, FA_, FB_, NA_, NB_, a_off, slot, half);   \
+        GG_ML(8, FA_, FB_, NA_, NB_, a_off, slot, half); GG_ML(9, FA_, FB_, NA_, NB_, a_off, slot, half);   \
+        GG_ML(10, FA_, FB_, NA_, NB_, a_off, slot, half); GG_ML(11, FA_, FB_, NA_, NB_, a_off, slot, half); \
+        GG_ML(12, FA_, FB_, NA_, NB_, a_off, slot, half); GG_ML(13, FA_, FB_, NA_, NB_, a_off, slot, half); \
+        GG_ML(14, FA_, FB_, NA_, NB_, a_off, slot, half); GG_ML(15, FA_, FB_, NA_, NB_, a_off, slot, half); \
     } while (0)
-#define GG_STAGE(fa, fb, na, nb, curA, curB, ks)                           \
-    do {                                                                   \
-        gg_frags<TM, TN>(fa, fb, pos1, a1, b1);                            \
-        gg_mmas<TM, TN, FP8>(acc, a0, b0);                                 \
-        GG_ORDER();                                                        \
-        gg_frags<TM, TN>(fa, fb, pos2, a0, b0);                            \
-        gg_mmas<TM, TN, FP8>(acc, a1, b1);                                 \
-        GG_ORDER();                                                        \
-        gg_frags<TM, TN>(fa, fb, pos3, a1, b1);                            \
-        gg_mmas<TM, TN, FP8>(acc, a0, b0);                                 \
-        GG_ORDER();                                                        \
-        if ((ks) + 1 < nk) {                                               \
-            gg_wait<0, 0>();                                               \
-            __syncthreads();                                               \
-            gg_frags<TM, TN>(na, nb, pos0, a0, b0);                        \
-            __builtin_amdgcn_sched_barrier(0);                             \
-        }                                                                  \
-        {                                                                  \
-            /* last MFMA block of the stage with the refill loads spread between its MFMAs: each load  \
-               is issued in the shadow of the MFMA before it, so the matrix pipe does not drain */     \
-            const bool more_ = (ks) + 2 < nk;                                                            \
-            const uint8_t* ap_ = gg_uniform(Ab + (size_t)((ks) + 2) * ROWB);                             \
-            const uint8_t* bp_ = gg_uniform(Bb + (size_t)((ks) + 2) * b_slab);                           \
-            const uint32_t la_ = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)((curA) + wave * 8 * CHUNKS)); \
-            const uint32_t lb_ = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)((curB) + wave * 8 * CHUNKS)); \
-            GG_MD(0); GG_MD(1); GG_MD(2); GG_MD(3); GG_MD(4); GG_MD(5); GG_MD(6); GG_MD(7);              \
-        }                                                                  \
-        __builtin_amdgcn_sched_barrier(0);                                 \
+        // Stage s of the tile sits in slot s % 4 (SL below).  Block 0 multiplies the fragments of its first
+        // K step while those of the second are read, and issues the second half of stage s+3's loads
+        // (slot SL+3); the hand-over waits for this wave's own loads of stage s+1 (everything issued
+        // after them -- stages s+2 and s+3 -- may stay in flight) and for its last fragments of stage s,
+        // then meets the other waves; block 1 reads the first fragments of stage s+1 and refills slot SL
+        // with the first half of stage s+4.  In the last stage of a tile block 1 still reads "the next
+        // stage" (whatever slot SL+1 holds): those fragments are never used.
+#define GG_STAGE(SL, s, last)                                                                            \
+    do {                                                                                                 \
+        GG_BLOCK(a0, b0, a1, b1, SL, pos1, (s) + 3, ((SL) + 3) & 3, 1);                                  \
+        if (!(last)) {                                                                                   \
+            gg_wait<2 * LPS, 0>();                                                                       \
+            __builtin_amdgcn_s_barrier();                                                                \
+        }                                                                                                \
+        GG_BLOCK(a1, b1, a0, b0, ((SL) + 1) & 3, pos0, (s) + 4, SL, 0);                                  \
     } while (0)
 
-        // stages 0 and 1 of this tile were requested before the previous tile's epilogue (or above, for the
-        // first tile); the epilogue's stores sit behind them in the same counter, so wait for everything
-        gg_wait_vm<0>();
+        // stages 0-2 and half of stage 3 of this tile were requested before the previous tile's epilogue
+        // (or above, for the first tile); the epilogue's stores sit behind them in the same counter, so
+        // wait for everything once per tile
+        gg_wait<0, 15>();
         __syncthreads();
-        gg_frags<TM, TN>(fa0, fb0, pos0, a0, b0);
-        for (int ks = 0; ks < nk; ks += 2) {
-            GG_STAGE(fa0, fb0, fa1, fb1, sA0, sB0, ks);
-            if (ks + 1 < nk) GG_STAGE(fa1, fb1, fa0, fb0, sA1, sB1, ks + 1);
-        }
+        gg_frags<TM, TN>(fa, fb, pos0, a0, b0);
+        // nk >= 2 and even: a loop that cannot run zero times keeps the accumulators in place from their
+        // zeroing to the epilogue
+        int ks = 0;
+        do {
+            GG_STAGE(0, ks, false);
+            GG_STAGE(1, ks + 1, ks + 2 >= nk);
+            if (ks + 2 < nk) {
+                GG_STAGE(2, ks + 2, false);
+                GG_STAGE(3, ks + 3, ks + 4 >= nk);
+            }
+            ks += 4;
+        } while (ks < nk);
 #undef GG_STAGE
-#undef GG_MD
-#undef GG_LD
-#undef GG_ORDER
-#undef GG_ISSUE
+#undef GG_BLOCK
+#undef GG_ML
+#undef GG_RD
+#undef GG_MM
 
-        // ---- next tile: decode it and request its first two stages now (both LDS buffers are free once
-        // every wave has passed the barrier: the last fragments of this tile are already in registers)
+        // ---- next tile: decode it and request its first stages now (every slot is free once all waves
+        // have passed the barrier: the last fragments of this tile are already in registers)
         const GgTile nxt = gg_next_tile<BM>(g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, total, my, gridDim.x, base);
         GG_TILE_PTRS(nxt, Ab_n, Bb_n, a_off_n);
         if (nxt.rv > 0) {
             __syncthreads();
-            GG_ISSUE_T(sA0, sB0, Ab_n, Bb_n, a_off_n, 0);
-            if (nk > 1) GG_ISSUE_T(sA1, sB1, Ab_n, Bb_n, a_off_n, 1);
+            GG_PROLOGUE(Ab_n, Bb_n, a_off_n);
         }
 
         // ---- epilogue: acc -> (scales) -> activation -> bf16 -> C
@@ -392,7 +468,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                         for (int e = 0; e < 4; ++e) {
                             float gv = acc[i][j][4 * q + e], uv = acc[i][j + 1][4 * q + e];
                             if constexpr (FP8) { gv *= cg[e]; uv *= cu[e]; }
-                            x[e] = act_silu(gv) * uv;
+                            x[e] = act_silu_fast(gv) * uv;
                         }
                     } else {
                         col = nt * BN + wn * (BN / 2) + j * 32 + 8 * q + chalf;
@@ -408,17 +484,20 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                             float v = acc[i][j][4 * q + e];
                             if constexpr (FP8) v *= cs[e];
                             if constexpr (EPI == EPI_GELU) v = act_gelu(v);
-                            if constexpr (EPI == EPI_SILU) v = act_silu(v);
+                            if constexpr (EPI == EPI_SILU) v = act_silu_fast(v);
                             x[e] = v;
                         }
                     }
                     if (ok && col < p.N) {
                         uint2 o;
-                        o.x = (uint32_t)f32_to_bf16(x[0]) | ((uint32_t)f32_to_bf16(x[1]) << 16);
-                        o.y = (uint32_t)f32_to_bf16(x[2]) | ((uint32_t)f32_to_bf16(x[3]) << 16);
+                        o.x = gg_pack_bf16(x[0], x[1]);
+                        o.y = gg_pack_bf16(x[2], x[3]);
                         *(uint2*)(crow + col) = o;
                     }
                 }
+                // keep the accumulator read-out of one 32x32 tile from being hoisted over the previous
+                // tile's stores (with 16 tiles per wave that would need every accumulator in a VGPR at once)
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         cur = nxt;
@@ -428,7 +507,10 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         for (int r = 0; r < RA; ++r) a_off[r] = a_off_n[r];
     }
 #undef GG_TILE_PTRS
-#undef GG_ISSUE_T
+#undef GG_LD
+#undef GG_STAGE_PTRS
+#undef GG_ISSUE_RANGE
+#undef GG_PROLOGUE
 }
 
 // ---- one-time weight re-tiling: w [E_l,K,N] (N contiguous) -> out [E_l][K/SK][Npad][SK], SK = one LDS
@@ -625,7 +707,7 @@ int launch_gemm(const GemmParams& p, int epi, hipStream_t s) {
 #define GG_EPI(EPIv)                          \
     do {                                      \
         if (small_m) GG_LAUNCH(128, 2, EPIv); \
-        else GG_LAUNCH(256, 4, EPIv);         \
+        else GG_LAUNCH(256, GG_BIG_NWM, EPIv); \
     } while (0)
     switch (epi) {
         case EPI_NONE: GG_EPI(EPI_NONE); break;
