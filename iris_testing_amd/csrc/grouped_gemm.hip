@@ -182,10 +182,17 @@ struct GgOrder {
         }
         return 0;
     }
-    // the read issued behind product I (-1: none): reads are spread evenly over the block
-    static constexpr int read_at(int I) {
+    // the n-th (0 or 1) read issued behind product I (-1: none).  Reads are spread evenly over the whole
+    // block, or over its first half when the block ends in a hand-over (the wave must hold its last
+    // fragments of a slot before it lets the other waves refill that slot).
+    static constexpr int read_at(int I, bool front, int n) {
+        const int span = front ? NT / 2 : NT;
+        int seen = 0;
         for (int R = 0; R < NR; ++R)
-            if ((R * NT) / NR == I) return R;
+            if ((R * span) / NR == I) {
+                if (seen == n) return R;
+                ++seen;
+            }
         return -1;
     }
 };
@@ -360,8 +367,9 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         if constexpr ((I) < NT) {                                                                        \
             GG_MM(I, FA_, FB_);                                                                          \
             __builtin_amdgcn_sched_barrier(0);                                                           \
-            constexpr int rd_ = Ord::read_at(I);                                                         \
+            constexpr int rd_ = Ord::read_at(I, (half) == 1, 0), rd2_ = Ord::read_at(I, (half) == 1, 1); \
             if constexpr (rd_ >= 0) GG_RD((rd_ >= 0 ? rd_ : 0), NA_, NB_);                               \
+            if constexpr (rd2_ >= 0) GG_RD((rd2_ >= 0 ? rd2_ : 0), NA_, NB_);                            \
             if constexpr (((I) + 1) * LH / NT > (I) * LH / NT) GG_LD((half) * LH + (I) * LH / NT, ap_, bp_, aoff_, slot); \
             __builtin_amdgcn_sched_barrier(0);                                                           \
         }                                                                                                \
