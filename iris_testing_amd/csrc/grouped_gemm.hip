@@ -74,6 +74,16 @@ __device__ __forceinline__ void mma(floatx16& acc, const uint4& a, const uint4& 
     }
 }
 
+// fp8: one 32x32x64 MFMA on 32 bytes of K per lane and operand (two 16-byte LDS chunks); both operands
+// are split over the lanes and registers in the same way, so every k is multiplied exactly once
+typedef int gg_i32x8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ void mma_fp8_k64(floatx16& acc, const uint4& a_lo, const uint4& a_hi, const uint4& b_lo, const uint4& b_hi) {
+    const gg_i32x8 a = {(int)a_lo.x, (int)a_lo.y, (int)a_lo.z, (int)a_lo.w, (int)a_hi.x, (int)a_hi.y, (int)a_hi.z, (int)a_hi.w};
+    const gg_i32x8 b = {(int)b_lo.x, (int)b_lo.y, (int)b_lo.z, (int)b_lo.w, (int)b_hi.x, (int)b_hi.y, (int)b_hi.z, (int)b_hi.w};
+    // format selectors 0/0 = fp8 (e4m3) for both operands, no block scales
+    acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc, 0, 0, 0, 0, 0, 0);
+}
+
 __device__ __forceinline__ int seg_of(const int* off, int n, int r) {
     int lo = 0, hi = n;
     while (hi - lo > 1) {
@@ -315,7 +325,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 0, 0, 0, LPS);        \
         GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 1, 1, 0, LPS);        \
         GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 2, 2, 0, LPS);        \
-        GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 3, 3, 0, LH);         \
+        GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 3, 3, 0, (FP8 ? LPS : LH)); \
     } while (0)
 
     int base = 0;
@@ -342,7 +352,6 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-        uint4 a0[TM], b0[TN], a1[TM], b1[TN];
         static_assert(NT == 8 || NT == 16, "GG_BLOCK is unrolled for 8 or 16 MFMA tiles per wave");
 
         // One MFMA block: the NT products of one 32-byte K step, with (a) the fragment reads of the next
@@ -410,24 +419,93 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         GG_BLOCK(a1, b1, a0, b0, ((SL) + 1) & 3, pos0, (s) + 4, SL, 0);                                  \
     } while (0)
 
-        // stages 0-2 and half of stage 3 of this tile were requested before the previous tile's epilogue
-        // (or above, for the first tile); the epilogue's stores sit behind them in the same counter, so
-        // wait for everything once per tile
-        gg_wait<0, 15>();
-        __syncthreads();
-        gg_frags<TM, TN>(fa, fb, pos0, a0, b0);
-        // nk >= 2 and even: a loop that cannot run zero times keeps the accumulators in place from their
-        // zeroing to the epilogue
-        int ks = 0;
-        do {
-            GG_STAGE(0, ks, false);
-            GG_STAGE(1, ks + 1, ks + 2 >= nk);
-            if (ks + 2 < nk) {
-                GG_STAGE(2, ks + 2, false);
-                GG_STAGE(3, ks + 3, ks + 4 >= nk);
-            }
-            ks += 4;
-        } while (ks < nk);
+        // ---- fp8: one MFMA block per 64-byte stage (K = 64 per 32x32x64 MFMA).  Block s multiplies the
+        // fragments of stage s, reads those of stage s+1 (two 16-byte chunks per operand row, all issued in
+        // the first half of the block) and refills slot s % 4, drained one block earlier, with stage s+4;
+        // the hand-over at its end waits for the wave's own loads of stage s+2.
+#define GG_WRD(R, NA_, NB_)                                                                              \
+    do {                                                                                                 \
+        constexpr bool ra_ = Ord::read((R) / 2, true) != 0;                                              \
+        constexpr int ri_ = Ord::read((R) / 2, false), rh_ = (R) % 2;                                    \
+        if constexpr (ra_) NA_[2 * ri_ + rh_] = nfa_[ri_ * 32 * CHUNKS + (npos_ ^ rh_)];                 \
+        else NB_[2 * ri_ + rh_] = nfb_[ri_ * 32 * CHUNKS + (npos_ ^ rh_)];                               \
+    } while (0)
+#define GG_WML(I, FA_, FB_, NA_, NB_, slot)                                                              \
+    do {                                                                                                 \
+        if constexpr ((I) < NT) {                                                                        \
+            constexpr int pa_ = Ord::prod(I, true), pb_ = Ord::prod(I, false);                           \
+            mma_fp8_k64(acc[pa_][pb_], FB_[2 * pb_], FB_[2 * pb_ + 1], FA_[2 * pa_], FA_[2 * pa_ + 1]);  \
+            __builtin_amdgcn_sched_barrier(0);                                                           \
+            if constexpr ((I) < Ord::NR) { GG_WRD(2 * ((I) < Ord::NR ? (I) : 0), NA_, NB_); GG_WRD(2 * ((I) < Ord::NR ? (I) : 0) + 1, NA_, NB_); } \
+            if constexpr (((I) + 1) * LPS / NT > (I) * LPS / NT) GG_LD((I) * LPS / NT, ap_, bp_, a_off, slot); \
+            __builtin_amdgcn_sched_barrier(0);                                                           \
+        }                                                                                                \
+    } while (0)
+#define GG_WSTAGE(FA_, FB_, NA_, NB_, SL, s, last)                                                       \
+    do {                                                                                                 \
+        GG_STAGE_PTRS(Ab, Bb, (s) + 4, ap_, bp_)                                                         \
+        const uint4* nfa_ = fa + (((SL) + 1) & 3) * ASLOT;                                               \
+        const uint4* nfb_ = fb + (((SL) + 1) & 3) * BSLOT;                                               \
+        const int npos_ = wpos;                                                                          \
+        __builtin_amdgcn_sched_barrier(0);                                                               \
+        GG_WML(0, FA_, FB_, NA_, NB_, SL); GG_WML(1, FA_, FB_, NA_, NB_, SL); GG_WML(2, FA_, FB_, NA_, NB_, SL);   \
+        GG_WML(3, FA_, FB_, NA_, NB_, SL); GG_WML(4, FA_, FB_, NA_, NB_, SL); GG_WML(5, FA_, FB_, NA_, NB_, SL);   \
+        GG_WML(6, FA_, FB_, NA_, NB_, SL); GG_WML(7, FA_, FB_, NA_, NB_, SL); GG_WML(8, FA_, FB_, NA_, NB_, SL);   \
+        GG_WML(9, FA_, FB_, NA_, NB_, SL); GG_WML(10, FA_, FB_, NA_, NB_, SL); GG_WML(11, FA_, FB_, NA_, NB_, SL); \
+        GG_WML(12, FA_, FB_, NA_, NB_, SL); GG_WML(13, FA_, FB_, NA_, NB_, SL); GG_WML(14, FA_, FB_, NA_, NB_, SL); \
+        GG_WML(15, FA_, FB_, NA_, NB_, SL);                                                              \
+        if (!(last)) {                                                                                   \
+            gg_wait<2 * LPS, 0>();                                                                       \
+            __builtin_amdgcn_s_barrier();                                                                \
+        }                                                                                                \
+    } while (0)
+        if constexpr (FP8) {
+            uint4 wa0[2 * TM], wb0[2 * TN], wa1[2 * TM], wb1[2 * TN];
+            const int wpos = (2 * khalf) ^ fswz;  // first of the lane's two chunks (the second is wpos ^ 1)
+            // all four stages of this tile were requested before the previous tile's epilogue
+            gg_wait<0, 15>();
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < TM; ++i) { wa0[2 * i] = fa[i * 32 * CHUNKS + wpos]; wa0[2 * i + 1] = fa[i * 32 * CHUNKS + (wpos ^ 1)]; }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) { wb0[2 * j] = fb[j * 32 * CHUNKS + wpos]; wb0[2 * j + 1] = fb[j * 32 * CHUNKS + (wpos ^ 1)]; }
+            // slot 0 is refilled from the first block on: every wave must hold its stage-0 fragments first
+            gg_wait<63, 0>();
+            __syncthreads();
+            int ks = 0;
+            do {
+                GG_WSTAGE(wa0, wb0, wa1, wb1, 0, ks, false);
+                GG_WSTAGE(wa1, wb1, wa0, wb0, 1, ks + 1, ks + 2 >= nk);
+                if (ks + 2 < nk) {
+                    GG_WSTAGE(wa0, wb0, wa1, wb1, 2, ks + 2, false);
+                    GG_WSTAGE(wa1, wb1, wa0, wb0, 3, ks + 3, ks + 4 >= nk);
+                }
+                ks += 4;
+            } while (ks < nk);
+        } else {
+            uint4 a0[TM], b0[TN], a1[TM], b1[TN];
+            // stages 0-2 and half of stage 3 of this tile were requested before the previous tile's epilogue
+            // (or above, for the first tile); the epilogue's stores sit behind them in the same counter, so
+            // wait for everything once per tile
+            gg_wait<0, 15>();
+            __syncthreads();
+            gg_frags<TM, TN>(fa, fb, pos0, a0, b0);
+            // nk >= 2 and even: a loop that cannot run zero times keeps the accumulators in place from their
+            // zeroing to the epilogue
+            int ks = 0;
+            do {
+                GG_STAGE(0, ks, false);
+                GG_STAGE(1, ks + 1, ks + 2 >= nk);
+                if (ks + 2 < nk) {
+                    GG_STAGE(2, ks + 2, false);
+                    GG_STAGE(3, ks + 3, ks + 4 >= nk);
+                }
+                ks += 4;
+            } while (ks < nk);
+        }
+#undef GG_WSTAGE
+#undef GG_WML
+#undef GG_WRD
 #undef GG_STAGE
 #undef GG_BLOCK
 #undef GG_ML
