@@ -53,6 +53,7 @@ def _t(a, dtype):
 
 @pytest.mark.parametrize("dtype,E_l,K,N,S", [("bf16", 2, 128, 256, 300), ("bf16", 5, 192, 328, 777),
                                               ("bf16", 1, 4096, 512, 1500), ("bf16", 32, 256, 256, 3000),
+                                              ("bf16", 3, 64, 264, 1000),  # K = one pair of LDS ring stages
                                               ("f32", 2, 24, 48, 99), ("f32", 5, 128, 128, 333)])
 def test_grouped_gemm(dtype, E_l, K, N, S):
     """expert(tokens, weights, cnt): one GEMM per group, the shapes the reference meant to test
@@ -124,7 +125,7 @@ def test_quantize_rows_fp8_bit_exact(R, C):
     assert_bits_equal(q, oq, "fp8 codes")
 
 
-@pytest.mark.parametrize("E_l,H,F,S", [(2, 256, 384, 400), (15, 2048, 1408, 2500)])
+@pytest.mark.parametrize("E_l,H,F,S", [(2, 256, 384, 400), (15, 2048, 1408, 2500), (1, 128, 128, 700)])
 def test_expert_mlp_fp8(E_l, H, F, S):
     """The two GEMMs are checked separately with tight bounds (the second one against the oracle fed
     with the GPU's own hidden activation).  End to end the bound is loose on purpose: re-quantising
