@@ -360,6 +360,9 @@ int launch_logits(const XT* x, const XT* w, const float* bias, float* logits, in
         route_logits_small_kernel<XT, 4><<<gx, RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
     } else if (E <= 32) {
         route_logits_kernel<XT, 2, 4, 8><<<dim3(gx, 1), RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
+    } else if (gx * ceil_div(E, 64) < 2 * 256) {
+        // too few 64 x 64 blocks to give every SIMD two waves: halve the expert tile instead
+        route_logits_kernel<XT, 2, 4, 8><<<dim3(gx, ceil_div(E, 32)), RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
     } else {
         route_logits_kernel<XT, 4, 4, 16><<<dim3(gx, ceil_div(E, 64)), RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
     }
