@@ -788,7 +788,12 @@ int round_up(int a, int b) { return (a + b - 1) / b * b; }
 template <bool FP8>
 int launch_gemm(const GemmParams& p, int epi, hipStream_t s) {
     const int grid = num_cus();
-    const bool small_m = p.S_rows < 1024 * p.E_l;  // average group under four 256-row tiles
+    // 256-row or 128-row tiles: the host knows only the total row count, so it compares the estimated number
+    // of rounds of the persistent grid (every group adds about half a tile of ragged tail); a 128-row tile
+    // costs about 0.62 of a 256-row one
+    const int nt = p.Npad / GG_BN;
+    const double t256 = ((double)p.S_rows / 256 + 0.5 * p.E_l) * nt, t128 = ((double)p.S_rows / 128 + 0.5 * p.E_l) * nt;
+    const bool small_m = 0.62 * ceil(t128 / grid) < ceil(t256 / grid);
 #define GG_LAUNCH(BMv, NWMv, EPIv) grouped_gemm_kernel<BMv, NWMv, EPIv, FP8><<<grid, NWMv * 2 * WAVE, 0, s>>>(p)
 #define GG_EPI(EPIv)                          \
     do {                                      \
