@@ -729,23 +729,54 @@ __global__ __launch_bounds__(256) void grouped_gemm_f32_kernel(const float* __re
 }
 
 // ---- per-row fp8 quantisation of bf16 rows (one wave per row) -------------------------------------
+// Rows of up to 64 * NV * 8 columns are held in registers between the amax pass and the conversion, so
+// they are read from memory once; longer rows are read twice.
+__device__ __forceinline__ float fp8_row_amax(const uint4& v, float amax) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        amax = fmaxf(amax, fabsf(__uint_as_float(w[i] << 16)));
+        amax = fmaxf(amax, fabsf(__uint_as_float(w[i] & 0xffff0000u)));
+    }
+    return amax;
+}
+__device__ __forceinline__ uint2 fp8_row_convert(const uint4& v, float inv) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    float f[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = __fmul_rn(__uint_as_float(w[i] << 16), inv);
+        f[2 * i + 1] = __fmul_rn(__uint_as_float(w[i] & 0xffff0000u), inv);
+    }
+    int lo = 0, hi = 0;
+    lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], lo, false);
+    lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
+    hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], hi, false);
+    hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
+    return make_uint2((uint32_t)lo, (uint32_t)hi);
+}
+
+template <int NV>  // 16-byte vectors per lane kept in registers (0: stream the row twice)
 __global__ __launch_bounds__(256) void quantize_rows_fp8_kernel(const bf16_t* __restrict__ x, int rows, int cols,
                                                                  uint8_t* __restrict__ q, float* __restrict__ scale,
                                                                  const int32_t* __restrict__ n_rows_dev) {
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const int limit = n_rows_dev ? min(rows, *n_rows_dev) : rows;
+    const int nv = cols / 8;
     for (int r = blockIdx.x * 4 + wave; r < limit; r += gridDim.x * 4) {
         const uint4* src = (const uint4*)(x + (size_t)r * cols);
-        const int nv = cols / 8;
+        uint4 held[NV > 0 ? NV : 1];
         float amax = 0.f;
-        for (int c = lane; c < nv; c += WAVE) {
-            const uint4 v = src[c];
-            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        if constexpr (NV > 0) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                amax = fmaxf(amax, fabsf(__uint_as_float(w[i] << 16)));
-                amax = fmaxf(amax, fabsf(__uint_as_float(w[i] & 0xffff0000u)));
+            for (int i = 0; i < NV; ++i) {
+                const int c = lane + i * WAVE;
+                held[i] = c < nv ? src[c] : make_uint4(0, 0, 0, 0);
             }
+#pragma unroll
+            for (int i = 0; i < NV; ++i) amax = fp8_row_amax(held[i], amax);
+        } else {
+            for (int c = lane; c < nv; c += WAVE) amax = fp8_row_amax(src[c], amax);
         }
 #pragma unroll
         for (int off = WAVE / 2; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, WAVE));
@@ -753,21 +784,14 @@ __global__ __launch_bounds__(256) void quantize_rows_fp8_kernel(const bf16_t* __
         const float inv = zero ? 1.f : __fdiv_rn(448.f, amax);
         if (lane == 0) scale[r] = zero ? 1.f : __fdiv_rn(amax, 448.f);
         uint2* dst = (uint2*)(q + (size_t)r * cols);
-        for (int c = lane; c < nv; c += WAVE) {
-            const uint4 v = src[c];
-            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-            float f[8];
+        if constexpr (NV > 0) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                f[2 * i] = __fmul_rn(__uint_as_float(w[i] << 16), inv);
-                f[2 * i + 1] = __fmul_rn(__uint_as_float(w[i] & 0xffff0000u), inv);
+            for (int i = 0; i < NV; ++i) {
+                const int c = lane + i * WAVE;
+                if (c < nv) dst[c] = fp8_row_convert(held[i], inv);
             }
-            int lo = 0, hi = 0;
-            lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], lo, false);
-            lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
-            hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], hi, false);
-            hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
-            dst[c] = make_uint2((uint32_t)lo, (uint32_t)hi);
+        } else {
+            for (int c = lane; c < nv; c += WAVE) dst[c] = fp8_row_convert(src[c], inv);
         }
     }
 }
@@ -931,7 +955,13 @@ extern "C" int moe_quantize_rows_fp8(const void* x_bf16, int rows, int cols, uin
     if (rows == 0) return MOE_OK;
     MOE_REQUIRE(x_bf16 && q && scale, MOE_ERR_INVALID, "quantize_rows_fp8: null pointer");
     const int blocks = min(ceil_div(rows, 4), 65535 * 8);
-    quantize_rows_fp8_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>((const bf16_t*)x_bf16, rows, cols, q, scale, n_rows_dev);
+    hipStream_t s = (hipStream_t)stream;
+    const int nv = ceil_div(cols / 8, WAVE);  // 16-byte vectors per lane
+    if (nv <= 2) quantize_rows_fp8_kernel<2><<<blocks, 256, 0, s>>>((const bf16_t*)x_bf16, rows, cols, q, scale, n_rows_dev);
+    else if (nv <= 4) quantize_rows_fp8_kernel<4><<<blocks, 256, 0, s>>>((const bf16_t*)x_bf16, rows, cols, q, scale, n_rows_dev);
+    else if (nv <= 8) quantize_rows_fp8_kernel<8><<<blocks, 256, 0, s>>>((const bf16_t*)x_bf16, rows, cols, q, scale, n_rows_dev);
+    else if (nv <= 16) quantize_rows_fp8_kernel<16><<<blocks, 256, 0, s>>>((const bf16_t*)x_bf16, rows, cols, q, scale, n_rows_dev);
+    else quantize_rows_fp8_kernel<0><<<blocks, 256, 0, s>>>((const bf16_t*)x_bf16, rows, cols, q, scale, n_rows_dev);
     return moe_check_launch("quantize_rows_fp8");
 }
 
