@@ -68,6 +68,9 @@ def main():
     ap.add_argument("--config", default="mixtral")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay timing")
+    ap.add_argument("--unfused", action="store_true",
+                    help="run the destination side as unpack + MLP + return pack (the reference's operator split) "
+                         "instead of gathering / scattering inside the GEMMs")
     ap.add_argument("--cpu-sample-tokens", type=int, default=0, help="0 = sized for roughly 10-30 s")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -90,7 +93,7 @@ def main():
     # ---- untimed set-up: W seeded shards routed and packed, rank 0's receive buffer assembled
     world = harness.build_world(cfg, dev)
     ew, raw, qs = harness.expert_weights(cfg, 0, dev)
-    pipe = DispatchPipeline(world, ew)
+    pipe = DispatchPipeline(world, ew, fused=False if args.unfused else None)
     # the returned buffer: slot 0 is rank 0's own return slot; the other slots stand in for what the
     # other ranks' experts would send back (same shape and dtype, arbitrary finite contents)
     pipe.step()
@@ -183,6 +186,7 @@ def main():
         "routed_rows_per_s": round(cfg.tokens * cfg.topk / (ms_per_step * 1e-3), 1),
         "host_wall_ms_per_step": round(wall * 1e3 / args.steps, 4),
         "launch": launch,
+        "destination_side": "gather/scatter inside the GEMMs" if pipe.fused else "unpack + MLP + return pack",
         "ms_per_step_stream": round(stream_ms_per_step, 4),
         "ms_per_step_graph": None if ms_graph is None else round(ms_graph, 4),
         "roofline": roofline,

@@ -172,6 +172,28 @@ int moe_grouped_mlp_fp8(const void* tokens_bf16, const int32_t* expert_cnt, int 
                         const float* sd, uint8_t* xq_ws, float* xs_ws, void* h_ws, uint8_t* hq_ws, float* hs_ws,
                         void* out, moe_stream_t stream);
 
+/* ---- a10 + a11/a12 + a13 without the two row copies ------------------------------------------------
+ * The expert-major unpack (token_shuffle.py:31-56) and the return pack only move rows; the grouped GEMM
+ * can read its input rows where the transfer left them and write its result rows where the way back
+ * wants them.  Three entry points make that path:
+ *   moe_recv_row_map        row_map[r] = row of the [W,M,H] receive buffer that holds expert-major row r
+ *                           (r < n_rows; rows past the received total map to row 0), expert_cnt (nullable)
+ *                           as in moe_unpack_expert_major; map_ws >= moe_recv_map_ints(W,E_l,n_rows) ints.
+ *                           The same map is the destination of result row r in the returned buffer.
+ *   moe_grouped_gemm_mapped moe_grouped_gemm_packed with row indirection: logical row r is read from row
+ *                           a_row_map[r] of a_base (a_rows rows of K, under 4 GiB) and written to row
+ *                           c_row_map[r] of out (out_rows rows of N); either map may be NULL (identity).
+ *                           Map entries must lie inside their buffers.
+ *   moe_zero_padding_rows   rows [sum_e recv_counts[s,e], M) of every slot s of buf [W,M,H] <- 0: what
+ *                           moe_return_pack writes besides the result rows. */
+int moe_recv_row_map(const int32_t* recv_counts, int W, int E_l, int M, int n_rows, int32_t* row_map,
+                     int32_t* expert_cnt, int32_t* map_ws, moe_stream_t stream);
+int moe_grouped_gemm_mapped(const void* a_base, int a_rows, const int32_t* a_row_map, const void* packed,
+                            const int32_t* expert_cnt, int S_rows, int K, int N, int E_l, int act, void* out,
+                            int out_rows, const int32_t* c_row_map, moe_stream_t stream);
+int moe_zero_padding_rows(void* buf, int dtype, int W, int M, int H, const int32_t* recv_counts, int E_l,
+                          moe_stream_t stream);
+
 /* ---- a13: return path and combine (not in the reference; defined by the task statement) -------
  * ret[s, expert_offs_s[e]+j, :] = y[off[e,s]+j, :], zero padding: the [W,M,H] buffer this rank
  * sends back, slot s in the order source s sent its rows. */

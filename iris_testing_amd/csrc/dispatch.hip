@@ -415,6 +415,42 @@ struct RecvTables {
 };
 // map_ws layout for the recv-driven entry points: [n_out map][tables]
 // three prefix tables plus room for a transposed copy of the counts
+// Expert-major row r of the receive side -> row of the [W,M,H] buffer that holds it (one thread per row,
+// binary search in the (expert, source)-major prefix).  The same index serves the way back: the result
+// row of r returns to the slot its input came from.  Rows past the received total map to row 0.
+__global__ __launch_bounds__(256) void row_map_kernel(const int32_t* __restrict__ row_off, const int32_t* __restrict__ src_off,
+                                                       int W, int E_l, int M, int n_rows, int32_t* __restrict__ map) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= n_rows) return;
+    const int n = W * E_l;
+    if (r >= row_off[n]) { map[r] = 0; return; }
+    int lo = 0, hi = n;  // row_off[0] = 0 <= r; the last of a run of equal offsets owns the row
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (row_off[mid] <= r) lo = mid; else hi = mid;
+    }
+    const int e = lo / W, s = lo % W;
+    const int m = src_off[s * E_l + e] + (r - row_off[lo]);
+    map[r] = s * M + min(m, M - 1);
+}
+
+// rows [size_s, M) of every slot s of a [W,M,row] buffer <- 0, size_s = sum over e of rc[s,e] (one wave per row)
+__global__ __launch_bounds__(256) void zero_padding_rows_kernel(u32x4* __restrict__ buf, const int32_t* __restrict__ rc, int W,
+                                                                 int E_l, int M, int row_vecs) {
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const int r = blockIdx.x * (blockDim.x / WAVE) + wave;
+    if (r >= W * M) return;
+    const int s = r / M, m = r % M;
+    int size = 0;
+    for (int e = lane; e < E_l; e += WAVE) size += rc[s * E_l + e];
+#pragma unroll
+    for (int off = WAVE / 2; off >= 1; off >>= 1) size += __shfl_xor(size, off, WAVE);
+    if (m < size) return;
+    u32x4* row = buf + (size_t)r * row_vecs;
+    const u32x4 z = {0u, 0u, 0u, 0u};
+    for (int c = lane; c < row_vecs; c += WAVE) __builtin_nontemporal_store(z, row + c);
+}
+
 size_t recv_tables_ints(int W, int E_l) { return (size_t)3 * (W * E_l + 1) + (size_t)W * E_l; }
 
 int check_rows(const char* who, int dtype, int H) {
@@ -557,6 +593,34 @@ extern "C" int moe_unpack_expert_major(const void* recv, int dtype, int W, int M
     MOE_REQUIRE(M >= 1, MOE_ERR_INVALID, "unpack_expert_major: M=%d", M);
     return recv_driven("unpack_expert_major", SRC_UNPACK, recv, shuffled, dtype, H, recv_counts, W, E_l, M, 1, S_rows, nullptr,
                        expert_cnt, map_ws, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int moe_recv_row_map(const int32_t* recv_counts, int W, int E_l, int M, int n_rows, int32_t* row_map,
+                                int32_t* expert_cnt, int32_t* map_ws, moe_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    MOE_REQUIRE(W > 0 && E_l > 0 && W * E_l <= MOE_MAX_EXPERTS, MOE_ERR_INVALID, "recv_row_map: bad W=%d E_l=%d", W, E_l);
+    MOE_REQUIRE(M >= 1 && n_rows >= 0 && recv_counts && map_ws, MOE_ERR_INVALID, "recv_row_map: bad arguments");
+    const int n = W * E_l;
+    int32_t* src_off = map_ws;
+    int32_t* row_off = map_ws + (n + 1);
+    int32_t* flat_off = map_ws + 2 * (n + 1);
+    recv_tables_kernel<<<1, WAVE, 0, s>>>(recv_counts, W, E_l, src_off, row_off, flat_off, nullptr, expert_cnt);
+    if (n_rows > 0) {
+        MOE_REQUIRE(row_map, MOE_ERR_INVALID, "recv_row_map: null pointer");
+        row_map_kernel<<<ceil_div(n_rows, 256), 256, 0, s>>>(row_off, src_off, W, E_l, M, n_rows, row_map);
+    }
+    return moe_check_launch("recv_row_map");
+}
+
+extern "C" int moe_zero_padding_rows(void* buf, int dtype, int W, int M, int H, const int32_t* recv_counts, int E_l,
+                                     moe_stream_t stream) {
+    int rc = check_rows("zero_padding_rows", dtype, H);
+    if (rc) return rc;
+    MOE_REQUIRE(W > 0 && E_l > 0 && M >= 1 && buf && recv_counts, MOE_ERR_INVALID, "zero_padding_rows: bad arguments");
+    MOE_REQUIRE((long long)W * M < (1ll << 31), MOE_ERR_UNSUPPORTED, "zero_padding_rows: too many rows");
+    zero_padding_rows_kernel<<<ceil_div(W * M, 4), 256, 0, (hipStream_t)stream>>>((u32x4*)buf, recv_counts, W, E_l, M,
+                                                                                  H * dtype_size(dtype) / 16);
+    return moe_check_launch("zero_padding_rows");
 }
 
 // token_buf -> shuffled: pca is [E_l,W]; the tables kernel wants [W,E_l] counts, so transpose first.

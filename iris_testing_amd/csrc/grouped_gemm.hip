@@ -43,6 +43,8 @@ struct GemmParams {
     const float* row_scale;   // fp8: [S_rows] per-row activation scale
     const float* col_scale;   // fp8: [E_l, ncs] per-output-channel scale (gate for SwiGLU)
     const float* col_scale2;  // fp8 SwiGLU: [E_l, ncs] up scales
+    const int32_t* a_map;     // optional: logical row -> row of A (gather while loading), else A is row r itself
+    const int32_t* c_map;     // optional: logical row -> row of C (scatter while storing)
     int E_l, K, N, Npad, ldc, S_rows, ncs;
 };
 
@@ -290,10 +292,13 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     const uint32_t b_off0 = (uint32_t)lrow * ROWB + lchunk * 16;
 
 #define GG_TILE_PTRS(t, Ab_, Bb_, aoff_)                                                                   \
-    const uint8_t* Ab_ = p.A + (size_t)(t).row0 * p.K * ES;                                                 \
+    const uint8_t* Ab_ = p.a_map ? p.A : p.A + (size_t)(t).row0 * p.K * ES;                                 \
     const uint8_t* Bb_ = p.B + (size_t)(t).g * p.Npad * p.K * ES + (size_t)(t).nt * BN * ROWB;               \
     uint32_t aoff_[RA];                                                                                     \
-    _Pragma("unroll") for (int r = 0; r < RA; ++r) aoff_[r] = (uint32_t)min(r * LR + lrow, (t).rv - 1) * ldk + lchunk * 16;
+    _Pragma("unroll") for (int r = 0; r < RA; ++r) {                                                         \
+        const int lr_ = max(min(r * LR + lrow, (t).rv - 1), 0);  /* tile row this lane fetches, clamped */     \
+        aoff_[r] = (uint32_t)(p.a_map ? p.a_map[(t).row0 + lr_] : lr_) * ldk + lchunk * 16;                   \
+    }
     // load d (0 .. LPS-1) of one stage: A rounds first, then B rounds
 #define GG_LD(d, ap_, bp_, aoff_, slot)                                                                       \
     do {                                                                                                      \
@@ -531,7 +536,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             const size_t grow = (size_t)(row0 + (ok ? r : 0));
             float rs = 1.f;
             if constexpr (FP8) rs = p.row_scale[grow];
-            bf16_t* crow = C + grow * p.ldc;
+            bf16_t* crow = C + (p.c_map ? (size_t)p.c_map[grow] : grow) * p.ldc;
 #pragma unroll
             for (int j = 0; j < TN; j += (EPI == EPI_SWIGLU ? 2 : 1)) {
 #pragma unroll
@@ -912,6 +917,26 @@ extern "C" int moe_grouped_gemm_packed(const void* tokens, const void* packed, c
     MOE_REQUIRE(tokens && packed && expert_cnt && out, MOE_ERR_INVALID, "grouped_gemm_packed: null pointer");
     GemmParams p{};
     p.A = (const uint8_t*)tokens; p.B = (const uint8_t*)packed; p.C = out; p.cnt = expert_cnt;
+    p.E_l = E_l; p.K = K; p.N = N; p.ldc = N; p.S_rows = S_rows;
+    p.Npad = round_up(act == EPI_SWIGLU ? 2 * N : N, GG_BN);
+    return launch_gemm<false>(p, act, (hipStream_t)stream);
+}
+
+extern "C" int moe_grouped_gemm_mapped(const void* a_base, int a_rows, const int32_t* a_row_map, const void* packed,
+                                       const int32_t* expert_cnt, int S_rows, int K, int N, int E_l, int act, void* out,
+                                       int out_rows, const int32_t* c_row_map, moe_stream_t stream) {
+    MOE_REQUIRE(S_rows >= 0 && K > 0 && N > 0 && E_l > 0 && E_l <= GG_MAXG, MOE_ERR_INVALID, "grouped_gemm_mapped: bad shape");
+    MOE_REQUIRE(act >= EPI_NONE && act <= EPI_SWIGLU, MOE_ERR_INVALID, "grouped_gemm_mapped: activation %d", act);
+    MOE_REQUIRE(K % 64 == 0 && N % 8 == 0, MOE_ERR_UNSUPPORTED, "grouped_gemm_mapped: needs K %% 64 == 0 and N %% 8 == 0 (K=%d N=%d)", K, N);
+    MOE_REQUIRE(a_rows >= 0 && out_rows >= 0, MOE_ERR_INVALID, "grouped_gemm_mapped: negative buffer rows");
+    // gathered rows are addressed with 32-bit byte offsets from a_base
+    MOE_REQUIRE(!a_row_map || (unsigned long long)a_rows * (unsigned long long)K * 2ull < (1ull << 32), MOE_ERR_UNSUPPORTED,
+                "grouped_gemm_mapped: the gathered buffer must be smaller than 4 GiB (%d rows of %d)", a_rows, K);
+    if (S_rows == 0) return MOE_OK;
+    MOE_REQUIRE(a_base && packed && expert_cnt && out, MOE_ERR_INVALID, "grouped_gemm_mapped: null pointer");
+    GemmParams p{};
+    p.A = (const uint8_t*)a_base; p.B = (const uint8_t*)packed; p.C = out; p.cnt = expert_cnt;
+    p.a_map = a_row_map; p.c_map = c_row_map;
     p.E_l = E_l; p.K = K; p.N = N; p.ldc = N; p.S_rows = S_rows;
     p.Npad = round_up(act == EPI_SWIGLU ? 2 * N : N, GG_BN);
     return launch_gemm<false>(p, act, (hipStream_t)stream);

@@ -322,6 +322,54 @@ def return_pack(y: torch.Tensor, recv_counts: torch.Tensor, M: int, out: Optiona
     return out
 
 
+# ---- destination side without the two row copies ------------------------------------------------
+def recv_row_map(recv_counts: torch.Tensor, M: int, n_rows: int, row_map: Optional[torch.Tensor] = None,
+                 expert_cnt: Optional[torch.Tensor] = None, map_ws=None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """row_map[r] = row of the flattened [W*M,H] receive buffer holding expert-major row r, and the
+    per-expert row counts (what unpack_expert_major returns beside the rows)."""
+    _req_i32(recv_counts, "recv_counts")
+    W, E_l = recv_counts.shape
+    dev = recv_counts.device
+    if row_map is None:
+        row_map = _i32((max(n_rows, 1),), dev)
+    if expert_cnt is None:
+        expert_cnt = _i32((E_l,), dev)
+    ws = _map_ws(W, E_l, n_rows, dev, map_ws)
+    L.check(L.lib().moe_recv_row_map(L.ptr(recv_counts), W, E_l, M, n_rows, L.ptr(row_map), L.ptr(expert_cnt), L.ptr(ws),
+                                     L.stream_ptr()))
+    return row_map, expert_cnt
+
+
+def grouped_gemm_mapped(a_base: torch.Tensor, a_row_map: Optional[torch.Tensor], packed: torch.Tensor,
+                        expert_cnt: torch.Tensor, S_rows: int, N: int, act: str, out: torch.Tensor,
+                        c_row_map: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """grouped_gemm_packed with row indirection on the way in (a_base rows a_row_map[r]) and / or on the
+    way out (out rows c_row_map[r]).  a_base and out are 2-D views [rows, K] / [rows, N]."""
+    _req_cuda(a_base, "a_base")
+    _req_i32(expert_cnt, "expert_cnt")
+    assert a_base.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and a_base.dim() == 2 and out.dim() == 2
+    assert a_base.is_contiguous() and out.is_contiguous() and out.shape[1] == N
+    for m, name in ((a_row_map, "a_row_map"), (c_row_map, "c_row_map")):
+        if m is not None:
+            _req_i32(m, name)
+            assert m.numel() >= S_rows, f"{name} must cover S_rows"
+    L.check(L.lib().moe_grouped_gemm_mapped(L.ptr(a_base), a_base.shape[0], L.ptr(a_row_map) if a_row_map is not None else None,
+                                            L.ptr(packed), L.ptr(expert_cnt), S_rows, a_base.shape[1], N, expert_cnt.numel(),
+                                            L.ACT[act], L.ptr(out), out.shape[0],
+                                            L.ptr(c_row_map) if c_row_map is not None else None, L.stream_ptr()))
+    return out
+
+
+def zero_padding_rows(buf: torch.Tensor, recv_counts: torch.Tensor) -> torch.Tensor:
+    """Zero the rows of a [W,M,H] buffer that lie past what each slot received."""
+    _req_cuda(buf, "buf")
+    _req_i32(recv_counts, "recv_counts")
+    W, M, H = buf.shape
+    L.check(L.lib().moe_zero_padding_rows(L.ptr(buf), L.dtype_code(buf.dtype), W, M, H, L.ptr(recv_counts),
+                                          recv_counts.shape[1], L.stream_ptr()))
+    return buf
+
+
 def combine(ret: torch.Tensor, topk_idx: torch.Tensor, pos: torch.Tensor, gate: torch.Tensor,
             dst_offsets: torch.Tensor, e_local: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     _req_cuda(ret, "ret")

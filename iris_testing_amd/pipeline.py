@@ -4,6 +4,9 @@ A step = what rank 0 does for one batch:
   as a source       route + top-k  ->  counts / offsets / positions  ->  pack into [W,M,H]
   as a destination  expert-major unpack of its receive buffer  ->  grouped expert MLP  ->  return pack
   as a source       top-k-weighted combine of the returned buffer into token order
+With ``fused=True`` (bf16 experts) the destination side skips the two row copies: "unpack" only builds the
+row map, the first GEMM gathers its input rows from the receive buffer, the second scatters its result rows
+into the returned layout, and "return_pack" only zeroes the padding rows.
 The two transfers in between are not part of a one-GPU build: the receive buffer and the returned
 buffer are assembled beforehand (harness.build_world) and stay fixed.  Each stage is one C-ABI call
 on the current stream; no stage synchronises or allocates.
@@ -22,8 +25,14 @@ STAGES = ["route", "count", "pack", "unpack", "mlp_up", "mlp_down", "return_pack
 
 
 class DispatchPipeline:
-    def __init__(self, world: World, weights: ExpertWeights, returned: Optional[torch.Tensor] = None):
+    def __init__(self, world: World, weights: ExpertWeights, returned: Optional[torch.Tensor] = None,
+                 fused: Optional[bool] = None):
         cfg = world.cfg
+        # gather / scatter inside the GEMMs needs the bf16 MFMA path and a receive buffer under 4 GiB
+        can_fuse = weights.dtype == torch.bfloat16 and world.recv.numel() * world.recv.element_size() < (1 << 32)
+        self.fused = can_fuse if fused is None else bool(fused)
+        if self.fused and not can_fuse:
+            raise ValueError("the fused destination path needs bf16 expert weights and a receive buffer under 4 GiB")
         self.world, self.cfg, self.weights = world, cfg, weights
         dev = world.x0.device
         T, H, E, k, W, E_l, F = cfg.tokens, cfg.hidden, cfg.experts, cfg.topk, cfg.world, cfg.e_local, cfg.ffn
@@ -51,6 +60,7 @@ class DispatchPipeline:
         self.y = torch.zeros((S, H), dtype=dt, device=dev)
         self.ret = torch.empty((W, M, H), dtype=dt, device=dev)
         self.ret_map = i32(lib.moe_recv_map_ints(W, E_l, W * M))
+        self.row_map = i32(max(S, 1))
         if weights.dtype == torch.uint8:
             self.xq = torch.empty((S, H), dtype=torch.uint8, device=dev)
             self.xs = torch.empty((S,), dtype=torch.float32, device=dev)
@@ -82,6 +92,10 @@ class DispatchPipeline:
 
     def unpack(self, s):
         c, w = self.cfg, self.world
+        if self.fused:
+            L.check(L.lib().moe_recv_row_map(self._p(w.recv_counts), c.world, c.e_local, w.M, self.S, self._p(self.row_map),
+                                             self._p(self.expert_cnt), self._p(self.unpack_map), s))
+            return
         L.check(L.lib().moe_unpack_expert_major(self._p(w.recv), self.code, c.world, w.M, c.hidden, self._p(w.recv_counts),
                                                 c.e_local, self._p(self.rows), self.S, self._p(self.expert_cnt),
                                                 self._p(self.unpack_map), s))
@@ -100,18 +114,32 @@ class DispatchPipeline:
             L.check(lib.moe_grouped_mlp(self._p(self.rows), self._p(self.expert_cnt), self.code, self.S, c.hidden, c.ffn,
                                         c.e_local, L.ACT[ew.act], self._p(ew.w1), self._p(ew.w_up), self._p(ew.w2),
                                         self._p(self.hidden), self._p(self.y), s))
+        elif self.fused:
+            w = self.world
+            L.check(lib.moe_grouped_gemm_mapped(self._p(w.recv), c.world * w.M, self._p(self.row_map), self._p(ew.w1),
+                                                self._p(self.expert_cnt), self.S, c.hidden, c.ffn, c.e_local, L.ACT[ew.act],
+                                                self._p(self.hidden), self.S, None, s))
         else:
             L.check(lib.moe_grouped_gemm_packed(self._p(self.rows), self._p(ew.w1), self._p(self.expert_cnt), self.S, c.hidden,
                                                 c.ffn, c.e_local, L.ACT[ew.act], self._p(self.hidden), s))
 
     def mlp_down(self, s):
         c, ew = self.cfg, self.weights
-        if ew.dtype == torch.bfloat16:
+        if ew.dtype == torch.bfloat16 and self.fused:
+            w = self.world
+            L.check(L.lib().moe_grouped_gemm_mapped(self._p(self.hidden), self.S, None, self._p(ew.w2), self._p(self.expert_cnt),
+                                                    self.S, c.ffn, c.hidden, c.e_local, 0, self._p(self.ret), c.world * w.M,
+                                                    self._p(self.row_map), s))
+        elif ew.dtype == torch.bfloat16:
             L.check(L.lib().moe_grouped_gemm_packed(self._p(self.hidden), self._p(ew.w2), self._p(self.expert_cnt), self.S,
                                                     c.ffn, c.hidden, c.e_local, 0, self._p(self.y), s))
 
     def return_pack(self, s):
         c, w = self.cfg, self.world
+        if self.fused:
+            L.check(L.lib().moe_zero_padding_rows(self._p(self.ret), self.code, c.world, w.M, c.hidden, self._p(w.recv_counts),
+                                                  c.e_local, s))
+            return
         L.check(L.lib().moe_return_pack(self._p(self.y), self.code, self.S, c.hidden, self._p(w.recv_counts), c.world,
                                         c.e_local, w.M, self._p(self.ret), self._p(self.ret_map), s))
 
@@ -161,11 +189,18 @@ class DispatchPipeline:
         else:
             mlp = {"mlp_up": dict(bound="mfma", amount=2 * S * H * F * up_mats),
                    "mlp_down": dict(bound="mfma", amount=2 * S * F * H)}
+        if self.fused:
+            # the row copies are gone: what is left of the two stages is the row map and the padding rows
+            unpack = dict(bound="hbm", amount=S * 4 + W * c.e_local * 4)
+            ret = dict(bound="hbm", amount=max(W * M - S, 0) * H * B)
+        else:
+            unpack = dict(bound="hbm", amount=2 * S * H * B)
+            ret = dict(bound="hbm", amount=S * H * B + W * M * H * B)
         return {
             "route": dict(bound="hbm", amount=T * H * B + H * E * B + T * k * 8),
             "pack": dict(bound="hbm", amount=T * H * B + W * M * H * B),
-            "unpack": dict(bound="hbm", amount=2 * S * H * B),
+            "unpack": unpack,
             **mlp,
-            "return_pack": dict(bound="hbm", amount=S * H * B + W * M * H * B),
+            "return_pack": ret,
             "combine": dict(bound="hbm", amount=T * k * H * B + T * H * B + T * k * 8),
         }

@@ -59,19 +59,19 @@ def test_dispatch_expert_combine_matches_dense(name):
     assert mx_rms < tol * 4, f"end-to-end error {mx_rms} of rms"
 
 
-@pytest.mark.parametrize("name", ["small", "zipf_k1"])
-def test_graph_replay_equals_eager(name):
+@pytest.mark.parametrize("name,fused", [("small", False), ("small", True), ("zipf_k1", False)])
+def test_graph_replay_equals_eager(name, fused):
     """The whole step captured as one HIP graph: every replay (with eager work and synchronisation in
     between, and outputs cleared before each replay) must reproduce the eager step bit for bit."""
     from iris_testing_amd.pipeline import DispatchPipeline
     cfg = CONFIGS[name]
     world = harness.build_world(cfg, DEV)
     ew, _, _ = harness.expert_weights(cfg, 0, DEV)
-    pipe = DispatchPipeline(world, ew)
+    pipe = DispatchPipeline(world, ew, fused=fused)
     pipe.returned.copy_(torch.randn(pipe.returned.shape, device=DEV).to(pipe.returned.dtype))
     pipe.step()
     torch.cuda.synchronize()
-    names = ["idx", "gate", "send_counts", "pos", "send", "rows", "y", "ret", "out"]
+    names = ["idx", "gate", "send_counts", "pos", "send", "ret", "out"] + (["row_map"] if fused else ["rows", "y"])
     eager = {n: getattr(pipe, n).clone() for n in names}
     graph = pipe.capture()
     for rep in range(3):
