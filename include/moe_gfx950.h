@@ -193,6 +193,14 @@ int moe_grouped_gemm_mapped(const void* a_base, int a_rows, const int32_t* a_row
                             int out_rows, const int32_t* c_row_map, moe_stream_t stream);
 int moe_zero_padding_rows(void* buf, int dtype, int W, int M, int H, const int32_t* recv_counts, int E_l,
                           moe_stream_t stream);
+/* moe_grouped_mlp_fp8 with the same row indirection: the row quantisation reads input row r from row
+ * a_row_map[r] of a_base_bf16 (a_rows rows of H), the down GEMM writes result row r to row c_row_map[r]
+ * of out (out_rows rows of H); either map may be NULL. */
+int moe_grouped_mlp_fp8_mapped(const void* a_base_bf16, int a_rows, const int32_t* a_row_map,
+                               const int32_t* expert_cnt, int S_rows, int H, int F, int E_l,
+                               const uint8_t* wgu_packed, const float* sg, const float* su, const uint8_t* wd_packed,
+                               const float* sd, uint8_t* xq_ws, float* xs_ws, void* h_ws, uint8_t* hq_ws, float* hs_ws,
+                               void* out, int out_rows, const int32_t* c_row_map, moe_stream_t stream);
 
 /* ---- a13: return path and combine (not in the reference; defined by the task statement) -------
  * ret[s, expert_offs_s[e]+j, :] = y[off[e,s]+j, :], zero padding: the [W,M,H] buffer this rank

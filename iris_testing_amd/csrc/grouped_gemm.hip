@@ -764,12 +764,13 @@ __device__ __forceinline__ uint2 fp8_row_convert(const uint4& v, float inv) {
 template <int NV>  // 16-byte vectors per lane kept in registers (0: stream the row twice)
 __global__ __launch_bounds__(256) void quantize_rows_fp8_kernel(const bf16_t* __restrict__ x, int rows, int cols,
                                                                  uint8_t* __restrict__ q, float* __restrict__ scale,
-                                                                 const int32_t* __restrict__ n_rows_dev) {
+                                                                 const int32_t* __restrict__ n_rows_dev,
+                                                                 const int32_t* __restrict__ src_map) {
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const int limit = n_rows_dev ? min(rows, *n_rows_dev) : rows;
     const int nv = cols / 8;
     for (int r = blockIdx.x * 4 + wave; r < limit; r += gridDim.x * 4) {
-        const uint4* src = (const uint4*)(x + (size_t)r * cols);
+        const uint4* src = (const uint4*)(x + (size_t)(src_map ? src_map[r] : r) * cols);
         uint4 held[NV > 0 ? NV : 1];
         float amax = 0.f;
         if constexpr (NV > 0) {
@@ -974,43 +975,62 @@ extern "C" int moe_grouped_mlp(const void* tokens, const int32_t* expert_cnt, in
     return launch_gemm<false>(q, EPI_NONE, s);
 }
 
+static int launch_quantize(const void* x_bf16, const int32_t* src_map, int rows, int cols, uint8_t* q, float* scale,
+                           const int32_t* n_rows_dev, hipStream_t s) {
+    const int blocks = min(ceil_div(rows, 4), 65535 * 8);
+    const int nv = ceil_div(cols / 8, WAVE);  // 16-byte vectors per lane
+#define GG_Q(NVv) quantize_rows_fp8_kernel<NVv><<<blocks, 256, 0, s>>>((const bf16_t*)x_bf16, rows, cols, q, scale, n_rows_dev, src_map)
+    if (nv <= 2) GG_Q(2);
+    else if (nv <= 4) GG_Q(4);
+    else if (nv <= 8) GG_Q(8);
+    else if (nv <= 16) GG_Q(16);
+    else GG_Q(0);
+#undef GG_Q
+    return moe_check_launch("quantize_rows_fp8");
+}
+
 extern "C" int moe_quantize_rows_fp8(const void* x_bf16, int rows, int cols, uint8_t* q, float* scale,
                                      const int32_t* n_rows_dev, moe_stream_t stream) {
     MOE_REQUIRE(rows >= 0 && cols > 0 && cols % 8 == 0, MOE_ERR_INVALID, "quantize_rows_fp8: cols must be a multiple of 8");
     if (rows == 0) return MOE_OK;
     MOE_REQUIRE(x_bf16 && q && scale, MOE_ERR_INVALID, "quantize_rows_fp8: null pointer");
-    const int blocks = min(ceil_div(rows, 4), 65535 * 8);
-    hipStream_t s = (hipStream_t)stream;
-    const int nv = ceil_div(cols / 8, WAVE);  // 16-byte vectors per lane
-    if (nv <= 2) quantize_rows_fp8_kernel<2><<<blocks, 256, 0, s>>>((const bf16_t*)x_bf16, rows, cols, q, scale, n_rows_dev);
-    else if (nv <= 4) quantize_rows_fp8_kernel<4><<<blocks, 256, 0, s>>>((const bf16_t*)x_bf16, rows, cols, q, scale, n_rows_dev);
-    else if (nv <= 8) quantize_rows_fp8_kernel<8><<<blocks, 256, 0, s>>>((const bf16_t*)x_bf16, rows, cols, q, scale, n_rows_dev);
-    else if (nv <= 16) quantize_rows_fp8_kernel<16><<<blocks, 256, 0, s>>>((const bf16_t*)x_bf16, rows, cols, q, scale, n_rows_dev);
-    else quantize_rows_fp8_kernel<0><<<blocks, 256, 0, s>>>((const bf16_t*)x_bf16, rows, cols, q, scale, n_rows_dev);
-    return moe_check_launch("quantize_rows_fp8");
+    return launch_quantize(x_bf16, nullptr, rows, cols, q, scale, n_rows_dev, (hipStream_t)stream);
 }
 
-extern "C" int moe_grouped_mlp_fp8(const void* tokens_bf16, const int32_t* expert_cnt, int S_rows, int H, int F, int E_l,
-                                   const uint8_t* wgu_packed, const float* sg, const float* su, const uint8_t* wd_packed,
-                                   const float* sd, uint8_t* xq_ws, float* xs_ws, void* h_ws, uint8_t* hq_ws, float* hs_ws,
-                                   void* out, moe_stream_t stream) {
+extern "C" int moe_grouped_mlp_fp8_mapped(const void* a_base_bf16, int a_rows, const int32_t* a_row_map,
+                                          const int32_t* expert_cnt, int S_rows, int H, int F, int E_l,
+                                          const uint8_t* wgu_packed, const float* sg, const float* su,
+                                          const uint8_t* wd_packed, const float* sd, uint8_t* xq_ws, float* xs_ws, void* h_ws,
+                                          uint8_t* hq_ws, float* hs_ws, void* out, int out_rows, const int32_t* c_row_map,
+                                          moe_stream_t stream) {
     hipStream_t s = (hipStream_t)stream;
     MOE_REQUIRE(S_rows >= 0 && H > 0 && F > 0 && E_l > 0 && E_l <= GG_MAXG, MOE_ERR_INVALID, "grouped_mlp_fp8: bad shape");
     MOE_REQUIRE(H % 128 == 0 && F % 128 == 0, MOE_ERR_UNSUPPORTED, "grouped_mlp_fp8: needs H, F multiples of 128 (H=%d F=%d)", H, F);
+    MOE_REQUIRE(a_rows >= 0 && out_rows >= 0, MOE_ERR_INVALID, "grouped_mlp_fp8: negative buffer rows");
     if (S_rows == 0) return MOE_OK;
-    MOE_REQUIRE(tokens_bf16 && expert_cnt && wgu_packed && sg && su && wd_packed && sd && xq_ws && xs_ws && h_ws && hq_ws &&
+    MOE_REQUIRE(a_base_bf16 && expert_cnt && wgu_packed && sg && su && wd_packed && sd && xq_ws && xs_ws && h_ws && hq_ws &&
                     hs_ws && out, MOE_ERR_INVALID, "grouped_mlp_fp8: null pointer");
-    int rc = moe_quantize_rows_fp8(tokens_bf16, S_rows, H, xq_ws, xs_ws, nullptr, stream);
+    // the row quantisation reads every input row once anyway: with a map it reads it where the transfer left it
+    int rc = launch_quantize(a_base_bf16, a_row_map, S_rows, H, xq_ws, xs_ws, nullptr, s);
     if (rc) return rc;
     GemmParams p{};
     p.A = xq_ws; p.B = wgu_packed; p.C = h_ws; p.cnt = expert_cnt; p.row_scale = xs_ws; p.col_scale = sg; p.col_scale2 = su;
     p.E_l = E_l; p.K = H; p.N = F; p.Npad = round_up(2 * F, GG_BN); p.ldc = F; p.S_rows = S_rows; p.ncs = F;
     rc = launch_gemm<true>(p, EPI_SWIGLU, s);
     if (rc) return rc;
-    rc = moe_quantize_rows_fp8(h_ws, S_rows, F, hq_ws, hs_ws, nullptr, stream);
+    rc = launch_quantize(h_ws, nullptr, S_rows, F, hq_ws, hs_ws, nullptr, s);
     if (rc) return rc;
     GemmParams q{};
     q.A = hq_ws; q.B = wd_packed; q.C = out; q.cnt = expert_cnt; q.row_scale = hs_ws; q.col_scale = sd;
+    q.c_map = c_row_map;
     q.E_l = E_l; q.K = F; q.N = H; q.Npad = round_up(H, GG_BN); q.ldc = H; q.S_rows = S_rows; q.ncs = H;
     return launch_gemm<true>(q, EPI_NONE, s);
+}
+
+extern "C" int moe_grouped_mlp_fp8(const void* tokens_bf16, const int32_t* expert_cnt, int S_rows, int H, int F, int E_l,
+                                   const uint8_t* wgu_packed, const float* sg, const float* su, const uint8_t* wd_packed,
+                                   const float* sd, uint8_t* xq_ws, float* xs_ws, void* h_ws, uint8_t* hq_ws, float* hs_ws,
+                                   void* out, moe_stream_t stream) {
+    return moe_grouped_mlp_fp8_mapped(tokens_bf16, S_rows, nullptr, expert_cnt, S_rows, H, F, E_l, wgu_packed, sg, su, wd_packed,
+                                      sd, xq_ws, xs_ws, h_ws, hq_ws, hs_ws, out, S_rows, nullptr, stream);
 }

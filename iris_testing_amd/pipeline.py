@@ -4,7 +4,7 @@ A step = what rank 0 does for one batch:
   as a source       route + top-k  ->  counts / offsets / positions  ->  pack into [W,M,H]
   as a destination  expert-major unpack of its receive buffer  ->  grouped expert MLP  ->  return pack
   as a source       top-k-weighted combine of the returned buffer into token order
-With ``fused=True`` (bf16 experts) the destination side skips the two row copies: "unpack" only builds the
+With ``fused=True`` (bf16 or fp8 experts) the destination side skips the two row copies: "unpack" only builds the
 row map, the first GEMM gathers its input rows from the receive buffer, the second scatters its result rows
 into the returned layout, and "return_pack" only zeroes the padding rows.
 The two transfers in between are not part of a one-GPU build: the receive buffer and the returned
@@ -29,10 +29,11 @@ class DispatchPipeline:
                  fused: Optional[bool] = None):
         cfg = world.cfg
         # gather / scatter inside the GEMMs needs the bf16 MFMA path and a receive buffer under 4 GiB
-        can_fuse = weights.dtype == torch.bfloat16 and world.recv.numel() * world.recv.element_size() < (1 << 32)
+        can_fuse = weights.dtype in (torch.bfloat16, torch.uint8) and \
+            world.recv.numel() * world.recv.element_size() < (1 << 32)
         self.fused = can_fuse if fused is None else bool(fused)
         if self.fused and not can_fuse:
-            raise ValueError("the fused destination path needs bf16 expert weights and a receive buffer under 4 GiB")
+            raise ValueError("the fused destination path needs bf16 or fp8 expert weights and a receive buffer under 4 GiB")
         self.world, self.cfg, self.weights = world, cfg, weights
         dev = world.x0.device
         T, H, E, k, W, E_l, F = cfg.tokens, cfg.hidden, cfg.experts, cfg.topk, cfg.world, cfg.e_local, cfg.ffn
@@ -106,6 +107,15 @@ class DispatchPipeline:
         if ew.dtype == torch.uint8:
             sg, su, sd = ew.scales
             # the fp8 entry point runs quantise + gate/up + quantise + down in one call
+            if self.fused:
+                w = self.world
+                L.check(lib.moe_grouped_mlp_fp8_mapped(self._p(w.recv), c.world * w.M, self._p(self.row_map),
+                                                       self._p(self.expert_cnt), self.S, c.hidden, c.ffn, c.e_local,
+                                                       self._p(ew.w1), self._p(sg), self._p(su), self._p(ew.w2), self._p(sd),
+                                                       self._p(self.xq), self._p(self.xs), self._p(self.hidden), self._p(self.hq),
+                                                       self._p(self.hs), self._p(self.ret), c.world * w.M,
+                                                       self._p(self.row_map), s))
+                return
             L.check(lib.moe_grouped_mlp_fp8(self._p(self.rows), self._p(self.expert_cnt), self.S, c.hidden, c.ffn, c.e_local,
                                             self._p(ew.w1), self._p(sg), self._p(su), self._p(ew.w2), self._p(sd),
                                             self._p(self.xq), self._p(self.xs), self._p(self.hidden), self._p(self.hq),

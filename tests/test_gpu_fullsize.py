@@ -87,7 +87,7 @@ def test_full_size_pipeline(name):
     assert_bits_equal(out1[:256], o_out, "combine (first 256 tokens)")
 
 
-@pytest.mark.parametrize("name", ["mixtral", "finegrained", "small"])
+@pytest.mark.parametrize("name", ["mixtral", "finegrained", "small", "zipf_k2"])
 def test_fused_destination_equals_copies(name):
     """The destination side without the two row copies (row map, gathering first GEMM, scattering second
     GEMM, zeroed padding rows) runs the same arithmetic on the same rows as unpack + MLP + return pack, so
