@@ -201,8 +201,8 @@ class DispatchPipeline:
                    "mlp_down": dict(bound="mfma", amount=2 * S * F * H)}
         if self.fused:
             # the row copies are gone: what is left of the two stages is the row map and the padding rows
-            unpack = dict(bound="hbm", amount=S * 4 + W * c.e_local * 4)
-            ret = dict(bound="hbm", amount=max(W * M - S, 0) * H * B)
+            unpack = dict(bound="latency", amount=S * 4 + W * c.e_local * 4)
+            ret = dict(bound="latency", amount=max(W * M - S, 0) * H * B)
         else:
             unpack = dict(bound="hbm", amount=2 * S * H * B)
             ret = dict(bound="hbm", amount=S * H * B + W * M * H * B)

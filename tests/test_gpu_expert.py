@@ -114,6 +114,49 @@ def test_expert_mlp(dtype, act, E_l, H, F, S):
     _check(out, want.astype(np.float64), r, a, f"expert_mlp {dtype} {act} E_l={E_l} H={H} F={F}")
 
 
+@pytest.mark.parametrize("E_l,K,N,S,act", [(3, 128, 264, 900, "none"), (4, 256, 512, 1500, "swiglu")])
+def test_grouped_gemm_mapped(E_l, K, N, S, act):
+    """Row indirection on both sides: logical row r is read from a scattered row of a larger buffer and its
+    result is written to a scattered row of a larger output.  The result must be bit for bit what the plain
+    kernel produces on the gathered rows (same arithmetic), rows outside the map stay untouched, and the
+    plain kernel itself is held to the oracle."""
+    from iris_testing_amd import _lib as L
+    rng = np.random.default_rng(K + N + E_l)
+    cnt = _groups(rng, E_l, S)
+    S_tot = int(cnt.sum())
+    n_in, n_out = S_tot + 500, S_tot + 300
+    a_map = rng.permutation(n_in)[:S_tot].astype(np.int32)
+    c_map = rng.permutation(n_out)[:S_tot].astype(np.int32)
+    base = _randn(rng, n_in, K)
+    w = _randn(rng, E_l, K, N, scale=K ** -0.5)
+    wu = _randn(rng, E_l, K, N, scale=K ** -0.5) if act == "swiglu" else None
+    packed = ops.prepack_weights(_t(w, "bf16"), None if wu is None else _t(wu, "bf16"))
+    cnt_t = torch.from_numpy(cnt).to(DEV)
+    base_t = _t(base, "bf16")
+    gathered = base_t[torch.from_numpy(a_map).long().to(DEV)].contiguous()
+    plain = torch.empty((S_tot, N), dtype=torch.bfloat16, device=DEV)
+    L.check(L.lib().moe_grouped_gemm_packed(L.ptr(gathered), L.ptr(packed), L.ptr(cnt_t), S_tot, K, N, E_l, L.ACT[act],
+                                            L.ptr(plain), L.stream_ptr()))
+    out = torch.full((n_out, N), -7.0, dtype=torch.bfloat16, device=DEV)
+    ops.grouped_gemm_mapped(base_t, torch.from_numpy(a_map).to(DEV), packed, cnt_t, S_tot, N, act, out,
+                            torch.from_numpy(c_map).to(DEV))
+    torch.cuda.synchronize()
+    got = out[torch.from_numpy(c_map).long().to(DEV)]
+    assert torch.equal(got.view(torch.int16), plain.view(torch.int16)), "mapped GEMM differs from the plain one"
+    untouched = np.setdiff1d(np.arange(n_out), c_map)
+    assert bool((out[torch.from_numpy(untouched).to(DEV)] == -7.0).all()), "rows outside the map were written"
+    if act == "none":
+        _check(to_np(plain), O.grouped_gemm(base[a_map], w, cnt, "bf16"), BF16_RTOL, BF16_ATOL, "gathered GEMM")
+    # argument checks happen before any launch
+    lib = L.lib()
+    rc = lib.moe_grouped_gemm_mapped(L.ptr(base_t), n_in, None, L.ptr(packed), L.ptr(cnt_t), S_tot, K + 8, N, E_l, 0,
+                                     L.ptr(out), n_out, None, L.stream_ptr())
+    assert rc != 0 and b"K" in lib.moe_last_error()
+    rc = lib.moe_grouped_gemm_mapped(L.ptr(base_t), 1 << 30, L.ptr(torch.from_numpy(a_map).to(DEV)), L.ptr(packed),
+                                     L.ptr(cnt_t), S_tot, K, N, E_l, 0, L.ptr(out), n_out, None, L.stream_ptr())
+    assert rc != 0 and b"4 GiB" in lib.moe_last_error()
+
+
 @pytest.mark.parametrize("R,C", [(5, 64), (300, 2048), (77, 1408)])
 def test_quantize_rows_fp8_bit_exact(R, C):
     rng = np.random.default_rng(R)
