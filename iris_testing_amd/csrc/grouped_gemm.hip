@@ -527,63 +527,69 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         }
 
         // ---- epilogue: acc -> (scales) -> activation -> bf16 -> C
+        // Column tiles outermost: the fp8 per-channel scales of a column tile are fetched once and serve
+        // the wave's TM row tiles.
         bf16_t* C = (bf16_t*)p.C;
         const int chalf = khalf * 4;
+        bool ok[TM];
+        bf16_t* crow[TM];
+        float rs[TM];
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             const int r = wm * (BM / NWM) + i * 32 + (lane & 31);
-            const bool ok = r < rv;
-            const size_t grow = (size_t)(row0 + (ok ? r : 0));
-            float rs = 1.f;
-            if constexpr (FP8) rs = p.row_scale[grow];
-            bf16_t* crow = C + (p.c_map ? (size_t)p.c_map[grow] : grow) * p.ldc;
+            ok[i] = r < rv;
+            const size_t grow = (size_t)(row0 + (ok[i] ? r : 0));
+            rs[i] = 1.f;
+            if constexpr (FP8) rs[i] = p.row_scale[grow];
+            crow[i] = C + (p.c_map ? (size_t)p.c_map[grow] : grow) * p.ldc;
+        }
 #pragma unroll
-            for (int j = 0; j < TN; j += (EPI == EPI_SWIGLU ? 2 : 1)) {
+        for (int j = 0; j < TN; j += (EPI == EPI_SWIGLU ? 2 : 1)) {
+            // first output column of this lane in the tile (SwiGLU: packed columns alternate gate/up in groups
+            // of 32, tile j = gate, j+1 = up, both land on output columns (packed column / 2))
+            const int colj = (EPI == EPI_SWIGLU ? ((nt * BN + wn * (BN / 2) + j * 32) >> 1) : nt * BN + wn * (BN / 2) + j * 32) + chalf;
+            float4 sc0[4], sc1[4];  // fp8: channel scales of the lane's 4 x 4 columns (gate / only; up)
+            if constexpr (FP8) {
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
+                    const int col = colj + 8 * q;
+                    sc0[q] = sc1[q] = make_float4(1.f, 1.f, 1.f, 1.f);
+                    if (col < p.N) {
+                        sc0[q] = *(const float4*)(p.col_scale + (size_t)g * p.ncs + col);
+                        if constexpr (EPI == EPI_SWIGLU) sc1[q] = *(const float4*)(p.col_scale2 + (size_t)g * p.ncs + col);
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int col = colj + 8 * q;
                     float x[4];
-                    int col;
                     if constexpr (EPI == EPI_SWIGLU) {
-                        // packed columns alternate gate/up in groups of 32: tile j = gate, j+1 = up
-                        col = ((nt * BN + wn * (BN / 2) + j * 32) >> 1) + 8 * q + chalf;
-                        float cg[4] = {1.f, 1.f, 1.f, 1.f}, cu[4] = {1.f, 1.f, 1.f, 1.f};
-                        if constexpr (FP8) {
-                            if (col < p.N) {
-                                const float4 g4 = *(const float4*)(p.col_scale + (size_t)g * p.ncs + col);
-                                const float4 u4 = *(const float4*)(p.col_scale2 + (size_t)g * p.ncs + col);
-                                cg[0] = g4.x * rs; cg[1] = g4.y * rs; cg[2] = g4.z * rs; cg[3] = g4.w * rs;
-                                cu[0] = u4.x * rs; cu[1] = u4.y * rs; cu[2] = u4.z * rs; cu[3] = u4.w * rs;
-                            }
-                        }
+                        const float cg[4] = {sc0[q].x, sc0[q].y, sc0[q].z, sc0[q].w}, cu[4] = {sc1[q].x, sc1[q].y, sc1[q].z, sc1[q].w};
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             float gv = acc[i][j][4 * q + e], uv = acc[i][j + 1][4 * q + e];
-                            if constexpr (FP8) { gv *= cg[e]; uv *= cu[e]; }
+                            if constexpr (FP8) { gv *= cg[e] * rs[i]; uv *= cu[e] * rs[i]; }
                             x[e] = act_silu_fast(gv) * uv;
                         }
                     } else {
-                        col = nt * BN + wn * (BN / 2) + j * 32 + 8 * q + chalf;
-                        float cs[4] = {1.f, 1.f, 1.f, 1.f};
-                        if constexpr (FP8) {
-                            if (col < p.N) {
-                                const float4 c4 = *(const float4*)(p.col_scale + (size_t)g * p.ncs + col);
-                                cs[0] = c4.x * rs; cs[1] = c4.y * rs; cs[2] = c4.z * rs; cs[3] = c4.w * rs;
-                            }
-                        }
+                        const float cs[4] = {sc0[q].x, sc0[q].y, sc0[q].z, sc0[q].w};
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             float v = acc[i][j][4 * q + e];
-                            if constexpr (FP8) v *= cs[e];
+                            if constexpr (FP8) v *= cs[e] * rs[i];
                             if constexpr (EPI == EPI_GELU) v = act_gelu(v);
                             if constexpr (EPI == EPI_SILU) v = act_silu_fast(v);
                             x[e] = v;
                         }
                     }
-                    if (ok && col < p.N) {
+                    if (ok[i] && col < p.N) {
                         uint2 o;
                         o.x = gg_pack_bf16(x[0], x[1]);
                         o.y = gg_pack_bf16(x[2], x[3]);
-                        *(uint2*)(crow + col) = o;
+                        *(uint2*)(crow[i] + col) = o;
                     }
                 }
                 // keep the accumulator read-out of one 32x32 tile from being hoisted over the previous
