@@ -157,6 +157,51 @@ def test_grouped_gemm_mapped(E_l, K, N, S, act):
     assert rc != 0 and b"4 GiB" in lib.moe_last_error()
 
 
+@pytest.mark.parametrize("W,E_l,M,H,F,fill", [(4, 3, 300, 128, 256, "ragged"), (8, 5, 64, 256, 128, "empty"),
+                                              (2, 1, 40, 128, 128, "full")])
+def test_copy_free_destination_equals_operator_chain(W, E_l, M, H, F, fill):
+    """unpack -> GEMM -> GEMM -> return pack against row map -> gathering GEMM -> scattering GEMM -> zeroed
+    padding rows, on receive buffers with empty (source, expert) segments, with nothing received at all,
+    and with every slot full: identical returned buffers, bit for bit."""
+    rng = np.random.default_rng(W * 100 + E_l)
+    if fill == "empty":
+        rc = np.zeros((W, E_l), np.int32)
+    else:
+        rc = np.zeros((W, E_l), np.int32)
+        for s_ in range(W):
+            tot = M if fill == "full" else int(rng.integers(0, M + 1))
+            rc[s_] = rng.multinomial(tot, rng.dirichlet(np.ones(E_l)))
+        if fill == "ragged":
+            rc[1, :] = 0      # a source that sent nothing
+            rc[:, 0] = 0      # an expert that got nothing
+    S = int(rc.sum())
+    recv = _t(_randn(rng, W, M, H), "bf16")
+    rc_t = torch.from_numpy(rc).to(DEV)
+    w1 = _t(_randn(rng, E_l, H, F, scale=H ** -0.5), "bf16")
+    w2 = _t(_randn(rng, E_l, F, H, scale=F ** -0.5), "bf16")
+    p1, p2 = ops.prepack_weights(w1), ops.prepack_weights(w2)
+    S_rows = max(S, 1)
+    from iris_testing_amd import _lib as L
+    # operator chain
+    rows, cnt = ops.unpack_expert_major(recv, rc_t, S_rows)
+    hid = torch.zeros((S_rows, F), dtype=torch.bfloat16, device=DEV)
+    y = torch.zeros((S_rows, H), dtype=torch.bfloat16, device=DEV)
+    lib = L.lib()
+    L.check(lib.moe_grouped_gemm_packed(L.ptr(rows), L.ptr(p1), L.ptr(cnt), S, H, F, E_l, L.ACT["gelu"], L.ptr(hid), L.stream_ptr()))
+    L.check(lib.moe_grouped_gemm_packed(L.ptr(hid), L.ptr(p2), L.ptr(cnt), S, F, H, E_l, 0, L.ptr(y), L.stream_ptr()))
+    want = ops.return_pack(y, rc_t, M)
+    # copy-free chain
+    row_map, cnt2 = ops.recv_row_map(rc_t, M, S)
+    hid2 = torch.zeros((S_rows, F), dtype=torch.bfloat16, device=DEV)
+    got = torch.full((W, M, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.grouped_gemm_mapped(recv.view(W * M, H), row_map, p1, cnt2, S, F, "gelu", hid2)
+    ops.grouped_gemm_mapped(hid2, None, p2, cnt2, S, H, "none", got.view(W * M, H), row_map)
+    ops.zero_padding_rows(got, rc_t)
+    torch.cuda.synchronize()
+    assert torch.equal(cnt, cnt2)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
 @pytest.mark.parametrize("R,C", [(5, 64), (300, 2048), (77, 1408)])
 def test_quantize_rows_fp8_bit_exact(R, C):
     rng = np.random.default_rng(R)
