@@ -410,11 +410,6 @@ int gather_rows(const void* src, void* dst, const RowSource& a, int n_rows, int 
     return moe_check_launch("gather_rows");
 }
 
-struct RecvTables {
-    int32_t *src_off, *row_off, *flat_off;
-};
-// map_ws layout for the recv-driven entry points: [n_out map][tables]
-// three prefix tables plus room for a transposed copy of the counts
 // Expert-major row r of the receive side -> row of the [W,M,H] buffer that holds it (one thread per row,
 // binary search in the (expert, source)-major prefix).  The same index serves the way back: the result
 // row of r returns to the slot its input came from.  Rows past the received total map to row 0.
@@ -451,6 +446,7 @@ __global__ __launch_bounds__(256) void zero_padding_rows_kernel(u32x4* __restric
     for (int c = lane; c < row_vecs; c += WAVE) __builtin_nontemporal_store(z, row + c);
 }
 
+// map_ws of the recv-driven entry points: three prefix tables plus room for a transposed copy of the counts
 size_t recv_tables_ints(int W, int E_l) { return (size_t)3 * (W * E_l + 1) + (size_t)W * E_l; }
 
 int check_rows(const char* who, int dtype, int H) {
