@@ -4,19 +4,19 @@
 // Replaces the reference's intended expert layer (layers/expert.py:31-60) and grouped_gemm kernel
 // (kernels.py:240-289): out[rows of group g] = tokens[rows of g] @ weights[g], fp32 accumulate,
 // persistent grid walking a tile list that spans all groups.  Differences in kind, not a port:
-//   * tiles are 256 (or 128) x 256, four wave64s each owning a 128 (64) x 128 block of 32x32x16 MFMAs
-//     with the accumulators in the accumulation registers;
+//   * tiles are 256 (or 128) x 256, four wave64s each owning a 128 (64) x 128 block of 16x16x32 (bf16) or
+//     32x32x64 (fp8) MFMAs with the accumulators in the accumulation registers;
 //   * operands go HBM -> LDS directly (global_load_lds, 16 bytes per lane) through a ring of four
-//     64-byte K stages, the loads of a stage spread over two MFMA blocks and issued two stages ahead;
-//     an XOR swizzle of the 16-byte chunks keeps MFMA fragment reads bank-conflict free;
-//   * fragment reads are interleaved one by one between the MFMAs of the previous K step, and the
-//     products of a step are taken in the order in which their operands arrive;
+//     64-byte K stages; the loads of a stage are spread evenly over one MFMA block and issued more than two
+//     blocks ahead; an XOR swizzle of the 16-byte chunks keeps MFMA fragment reads bank-conflict free;
+//   * one MFMA block per stage: fragment reads and loads are interleaved one by one between its MFMAs;
 //   * weights are re-tiled once into a K-contiguous layout (gate/up interleaved for SwiGLU) so both
 //     MFMA operands are read as 128-bit fragments;
 //   * ragged group tails are masked (the reference assumes full tiles, kernels.py:270,282);
 //   * the tile walk is XCD-aware: the 32 workgroups that share an L2 take a compact 4 x 8 patch of
 //     a 16 x 16 super-tile.
 #include "common.h"
+#include <type_traits>
 
 namespace moe_gg {
 
@@ -61,19 +61,10 @@ __device__ __forceinline__ float act_silu_fast(float x) { return x * __builtin_a
 __device__ __forceinline__ float act_silu(float x) { return x / (1.0f + __expf(-x)); }
 __device__ __forceinline__ float act_gelu(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }
 
-template <bool FP8>
-__device__ __forceinline__ void mma(floatx16& acc, const uint4& a, const uint4& b) {
-    if constexpr (FP8) {
-        // 16 bytes per lane = two 8-byte K groups; both operands are split the same way, so every
-        // k of the 32 covered by the lane pair is multiplied exactly once.
-        const long a0 = (long)(((unsigned long)a.y << 32) | a.x), a1 = (long)(((unsigned long)a.w << 32) | a.z);
-        const long b0 = (long)(((unsigned long)b.y << 32) | b.x), b1 = (long)(((unsigned long)b.w << 32) | b.z);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a0, b0, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(a1, b1, acc, 0, 0, 0);
-    } else {
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
-                                                      acc, 0, 0, 0);
-    }
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+// bf16: one 16x16x32 MFMA; lanes 16q .. 16q+15 hold K elements 8q .. 8q+7 (16 bytes) of rows 0 .. 15 of both operands
+__device__ __forceinline__ void mma_bf16_k32(floatx4& acc, const uint4& a, const uint4& b) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
 }
 
 // fp8: one 32x32x64 MFMA on 32 bytes of K per lane and operand (two 16-byte LDS chunks); both operands
@@ -157,58 +148,6 @@ __device__ __forceinline__ const uint8_t* gg_uniform(const uint8_t* p) {
     return (const uint8_t*)(((uint64_t)hi << 32) | lo);
 }
 
-template <int TM, int TN>
-__device__ __forceinline__ void gg_frags(const uint4* fa, const uint4* fb, int pos, uint4 (&a)[TM], uint4 (&b)[TN]) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i) a[i] = fa[i * 32 * CHUNKS + pos];
-#pragma unroll
-    for (int j = 0; j < TN; ++j) b[j] = fb[j * 32 * CHUNKS + pos];
-}
-
-// Order of the TM x TN products of one MFMA block and of the TM + TN fragment reads that feed the
-// next block: fragments are read a0, b0, a1, b1, ... and the products are taken in the order in which
-// their operands arrive ((0,0); then everything that needs a1; then everything that needs b1; ...), so
-// a read issued late in one block is not needed before late in the next.
-template <int TM, int TN>
-struct GgOrder {
-    static constexpr int NT = TM * TN, NR = TM + TN, D = TM > TN ? TM : TN;
-    // I-th product -> (a index, b index)
-    static constexpr int prod(int I, bool want_a) {
-        int n = 0;
-        for (int d = 0; d < D; ++d) {
-            if (d < TM)
-                for (int j = 0; j < (d < TN ? d : TN); ++j, ++n)
-                    if (n == I) return want_a ? d : j;
-            if (d < TN)
-                for (int i = 0; i <= (d < TM ? d : TM - 1); ++i, ++n)
-                    if (n == I) return want_a ? i : d;
-        }
-        return 0;
-    }
-    // R-th read -> operand (true: a) and index
-    static constexpr int read(int R, bool want_is_a) {
-        int n = 0;
-        for (int d = 0; d < D; ++d) {
-            if (d < TM) { if (n == R) return want_is_a ? 1 : d; ++n; }
-            if (d < TN) { if (n == R) return want_is_a ? 0 : d; ++n; }
-        }
-        return 0;
-    }
-    // the n-th (0 or 1) read issued behind product I (-1: none).  Reads are spread evenly over the whole
-    // block, or over its first half when the block ends in a hand-over (the wave must hold its last
-    // fragments of a slot before it lets the other waves refill that slot).
-    static constexpr int read_at(int I, bool front, int n) {
-        const int span = front ? NT / 2 : NT;
-        int seen = 0;
-        for (int R = 0; R < NR; ++R)
-            if ((R * span) / NR == I) {
-                if (seen == n) return R;
-                ++seen;
-            }
-        return -1;
-    }
-};
-
 // s_waitcnt through the builtin (not inline asm) so that the compiler's own wait-count bookkeeping
 // sees it.  gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14.
 template <int VM, int LGKM>
@@ -217,9 +156,6 @@ __device__ __forceinline__ void gg_wait() {
     __builtin_amdgcn_s_waitcnt((VM & 15) | (7 << 4) | (LGKM << 8) | ((VM >> 4) << 14));
 }
 
-// acc(i,j) holds the TRANSPOSED 32x32 product (weights as the MFMA A operand, activations as B):
-// lane l owns token row l%32 and output columns 8*(v/4) + 4*(l/32) + v%4, v = 0..15, i.e. four runs
-// of four consecutive columns -> 8-byte bf16 stores.
 // NWM x 2 wave64s per workgroup; every wave owns a (BM/NWM) x 128 block of the tile.
 //
 // K moves through LDS in a ring of NRING stages of ROWB bytes per tile row.  A stage is two MFMA
@@ -232,15 +168,30 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     constexpr int BN = GG_BN;
     constexpr int ES = FP8 ? 1 : 2;
     constexpr int NW = NWM * 2;                        // waves per workgroup
-    constexpr int TM = BM / (NWM * 32), TN = BN / 64;  // 32x32 MFMA tiles per wave
-    constexpr int NT = TM * TN;
+    // bf16: 16x16x32 MFMAs (4 accumulator registers each; under the power limit this shape sustains about
+    // 15 % more than 32x32x16, which moves twice the accumulator bytes per flop); fp8: 32x32x64
+    constexpr int MT = FP8 ? 32 : 16;                  // MFMA tile edge
+    constexpr int CF = FP8 ? 2 : 1;                    // 16-byte LDS chunks per fragment and lane
+    constexpr int TM = BM / (NWM * MT), TN = BN / (2 * MT);  // MFMA tiles per wave
+    constexpr int NT = TM * TN;                        // MFMAs per K stage and wave
+    constexpr int NRD = (TM + TN) * CF;                // fragment reads per K stage and wave
     constexpr int LR = NW * WROWS;                     // rows fetched per load round (16 per wave)
     constexpr int RA = BM / LR, RB = BN / LR;          // load rounds per stage
     constexpr int LPS = RA + RB;                       // HBM->LDS loads per lane per stage
-    constexpr int LH = LPS / 2;                        // ... per MFMA block
+    // Where the other instructions of a block sit.  bf16: a 16x16x32 MFMA covers only 16 cycles of other issue,
+    // so no MFMA gets more than one: the fragment reads go behind every RSTEP-th MFMA of the first half of the
+    // block (they must have landed when the block ends in the hand-over), the loads are spread evenly over the
+    // whole block, behind other MFMAs where that fits (a steady stream to the load pipe: bunched at either end
+    // of the block they cost 7 % more cycles).  fp8: a 32x32x64 MFMA covers 64 cycles and there are few of them;
+    // two reads go behind each of the first MFMAs.
+    constexpr int RPM = NRD > NT / 2 ? 2 : 1;                 // reads behind one MFMA
+    constexpr int RFIRST = 0;                                 // first MFMA with a read behind it
+    constexpr int RSTEP = (NT / 2) * RPM / NRD > 0 ? (NT / 2) * RPM / NRD : 1;  // MFMAs from one read group to the next
+    constexpr int LFIRST = NT > LPS ? 1 : 0;                  // first MFMA with a load behind it
+    constexpr int LSTEP = (NT - LFIRST) / LPS;                // MFMAs from one load to the next
     constexpr int ASLOT = BM * CHUNKS, BSLOT = BN * CHUNKS;  // uint4 per ring slot
-    static_assert(TM * 32 * NWM == BM && BM % LR == 0 && BN % LR == 0 && LPS % 2 == 0 && LH <= NT, "tile shape");
-    static_assert(CHUNKS == 4 && NRING == 4, "the stage schedule below is written for two MFMA blocks per stage and four slots");
+    static_assert(TM * MT * NWM == BM && BM % LR == 0 && BN % LR == 0 && NT <= 64 && LSTEP >= 1 && LFIRST + LSTEP * (LPS - 1) < NT && RFIRST + RSTEP * ((NRD - 1) / RPM) < NT, "tile shape");
+    static_assert(CHUNKS == 4 && NRING == 4, "the stage schedule below is written for 64-byte stages in four slots");
 
     __shared__ __align__(1024) uint4 sA[NRING * ASLOT];
     __shared__ __align__(1024) uint4 sB[NRING * BSLOT];
@@ -279,17 +230,21 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     // and the 128-bit fragment reads (rows = lane % 32) bank-conflict free.
     const int lrow = wave * WROWS + (lane >> 2);         // row inside a load round
     const int lchunk = (lane & 3) ^ ((lane >> 4) & 3);   // global 16-byte chunk this lane fetches
-    const int fswz = (lane >> 2) & 3;                    // swizzle of the fragment row
-    const int khalf = lane >> 5;
-    const int pos0 = (0 + khalf) ^ fswz, pos1 = (2 + khalf) ^ fswz;
-    const uint4* fa = sA + (wm * (BM / NWM) + (lane & 31)) * CHUNKS;
-    const uint4* fb = sB + (wn * (BN / 2) + (lane & 31)) * CHUNKS;
+    const int fswz = (lane >> 2) & 3;                    // swizzle of the fragment row (tile rows start at multiples of 16)
+    // first 16-byte chunk of the lane's fragment: bf16 lanes 16q .. 16q+15 take chunk q of rows 0 .. 15;
+    // fp8 lanes 32h .. 32h+31 take chunks 2h, 2h+1 of rows 0 .. 31
+    const int fpos = (FP8 ? 2 * (lane >> 5) : (lane >> 4)) ^ fswz;
+    const uint4* fa = sA + (wm * (BM / NWM) + (lane & (MT - 1))) * CHUNKS;
+    const uint4* fb = sB + (wn * (BN / 2) + (lane & (MT - 1))) * CHUNKS;
     const uint32_t la0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(sA + wave * WROWS * CHUNKS));
     const uint32_t lb0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(sB + wave * WROWS * CHUNKS));
 
     const uint32_t ldk = (uint32_t)(p.K * ES);
     const size_t b_slab = (size_t)p.Npad * ROWB;  // packed weights are slab-major: [group][K slab][Npad rows][ROWB bytes]
-    const uint32_t b_off0 = (uint32_t)lrow * ROWB + lchunk * 16;
+    // per-round lane offsets into the weight slab (vector registers: no scalar address arithmetic per load)
+    uint32_t b_off[RB];
+#pragma unroll
+    for (int r = 0; r < RB; ++r) b_off[r] = (uint32_t)(r * LR + lrow) * ROWB + lchunk * 16;
 
 #define GG_TILE_PTRS(t, Ab_, Bb_, aoff_)                                                                   \
     const uint8_t* Ab_ = p.a_map ? p.A : p.A + (size_t)(t).row0 * p.K * ES;                                 \
@@ -303,7 +258,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 #define GG_LD(d, ap_, bp_, aoff_, slot)                                                                       \
     do {                                                                                                      \
         if constexpr ((d) < RA) gg_dma16(ap_, aoff_[(d) < RA ? (d) : 0], la0 + ((slot) * ASLOT + (d) * LR * CHUNKS) * 16); \
-        else gg_dma16(bp_ + (size_t)((d) - RA) * (LR * ROWB), b_off0, lb0 + ((slot) * BSLOT + ((d) - RA) * LR * CHUNKS) * 16); \
+        else gg_dma16(bp_, b_off[(d) >= RA ? (d) - RA : 0], lb0 + ((slot) * BSLOT + ((d) - RA) * LR * CHUNKS) * 16); \
     } while (0)
     // loads [first, first + count) of stage `st` (clamped to the last stage: the ring never holds data
     // of another tile, and a repeated load of the last stage lands in a slot nobody reads again)
@@ -324,13 +279,13 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         if constexpr ((first) + 7 < (first) + (count)) GG_LD((first) + 7 < LPS ? (first) + 7 : 0, ap_i, bp_i, aoff_, slot); \
         static_assert((count) <= 8, "GG_ISSUE_RANGE is unrolled for eight loads");             \
     } while (0)
-    // what a tile has in flight before its first MFMA: stages 0, 1, 2 and the first half of stage 3
+    // what a tile has in flight before its first MFMA: its first four stages, one per ring slot
 #define GG_PROLOGUE(Ab_, Bb_, aoff_)                          \
     do {                                                      \
         GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 0, 0, 0, LPS);        \
         GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 1, 1, 0, LPS);        \
         GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 2, 2, 0, LPS);        \
-        GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 3, 3, 0, (FP8 ? LPS : LH)); \
+        GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 3, 3, 0, LPS);        \
     } while (0)
 
     int base = 0;
@@ -349,173 +304,101 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         const int g = __builtin_amdgcn_readfirstlane(cur.g), nt = __builtin_amdgcn_readfirstlane(cur.nt);
         const int row0 = __builtin_amdgcn_readfirstlane(cur.row0), rv = __builtin_amdgcn_readfirstlane(cur.rv);
 
-        floatx16 acc[TM][TN];
+        typedef typename std::conditional<FP8, floatx16, floatx4>::type acc_t;
+        acc_t acc[TM][TN];
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+                for (int v = 0; v < (FP8 ? 16 : 4); ++v) acc[i][j][v] = 0.f;
 
-        static_assert(NT == 8 || NT == 16, "GG_BLOCK is unrolled for 8 or 16 MFMA tiles per wave");
-
-        // One MFMA block: the NT products of one 32-byte K step, with (a) the fragment reads of the next
-        // step right behind the first MFMA and (b) LH loads of a later stage spread between the MFMAs.
-        // Everything is pinned by scheduling fences: each load is issued in the shadow of an MFMA.
-        using Ord = GgOrder<TM, TN>;
-#define GG_MM(I, FA_, FB_)                                                                               \
-    do {                                                                                                 \
-        constexpr int pa_ = Ord::prod(I, true), pb_ = Ord::prod(I, false);                               \
-        mma<FP8>(acc[pa_][pb_], FB_[pb_], FA_[pa_]);                                                     \
-    } while (0)
-        // fragment read R of the next step, from slot-relative bases nfa_/nfb_ at chunk position npos_
+        // ---- One MFMA block per 64-byte stage.  Block s multiplies the fragments of stage s, reads those of
+        // stage s+1 (all issued in the first half of the block, so they have landed when the block ends) and
+        // refills slot s % 4, drained one block earlier, with stage s+4, its loads spread between the MFMAs
+        // (a steady stream instead of a burst, each with three blocks of MFMA work to land); the hand-over at
+        // its end waits for the wave's own loads of stage s+2 -- everything issued after them, stages s+3 and
+        // s+4, may stay in flight -- and meets the other waves.  Loads past the end of the tile are clamped
+        // to its last stage (straight-line code, constant wait counts); in the last block the "next
+        // fragments" are whatever the next slot holds and are never used.  Every instruction is pinned by
+        // scheduling fences: each read and each load is issued in the shadow of an MFMA.
+        // fragment read R of the next stage: operand R / CF (activation rows first, then weight rows), chunk R % CF
 #define GG_RD(R, NA_, NB_)                                                                               \
     do {                                                                                                 \
-        constexpr bool ra_ = Ord::read(R, true) != 0;                                                    \
-        constexpr int ri_ = Ord::read(R, false);                                                         \
-        if constexpr (ra_) NA_[ri_] = nfa_[ri_ * 32 * CHUNKS + npos_];                                   \
-        else NB_[ri_] = nfb_[ri_ * 32 * CHUNKS + npos_];                                                 \
+        constexpr int ro_ = (R) / CF, rh_ = (R) % CF;                                                    \
+        if constexpr (ro_ < TM) NA_[ro_ * CF + rh_] = nfa_[ro_ * MT * CHUNKS + (fpos ^ rh_)];            \
+        else NB_[(ro_ - TM) * CF + rh_] = nfb_[(ro_ - TM) * MT * CHUNKS + (fpos ^ rh_)];                 \
     } while (0)
-#define GG_ML(I, FA_, FB_, NA_, NB_, aoff_, slot, half)                                                  \
+#define GG_ML(I, FA_, FB_, NA_, NB_, slot)                                                               \
     do {                                                                                                 \
         if constexpr ((I) < NT) {                                                                        \
-            GG_MM(I, FA_, FB_);                                                                          \
+            constexpr int pa_ = (I) / TN, pb_ = (I) % TN;                                                \
+            if constexpr (FP8) mma_fp8_k64(acc[pa_][pb_], FB_[2 * pb_], FB_[2 * pb_ + 1], FA_[2 * pa_], FA_[2 * pa_ + 1]); \
+            else mma_bf16_k32(acc[pa_][pb_], FB_[pb_], FA_[pa_]);                                        \
             __builtin_amdgcn_sched_barrier(0);                                                           \
-            constexpr int rd_ = Ord::read_at(I, (half) == 1, 0), rd2_ = Ord::read_at(I, (half) == 1, 1); \
-            if constexpr (rd_ >= 0) GG_RD((rd_ >= 0 ? rd_ : 0), NA_, NB_);                               \
-            if constexpr (rd2_ >= 0) GG_RD((rd2_ >= 0 ? rd2_ : 0), NA_, NB_);                            \
-            if constexpr (((I) + 1) * LH / NT > (I) * LH / NT) GG_LD((half) * LH + (I) * LH / NT, ap_, bp_, aoff_, slot); \
-            __builtin_amdgcn_sched_barrier(0);                                                           \
-        }                                                                                                \
-    } while (0)
-        // One MFMA block: the NT products of one 32-byte K step (FA_, FB_), with the fragment reads of the
-        // next step (into NA_, NB_) and LH loads of a later stage spread between them.  Everything is
-        // pinned by scheduling fences: each read and each load is issued in the shadow of an MFMA.
-#define GG_BLOCK(FA_, FB_, NA_, NB_, nslot, npos, st, slot, half)                                        \
-    do {                                                                                                 \
-        GG_STAGE_PTRS(Ab, Bb, st, ap_, bp_)                                                              \
-        const uint4* nfa_ = fa + (nslot) * ASLOT;                                                        \
-        const uint4* nfb_ = fb + (nslot) * BSLOT;                                                        \
-        const int npos_ = (npos);                                                                        \
-        __builtin_amdgcn_sched_barrier(0);                                                               \
-        GG_ML(0, FA_, FB_, NA_, NB_, a_off, slot, half); GG_ML(1, FA_, FB_, NA_, NB_, a_off, slot, half);   \
-        GG_ML(2, FA_, FB_, NA_, NB_, a_off, slot, half); GG_ML(3, FA_, FB_, NA_, NB_, a_off, slot, half);   \
-        GG_ML(4, FA_, FB_, NA_, NB_, a_off, slot, half); GG_ML(5, FA_, FB_, NA_, NB_, a_off, slot, half);   \
-        GG_ML(6, FA_, FB_, NA_, NB_, a_off, slot, half); GG_ML(7, FA_, FB_, NA_, NB_, a_off, slot, half);   \
-        GG_ML(8, FA_, FB_, NA_, NB_, a_off, slot, half); GG_ML(9, FA_, FB_, NA_, NB_, a_off, slot, half);   \
-        GG_ML(10, FA_, FB_, NA_, NB_, a_off, slot, half); GG_ML(11, FA_, FB_, NA_, NB_, a_off, slot, half); \
-        GG_ML(12, FA_, FB_, NA_, NB_, a_off, slot, half); GG_ML(13, FA_, FB_, NA_, NB_, a_off, slot, half); \
-        GG_ML(14, FA_, FB_, NA_, NB_, a_off, slot, half); GG_ML(15, FA_, FB_, NA_, NB_, a_off, slot, half); \
-    } while (0)
-        // Stage s of the tile sits in slot s % 4 (SL below).  Block 0 multiplies the fragments of its first
-        // K step while those of the second are read, and issues the second half of stage s+3's loads
-        // (slot SL+3); the hand-over waits for this wave's own loads of stage s+1 (everything issued
-        // after them -- stages s+2 and s+3 -- may stay in flight) and for its last fragments of stage s,
-        // then meets the other waves; block 1 reads the first fragments of stage s+1 and refills slot SL
-        // with the first half of stage s+4.  In the last stage of a tile block 1 still reads "the next
-        // stage" (whatever slot SL+1 holds): those fragments are never used.
-#define GG_STAGE(SL, s, last)                                                                            \
-    do {                                                                                                 \
-        GG_BLOCK(a0, b0, a1, b1, SL, pos1, (s) + 3, ((SL) + 3) & 3, 1);                                  \
-        if (!(last)) {                                                                                   \
-            gg_wait<2 * LPS, 0>();                                                                       \
-            __builtin_amdgcn_s_barrier();                                                                \
-        }                                                                                                \
-        GG_BLOCK(a1, b1, a0, b0, ((SL) + 1) & 3, pos0, (s) + 4, SL, 0);                                  \
-    } while (0)
-
-        // ---- fp8: one MFMA block per 64-byte stage (K = 64 per 32x32x64 MFMA).  Block s multiplies the
-        // fragments of stage s, reads those of stage s+1 (two 16-byte chunks per operand row, all issued in
-        // the first half of the block) and refills slot s % 4, drained one block earlier, with stage s+4;
-        // the hand-over at its end waits for the wave's own loads of stage s+2.
-#define GG_WRD(R, NA_, NB_)                                                                              \
-    do {                                                                                                 \
-        constexpr bool ra_ = Ord::read((R) / 2, true) != 0;                                              \
-        constexpr int ri_ = Ord::read((R) / 2, false), rh_ = (R) % 2;                                    \
-        if constexpr (ra_) NA_[2 * ri_ + rh_] = nfa_[ri_ * 32 * CHUNKS + (npos_ ^ rh_)];                 \
-        else NB_[2 * ri_ + rh_] = nfb_[ri_ * 32 * CHUNKS + (npos_ ^ rh_)];                               \
-    } while (0)
-#define GG_WML(I, FA_, FB_, NA_, NB_, slot)                                                              \
-    do {                                                                                                 \
-        if constexpr ((I) < NT) {                                                                        \
-            constexpr int pa_ = Ord::prod(I, true), pb_ = Ord::prod(I, false);                           \
-            mma_fp8_k64(acc[pa_][pb_], FB_[2 * pb_], FB_[2 * pb_ + 1], FA_[2 * pa_], FA_[2 * pa_ + 1]);  \
-            __builtin_amdgcn_sched_barrier(0);                                                           \
-            if constexpr ((I) < Ord::NR) { GG_WRD(2 * ((I) < Ord::NR ? (I) : 0), NA_, NB_); GG_WRD(2 * ((I) < Ord::NR ? (I) : 0) + 1, NA_, NB_); } \
-            if constexpr (((I) + 1) * LPS / NT > (I) * LPS / NT) GG_LD((I) * LPS / NT, ap_, bp_, a_off, slot); \
+            constexpr int ld_ = (I) >= LFIRST && ((I) - LFIRST) % LSTEP == 0 ? ((I) - LFIRST) / LSTEP : LPS;  /* load behind this MFMA */ \
+            if constexpr (ld_ < LPS) GG_LD((ld_ < LPS ? ld_ : 0), ap_, bp_, a_off, slot);                \
+            constexpr int r0_ = (I) >= RFIRST && ((I) - RFIRST) % RSTEP == 0 ? (((I) - RFIRST) / RSTEP) * RPM : NRD; /* first read */ \
+            if constexpr (r0_ < NRD) GG_RD((r0_ < NRD ? r0_ : 0), NA_, NB_);                             \
+            if constexpr (RPM > 1 && r0_ + 1 < NRD) GG_RD((r0_ + 1 < NRD ? r0_ + 1 : 0), NA_, NB_);      \
             __builtin_amdgcn_sched_barrier(0);                                                           \
         }                                                                                                \
     } while (0)
-#define GG_WSTAGE(FA_, FB_, NA_, NB_, SL, s, last)                                                       \
+#define GG_ML8(I, FA_, FB_, NA_, NB_, slot)                                                              \
+    GG_ML((I) + 0, FA_, FB_, NA_, NB_, slot); GG_ML((I) + 1, FA_, FB_, NA_, NB_, slot);                   \
+    GG_ML((I) + 2, FA_, FB_, NA_, NB_, slot); GG_ML((I) + 3, FA_, FB_, NA_, NB_, slot);                   \
+    GG_ML((I) + 4, FA_, FB_, NA_, NB_, slot); GG_ML((I) + 5, FA_, FB_, NA_, NB_, slot);                   \
+    GG_ML((I) + 6, FA_, FB_, NA_, NB_, slot); GG_ML((I) + 7, FA_, FB_, NA_, NB_, slot)
+#define GG_STAGE(FA_, FB_, NA_, NB_, SL, s, last)                                                        \
     do {                                                                                                 \
         GG_STAGE_PTRS(Ab, Bb, (s) + 4, ap_, bp_)                                                         \
         const uint4* nfa_ = fa + (((SL) + 1) & 3) * ASLOT;                                               \
         const uint4* nfb_ = fb + (((SL) + 1) & 3) * BSLOT;                                               \
-        const int npos_ = wpos;                                                                          \
         __builtin_amdgcn_sched_barrier(0);                                                               \
-        GG_WML(0, FA_, FB_, NA_, NB_, SL); GG_WML(1, FA_, FB_, NA_, NB_, SL); GG_WML(2, FA_, FB_, NA_, NB_, SL);   \
-        GG_WML(3, FA_, FB_, NA_, NB_, SL); GG_WML(4, FA_, FB_, NA_, NB_, SL); GG_WML(5, FA_, FB_, NA_, NB_, SL);   \
-        GG_WML(6, FA_, FB_, NA_, NB_, SL); GG_WML(7, FA_, FB_, NA_, NB_, SL); GG_WML(8, FA_, FB_, NA_, NB_, SL);   \
-        GG_WML(9, FA_, FB_, NA_, NB_, SL); GG_WML(10, FA_, FB_, NA_, NB_, SL); GG_WML(11, FA_, FB_, NA_, NB_, SL); \
-        GG_WML(12, FA_, FB_, NA_, NB_, SL); GG_WML(13, FA_, FB_, NA_, NB_, SL); GG_WML(14, FA_, FB_, NA_, NB_, SL); \
-        GG_WML(15, FA_, FB_, NA_, NB_, SL);                                                              \
+        GG_ML8(0, FA_, FB_, NA_, NB_, SL); GG_ML8(8, FA_, FB_, NA_, NB_, SL);                             \
+        GG_ML8(16, FA_, FB_, NA_, NB_, SL); GG_ML8(24, FA_, FB_, NA_, NB_, SL);                           \
+        GG_ML8(32, FA_, FB_, NA_, NB_, SL); GG_ML8(40, FA_, FB_, NA_, NB_, SL);                           \
+        GG_ML8(48, FA_, FB_, NA_, NB_, SL); GG_ML8(56, FA_, FB_, NA_, NB_, SL);                           \
         if (!(last)) {                                                                                   \
             gg_wait<2 * LPS, 0>();                                                                       \
             __builtin_amdgcn_s_barrier();                                                                \
         }                                                                                                \
     } while (0)
-        if constexpr (FP8) {
-            uint4 wa0[2 * TM], wb0[2 * TN], wa1[2 * TM], wb1[2 * TN];
-            const int wpos = (2 * khalf) ^ fswz;  // first of the lane's two chunks (the second is wpos ^ 1)
-            // all four stages of this tile were requested before the previous tile's epilogue
+        {
+            uint4 fA0[TM * CF], fB0[TN * CF], fA1[TM * CF], fB1[TN * CF];
+            // the four stages of this tile were requested before the previous tile's epilogue (or above, for
+            // the first tile); the epilogue's stores sit behind them in the same counter, so wait for
+            // everything once per tile
             gg_wait<0, 15>();
             __syncthreads();
 #pragma unroll
-            for (int i = 0; i < TM; ++i) { wa0[2 * i] = fa[i * 32 * CHUNKS + wpos]; wa0[2 * i + 1] = fa[i * 32 * CHUNKS + (wpos ^ 1)]; }
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) { wb0[2 * j] = fb[j * 32 * CHUNKS + wpos]; wb0[2 * j + 1] = fb[j * 32 * CHUNKS + (wpos ^ 1)]; }
+                for (int h = 0; h < CF; ++h) fA0[i * CF + h] = fa[i * MT * CHUNKS + (fpos ^ h)];
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int h = 0; h < CF; ++h) fB0[j * CF + h] = fb[j * MT * CHUNKS + (fpos ^ h)];
             // slot 0 is refilled from the first block on: every wave must hold its stage-0 fragments first
             gg_wait<63, 0>();
             __syncthreads();
-            int ks = 0;
-            do {
-                GG_WSTAGE(wa0, wb0, wa1, wb1, 0, ks, false);
-                GG_WSTAGE(wa1, wb1, wa0, wb0, 1, ks + 1, ks + 2 >= nk);
-                if (ks + 2 < nk) {
-                    GG_WSTAGE(wa0, wb0, wa1, wb1, 2, ks + 2, false);
-                    GG_WSTAGE(wa1, wb1, wa0, wb0, 3, ks + 3, ks + 4 >= nk);
-                }
-                ks += 4;
-            } while (ks < nk);
-        } else {
-            uint4 a0[TM], b0[TN], a1[TM], b1[TN];
-            // stages 0-2 and half of stage 3 of this tile were requested before the previous tile's epilogue
-            // (or above, for the first tile); the epilogue's stores sit behind them in the same counter, so
-            // wait for everything once per tile
-            gg_wait<0, 15>();
-            __syncthreads();
-            gg_frags<TM, TN>(fa, fb, pos0, a0, b0);
             // nk >= 2 and even: a loop that cannot run zero times keeps the accumulators in place from their
             // zeroing to the epilogue
             int ks = 0;
             do {
-                GG_STAGE(0, ks, false);
-                GG_STAGE(1, ks + 1, ks + 2 >= nk);
+                GG_STAGE(fA0, fB0, fA1, fB1, 0, ks, false);
+                GG_STAGE(fA1, fB1, fA0, fB0, 1, ks + 1, ks + 2 >= nk);
                 if (ks + 2 < nk) {
-                    GG_STAGE(2, ks + 2, false);
-                    GG_STAGE(3, ks + 3, ks + 4 >= nk);
+                    GG_STAGE(fA0, fB0, fA1, fB1, 2, ks + 2, false);
+                    GG_STAGE(fA1, fB1, fA0, fB0, 3, ks + 3, ks + 4 >= nk);
                 }
                 ks += 4;
             } while (ks < nk);
         }
-#undef GG_WSTAGE
-#undef GG_WML
-#undef GG_WRD
 #undef GG_STAGE
-#undef GG_BLOCK
+#undef GG_ML8
 #undef GG_ML
 #undef GG_RD
-#undef GG_MM
 
         // ---- next tile: decode it and request its first stages now (every slot is free once all waves
         // have passed the barrier: the last fragments of this tile are already in registers)
@@ -527,16 +410,24 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         }
 
         // ---- epilogue: acc -> (scales) -> activation -> bf16 -> C
-        // Column tiles outermost: the fp8 per-channel scales of a column tile are fetched once and serve
-        // the wave's TM row tiles.
+        // acc(i,j) holds the TRANSPOSED MT x MT product (weights as the MFMA A operand, activations as B):
+        // a lane owns one token row of the tile and runs of four consecutive output columns -> 8-byte stores.
+        //   bf16 (16x16): row l % 16, columns 4 * (l / 16) + v, v = 0..3
+        //   fp8  (32x32): row l % 32, columns 8 * q + 4 * (l / 32) + v for the four register quads q
+        // SwiGLU: packed columns alternate gate / up in groups of 32, so the gate tile and its up tile lie
+        // 32 packed columns apart and land on output column (packed column of the gate) / 2 + ... .
+        // Column tiles are walked outermost: the fp8 per-channel scales of a column tile are fetched once and
+        // serve the wave's TM row tiles.
         bf16_t* C = (bf16_t*)p.C;
-        const int chalf = khalf * 4;
+        constexpr int NQ = FP8 ? 4 : 1;              // runs of four columns per lane and tile
+        constexpr int UPJ = 32 / MT;                 // tiles between a gate tile and its up tile
+        const int clane = FP8 ? (lane >> 5) * 4 : (lane >> 4) * 4;  // first column of the lane's run inside 8 (fp8) / 16 (bf16) columns
         bool ok[TM];
         bf16_t* crow[TM];
         float rs[TM];
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            const int r = wm * (BM / NWM) + i * 32 + (lane & 31);
+            const int r = wm * (BM / NWM) + i * MT + (lane & (MT - 1));
             ok[i] = r < rv;
             const size_t grow = (size_t)(row0 + (ok[i] ? r : 0));
             rs[i] = 1.f;
@@ -544,14 +435,16 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             crow[i] = C + (p.c_map ? (size_t)p.c_map[grow] : grow) * p.ldc;
         }
 #pragma unroll
-        for (int j = 0; j < TN; j += (EPI == EPI_SWIGLU ? 2 : 1)) {
-            // first output column of this lane in the tile (SwiGLU: packed columns alternate gate/up in groups
-            // of 32, tile j = gate, j+1 = up, both land on output columns (packed column / 2))
-            const int colj = (EPI == EPI_SWIGLU ? ((nt * BN + wn * (BN / 2) + j * 32) >> 1) : nt * BN + wn * (BN / 2) + j * 32) + chalf;
-            float4 sc0[4], sc1[4];  // fp8: channel scales of the lane's 4 x 4 columns (gate / only; up)
+        for (int j = 0; j < TN; ++j) {
+            if constexpr (EPI == EPI_SWIGLU) {
+                if ((j / UPJ) % 2 == 1) continue;  // an up tile: consumed together with its gate tile
+            }
+            const int pcol = nt * BN + wn * (BN / 2) + j * MT;  // first packed column of the tile
+            const int colj = (EPI == EPI_SWIGLU ? (pcol / 64) * 32 + pcol % 32 : pcol) + clane;
+            float4 sc0[NQ], sc1[NQ];  // fp8: channel scales of the lane's columns (gate / only; up)
             if constexpr (FP8) {
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
+                for (int q = 0; q < NQ; ++q) {
                     const int col = colj + 8 * q;
                     sc0[q] = sc1[q] = make_float4(1.f, 1.f, 1.f, 1.f);
                     if (col < p.N) {
@@ -563,19 +456,25 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
+                for (int q = 0; q < NQ; ++q) {
                     const int col = colj + 8 * q;
                     float x[4];
                     if constexpr (EPI == EPI_SWIGLU) {
-                        const float cg[4] = {sc0[q].x, sc0[q].y, sc0[q].z, sc0[q].w}, cu[4] = {sc1[q].x, sc1[q].y, sc1[q].z, sc1[q].w};
+                        constexpr int ju_ = UPJ;  // offset of the up tile
+                        float cg[4] = {1.f, 1.f, 1.f, 1.f}, cu[4] = {1.f, 1.f, 1.f, 1.f};
+                        if constexpr (FP8) {
+                            cg[0] = sc0[q].x; cg[1] = sc0[q].y; cg[2] = sc0[q].z; cg[3] = sc0[q].w;
+                            cu[0] = sc1[q].x; cu[1] = sc1[q].y; cu[2] = sc1[q].z; cu[3] = sc1[q].w;
+                        }
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            float gv = acc[i][j][4 * q + e], uv = acc[i][j + 1][4 * q + e];
+                            float gv = acc[i][j][4 * q + e], uv = acc[i][(j + ju_) % TN][4 * q + e];
                             if constexpr (FP8) { gv *= cg[e] * rs[i]; uv *= cu[e] * rs[i]; }
                             x[e] = act_silu_fast(gv) * uv;
                         }
                     } else {
-                        const float cs[4] = {sc0[q].x, sc0[q].y, sc0[q].z, sc0[q].w};
+                        float cs[4] = {1.f, 1.f, 1.f, 1.f};
+                        if constexpr (FP8) { cs[0] = sc0[q].x; cs[1] = sc0[q].y; cs[2] = sc0[q].z; cs[3] = sc0[q].w; }
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             float v = acc[i][j][4 * q + e];
@@ -592,9 +491,9 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                         *(uint2*)(crow[i] + col) = o;
                     }
                 }
-                // keep the accumulator read-out of one 32x32 tile from being hoisted over the previous
-                // tile's stores (with 16 tiles per wave that would need every accumulator in a VGPR at once)
-                __builtin_amdgcn_sched_barrier(0);
+                // keep the accumulator read-out of one tile from being hoisted over the previous tile's stores
+                // (that would need every accumulator in a VGPR at once)
+                if (FP8 || (i % 2 == 1)) __builtin_amdgcn_sched_barrier(0);
             }
         }
         cur = nxt;
