@@ -162,7 +162,7 @@ def main():
                      "frac": round(ach / peak, 4)}
     # HBM traffic per launch of the dominant kernel, from the FETCH_SIZE / WRITE_SIZE runs summarised in
     # profiles/mixtral_hbm_traffic.txt (bytes; only measured for the default workload)
-    measured_traffic = {"mixtral": 12.49e9}
+    measured_traffic = {"mixtral": 12.52e9}
     dom = "mlp_up"  # the gate/up grouped GEMM: most of the flops of a step
     if cfg.quant == "fp8":
         kname = "moe_grouped_mlp_fp8 (row quantisation + gate/up GEMM + SwiGLU + re-quantisation + down GEMM)"

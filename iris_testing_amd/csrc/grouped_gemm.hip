@@ -434,15 +434,20 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             if constexpr (FP8) rs[i] = p.row_scale[grow];
             crow[i] = C + (p.c_map ? (size_t)p.c_map[grow] : grow) * p.ldc;
         }
+        float4 sc0[NQ], sc1[NQ];  // fp8: channel scales of the lane's columns (gate / only; up)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
+        for (int o = 0; o < TM * TN; ++o) {
+            // fp8: column tiles outermost (the channel scales of a column tile are fetched once and serve the
+            // wave's TM row tiles); bf16: row tiles outermost, so that the stores of one row tile fill whole
+            // cache lines back to back (the other order wrote 50 % more bytes to memory: lines left the L2
+            // half written)
+            const int i = FP8 ? o % TM : o / TN, j = FP8 ? o / TM : o % TN;
             if constexpr (EPI == EPI_SWIGLU) {
                 if ((j / UPJ) % 2 == 1) continue;  // an up tile: consumed together with its gate tile
             }
             const int pcol = nt * BN + wn * (BN / 2) + j * MT;  // first packed column of the tile
             const int colj = (EPI == EPI_SWIGLU ? (pcol / 64) * 32 + pcol % 32 : pcol) + clane;
-            float4 sc0[NQ], sc1[NQ];  // fp8: channel scales of the lane's columns (gate / only; up)
-            if constexpr (FP8) {
+            if (FP8 && i == 0) {
 #pragma unroll
                 for (int q = 0; q < NQ; ++q) {
                     const int col = colj + 8 * q;
@@ -453,8 +458,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                     }
                 }
             }
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
+            {
 #pragma unroll
                 for (int q = 0; q < NQ; ++q) {
                     const int col = colj + 8 * q;
@@ -493,7 +497,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                 }
                 // keep the accumulator read-out of one tile from being hoisted over the previous tile's stores
                 // (that would need every accumulator in a VGPR at once)
-                if (FP8 || (i % 2 == 1)) __builtin_amdgcn_sched_barrier(0);
+                if (FP8 || (o % 2 == 1)) __builtin_amdgcn_sched_barrier(0);
             }
         }
         cur = nxt;
