@@ -93,6 +93,14 @@ int moe_pack(const void* x, int dtype, int T, int H, const int32_t* row_token, c
              const int32_t* dst_offsets, int W, int M, void* send_buf, int32_t* map_ws, int32_t* status,
              moe_stream_t stream);
 
+/* The same send buffer, written token by token: every token row is read once and stored to the k slots
+ * send[dst,m,:] with dst = topk_idx[t,kk] / E_l, m = pos[t,kk] - dst_offsets[dst] (pos as returned by
+ * moe_count_and_offsets), padding rows zeroed; bit-identical to moe_pack with k times fewer token reads.
+ * Restates the same README.md:5-7 layout from the per-token side of utils.py:210-219. */
+int moe_pack_tokens(const void* x, int dtype, int T, int H, const int32_t* topk_idx, const int32_t* pos, int k,
+                    int E_l, const int32_t* dst_sizes, const int32_t* dst_offsets, int W, int M, void* send_buf,
+                    int32_t* status, moe_stream_t stream);
+
 /* ---- a9: receive layout (reference baseline.py:178-222; kernels.py:93-102,124-125) ------------
  * recv [W,M,H]: slot s holds what source s sent to this rank ((el, token) order, zero padded);
  * recv_counts [W,E_l]: recv_counts[s,e] rows from source s for local expert e.

@@ -39,6 +39,7 @@ _SIGNATURES = {
     "moe_max_floor1": (c_int, [P, c_int, P, P]),
     "moe_pack_payload": (c_int, [P, c_int, c_int, c_int, P, c_int, P, P]),
     "moe_pack": (c_int, [P, c_int, c_int, c_int, P, P, P, c_int, c_int, P, P, P, P]),
+    "moe_pack_tokens": (c_int, [P, c_int, c_int, c_int, P, P, c_int, c_int, P, P, c_int, c_int, P, P, P]),
     "moe_recv_map_ints": (c_size_t, [c_int, c_int, c_int]),
     "moe_unpack_token_buf": (c_int, [P, c_int, c_int, c_int, c_int, P, c_int, c_int, P, P, P, P, P]),
     "moe_reorder_flat_to_token_buf": (c_int, [P, c_int, c_int, c_int, P, c_int, c_int, c_int, P, P, P, P]),

@@ -312,6 +312,63 @@ __global__ __launch_bounds__(WPB * WAVE) void gather_rows_kernel(const u32x4* __
     }
 }
 
+// ---- pack, token-major: every token row is read once and stored to its k send slots ------------------
+// Rows [0, T) of the launch are tokens, rows [T, T + W*M) are send slots that only get zeros when they are
+// padding.  Same bytes in send_buf as the slot-major gather (SRC_PACK), with x read once instead of k times.
+template <int WPB>
+__global__ __launch_bounds__(WPB * WAVE) void pack_tokens_kernel(const u32x4* __restrict__ x, u32x4* __restrict__ send,
+                                                                  const int32_t* __restrict__ idx, const int32_t* __restrict__ pos,
+                                                                  const int32_t* __restrict__ dst_sizes,
+                                                                  const int32_t* __restrict__ dst_offsets, int T, int k, int E_l,
+                                                                  int W, int M, int row_vec, int32_t* __restrict__ status) {
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const int n_rows = T + W * M;
+    for (int r = blockIdx.x * WPB + wave; r < n_rows; r += gridDim.x * WPB) {
+        if (r >= T) {
+            const int d = (r - T) / M, m = (r - T) % M;
+            const int cnt = dst_sizes[d];
+            if (m == 0 && cnt > M && status && lane == 0) *status = 1;
+            if (m < cnt) continue;
+            u32x4* o = send + (size_t)(r - T) * row_vec;
+            const u32x4 z = {0u, 0u, 0u, 0u};
+            for (int c = lane; c < row_vec; c += WAVE) __builtin_nontemporal_store(z, o + c);
+            continue;
+        }
+        // destination rows of the token's k slots (-1: beyond the pair capacity, dropped like the gather drops it)
+        int drow[MOE_MAX_TOPK];
+#pragma unroll
+        for (int j = 0; j < MOE_MAX_TOPK; ++j) {
+            drow[j] = -1;
+            if (j < k) {
+                const int d = idx[(size_t)r * k + j] / E_l;
+                const int m = pos[(size_t)r * k + j] - dst_offsets[d];
+                if ((unsigned)d < (unsigned)W && (unsigned)m < (unsigned)M) drow[j] = d * M + m;
+            }
+        }
+        const u32x4* src = x + (size_t)r * row_vec;
+        int c = lane;
+        for (; c + 7 * WAVE < row_vec; c += 8 * WAVE) {
+            u32x4 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(src + c + u * WAVE);
+#pragma unroll
+            for (int j = 0; j < MOE_MAX_TOPK; ++j) {
+                if (j < k && drow[j] >= 0) {
+                    u32x4* o = send + (size_t)drow[j] * row_vec + c;
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) __builtin_nontemporal_store(v[u], o + u * WAVE);
+                }
+            }
+        }
+        for (; c < row_vec; c += WAVE) {
+            const u32x4 v = __builtin_nontemporal_load(src + c);
+#pragma unroll
+            for (int j = 0; j < MOE_MAX_TOPK; ++j)
+                if (j < k && drow[j] >= 0) __builtin_nontemporal_store(v, send + (size_t)drow[j] * row_vec + c);
+        }
+    }
+}
+
 // ---- combine: out[t,:] = sum_kk gate[t,kk] * ret[slot(t,kk),:] --------------------------------------
 template <typename XT>
 struct Vec16;
@@ -368,7 +425,11 @@ __global__ __launch_bounds__(WPB * WAVE) void combine_kernel(const uint4* __rest
             uint4 v[KMAX];
 #pragma unroll
             for (int j = 0; j < KMAX; ++j)
-                if (j < k) v[j] = ret[rows[j] + c];
+                if (j < k) {
+                    // every returned row is read once: no cache retention wanted
+                    const u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(ret + rows[j] + c));
+                    v[j] = make_uint4(raw.x, raw.y, raw.z, raw.w);
+                }
             float acc[N];
 #pragma unroll
             for (int i = 0; i < N; ++i) acc[i] = 0.f;
@@ -381,7 +442,9 @@ __global__ __launch_bounds__(WPB * WAVE) void combine_kernel(const uint4* __rest
                     for (int i = 0; i < N; ++i) acc[i] = __fadd_rn(acc[i], __fmul_rn(g[j], f[i]));
                 }
             }
-            out[(size_t)t * row_vec + c] = Vec16<XT>::pack(acc);
+            const uint4 o = Vec16<XT>::pack(acc);
+            const u32x4 ov = {o.x, o.y, o.z, o.w};
+            __builtin_nontemporal_store(ov, reinterpret_cast<u32x4*>(out + (size_t)t * row_vec + c));
         }
     }
 }
@@ -534,6 +597,24 @@ extern "C" int moe_pack(const void* x, int dtype, int T, int H, const int32_t* r
     a.M = M;
     a.status = status;
     return gather_rows(x, send_buf, a, W * M, H * dtype_size(dtype), s);
+}
+
+extern "C" int moe_pack_tokens(const void* x, int dtype, int T, int H, const int32_t* topk_idx, const int32_t* pos, int k,
+                               int E_l, const int32_t* dst_sizes, const int32_t* dst_offsets, int W, int M, void* send_buf,
+                               int32_t* status, moe_stream_t stream) {
+    int rc = check_rows("pack_tokens", dtype, H);
+    if (rc) return rc;
+    MOE_REQUIRE(W > 0 && M >= 1 && T >= 0 && E_l > 0, MOE_ERR_INVALID, "pack_tokens: bad shape W=%d M=%d E_l=%d", W, M, E_l);
+    MOE_REQUIRE(k >= 1 && k <= MOE_MAX_TOPK, MOE_ERR_UNSUPPORTED, "pack_tokens: topk=%d outside [1,%d]", k, MOE_MAX_TOPK);
+    MOE_REQUIRE((long long)W * M + T < (1ll << 31), MOE_ERR_UNSUPPORTED, "pack_tokens: W*M + T too large");
+    MOE_REQUIRE(send_buf && dst_sizes && dst_offsets, MOE_ERR_INVALID, "pack_tokens: null pointer");
+    MOE_REQUIRE(T == 0 || (x && topk_idx && pos), MOE_ERR_INVALID, "pack_tokens: null pointer");
+    const int n_rows = T + W * M;
+    const int blocks = min(ceil_div(n_rows, 4), 65535 * 8);
+    pack_tokens_kernel<4><<<blocks, 4 * WAVE, 0, (hipStream_t)stream>>>((const u32x4*)x, (u32x4*)send_buf, topk_idx, pos, dst_sizes,
+                                                                        dst_offsets, T, k, E_l, W, M,
+                                                                        H * dtype_size(dtype) / 16, status);
+    return moe_check_launch("pack_tokens");
 }
 
 static int recv_driven(const char* who, int mode, const void* src, void* dst, int dtype, int H, const int32_t* rc_dev,

@@ -116,6 +116,27 @@ def pack_fixed_m(x: torch.Tensor, row_token: torch.Tensor, dst_sizes: torch.Tens
     return out
 
 
+def pack_tokens(x: torch.Tensor, topk_idx: torch.Tensor, pos: torch.Tensor, dst_sizes: torch.Tensor,
+                dst_offsets: torch.Tensor, e_local: int, M: int, out: Optional[torch.Tensor] = None,
+                status: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The send buffer of pack_fixed_m written token by token (every token row read once, stored k times)."""
+    _req_cuda(x, "tokens")
+    _req_i32(topk_idx, "topk_idx")
+    _req_i32(pos, "pos")
+    _req_i32(dst_sizes, "dst_sizes")
+    _req_i32(dst_offsets, "dst_offsets")
+    T, H = x.shape
+    W = dst_sizes.numel()
+    k = topk_idx.shape[1] if topk_idx.dim() == 2 else 1
+    assert topk_idx.numel() == T * k and pos.numel() == T * k
+    if out is None:
+        out = torch.empty((W, M, H), dtype=x.dtype, device=x.device)
+    assert out.shape == (W, M, H) and out.dtype == x.dtype and out.is_contiguous()
+    L.check(L.lib().moe_pack_tokens(L.ptr(x), L.dtype_code(x.dtype), T, H, L.ptr(topk_idx), L.ptr(pos), k, e_local,
+                                    L.ptr(dst_sizes), L.ptr(dst_offsets), W, M, L.ptr(out), L.ptr(status), L.stream_ptr()))
+    return out
+
+
 # ---- a9 / a10 -------------------------------------------------------------------------------
 def _map_ws(W, E_l, n_out, device, map_ws=None):
     need = L.lib().moe_recv_map_ints(W, E_l, n_out)

@@ -87,9 +87,9 @@ class DispatchPipeline:
 
     def pack(self, s):
         c, w = self.cfg, self.world
-        L.check(L.lib().moe_pack(self._p(w.x0), self.code, c.tokens, c.hidden, self._p(self.row_token),
-                                 self._p(self.dst_sizes), self._p(self.dst_offsets), c.world, w.M, self._p(self.send),
-                                 None, self._p(self.status), s))
+        L.check(L.lib().moe_pack_tokens(self._p(w.x0), self.code, c.tokens, c.hidden, self._p(self.idx), self._p(self.pos),
+                                        c.topk, c.e_local, self._p(self.dst_sizes), self._p(self.dst_offsets), c.world, w.M,
+                                        self._p(self.send), self._p(self.status), s))
 
     def unpack(self, s):
         c, w = self.cfg, self.world

@@ -70,6 +70,11 @@ def test_route_count_pack_bit_exact(name, tokens):
     send = ops.pack_fixed_m(xd, c.row_token, c.dst_sizes, c.dst_offsets, M, status=status)
     assert_bits_equal(send, O.pack_fixed_m(o_payload, o_offs, o_sizes, M), "send [W,M,H]")
     assert int(status.item()) == 0
+    # the token-major writer of the same buffer (each token row read once), into a buffer full of garbage
+    send2 = torch.full_like(send, 3.0)
+    ops.pack_tokens(xd, idx, c.pos, c.dst_sizes, c.dst_offsets, cfg.e_local, M, out=send2, status=status)
+    assert_bits_equal(send2, O.pack_fixed_m(o_payload, o_offs, o_sizes, M), "send [W,M,H], token-major")
+    assert int(status.item()) == 0
 
 
 def test_route_ties_prefer_lower_expert():
@@ -122,6 +127,14 @@ def test_zero_tokens_and_overflow_flag():
                      status=status)
     assert int(status.item()) == 1
     assert (guard[cfg.world * M:] == 7.0).all()
+    kept = guard[:cfg.world * M].clone()
+    status.zero_()
+    guard.fill_(7.0)
+    ops.pack_tokens(xd, idx, c.pos, c.dst_sizes, c.dst_offsets, cfg.e_local, M,
+                    out=guard[:cfg.world * M].view(cfg.world, M, -1), status=status)
+    assert int(status.item()) == 1
+    assert (guard[cfg.world * M:] == 7.0).all()
+    assert torch.equal(guard[:cfg.world * M], kept), "token-major pack drops the same rows as the slot-major one"
 
 
 UNPACK_CASES = [("plumbing", None), ("small", None), ("mixtral", 1024), ("finegrained", 512), ("zipf_k4", 1024)]
