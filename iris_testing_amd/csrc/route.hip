@@ -6,16 +6,16 @@
 //
 // Reduction order (what makes the indices reproducible bit-for-bit on a CPU):
 //   logit[t,e] = bias[e] + chain,  chain = fmaf(x[t,h], w[h,e], chain) for h = 0..H-1, chain0 = +0.0f
-// Every (t,e) chain lives in ONE thread; H is walked in ascending order through LDS tiles, so no
-// cross-lane or cross-block partial sums exist.  MFMA is deliberately not used here: its internal
-// summation order is not specified.
+// Every (t,e) chain is one accumulator element walked over H in ascending order, so no cross-lane or
+// cross-block partial sums exist.  The chains run on the matrix cores, but only through K = 1 fp32 MFMAs,
+// which perform exactly one fused multiply-add per output element and instruction; MFMAs with K > 1 (and all
+// bf16 ones) sum several products in an order that is not specified and are not used.
 #include "common.h"
+#include <type_traits>
 
 namespace {
 
-constexpr int RT_THREADS = 256;
-constexpr int RT_KC = 32;  // h per LDS tile
-constexpr int RT_TB = 64;  // tokens per block
+constexpr int RT_TB = 64;  // tokens per block: one per lane
 
 template <typename XT>
 struct VecLoad;
@@ -41,236 +41,188 @@ struct VecLoad<float> {
     }
 };
 
-// Block = 256 threads = NEX expert-threads x NTY token-threads; thread computes TT tokens x EE experts.
-template <typename XT, int TT, int EE, int NEX>
-__global__ __launch_bounds__(RT_THREADS) void route_logits_kernel(const XT* __restrict__ x,
-                                                                   const XT* __restrict__ w,
-                                                                   const float* __restrict__ bias,
-                                                                   float* __restrict__ logits, int T, int H, int E) {
-    constexpr int NTY = RT_THREADS / NEX;
-    constexpr int TB = NTY * TT;
-    constexpr int EB = NEX * EE;
-    static_assert(TB == RT_TB, "token tile");
-    constexpr int XS = TB + 4;  // padded row stride (keeps 16-byte alignment of the per-thread token vector)
-    __shared__ __align__(16) float xs[RT_KC][XS];
-    __shared__ __align__(16) float ws[RT_KC][EB];
+// ---- logits on the matrix cores, still one fused multiply-add per (t, e, h) in ascending h -------------
+// A K = 1 fp32 MFMA (v_mfma_f32_16x16x1_4b_f32, v_mfma_f32_4x4x1_16b_f32) performs, for every output element,
+// exactly one D = fma(a, b, C) with a single rounding -- the same operation, bit for bit (subnormals
+// included), as a v_fma_f32 or the fmaf of a CPU (checked on the GPU against fmaf chains over normal, wide-range,
+// subnormal and bf16-valued operands); it runs the chains of 64 tokens x SHAPE experts in one instruction, at
+// up to twice the vector rate, and takes its operands from two registers instead of 64 x SHAPE LDS reads.
+//   A operand: lane l holds x[t0 + l][h]                 (lane = token: the wave's 64 tokens)
+//   B operand: lane l holds w[h][e0 + l % SHAPE]         (the SHAPE experts, repeated across the lanes)
+//   D, SHAPE = 16: register v holds token t0 + 16 * (v / 4) + 4 * (l / 16) + v % 4, expert e0 + l % 16
+//   D, SHAPE = 4:  register v holds token t0 + 4 * (l / 4) + v,                     expert e0 + l % 4
+// Block = NWV waves on the same 64 tokens, wave i on experts [e0 + i * SHAPE, + SHAPE).  x goes through LDS in
+// its storage type (the lane reads its own row, 16 bytes at a time), the router slab is converted to fp32 and
+// transposed on its way into LDS (the lane reads four consecutive h of its expert with one 128-bit read).
+typedef float rt_f4 __attribute__((ext_vector_type(4)));
+typedef float rt_f16 __attribute__((ext_vector_type(16)));
+typedef unsigned int rt_u4 __attribute__((ext_vector_type(4)));
 
-    const int tid = threadIdx.x;
-    const int tx = tid % NEX, ty = tid / NEX;
-    const int t0 = blockIdx.x * TB, e0 = blockIdx.y * EB;
-
-    float acc[TT][EE];
-#pragma unroll
-    for (int i = 0; i < TT; ++i)
-#pragma unroll
-        for (int j = 0; j < EE; ++j) acc[i][j] = 0.0f;
-
-    constexpr int VN = VecLoad<XT>::N;
-    constexpr int CH_PER_TOK = RT_KC / VN;
-    constexpr int X_CHUNKS = TB * CH_PER_TOK;
-    constexpr int XPT = (X_CHUNKS + RT_THREADS - 1) / RT_THREADS;
-    constexpr int WPT = RT_KC * EB / RT_THREADS;
-    static_assert(X_CHUNKS % RT_THREADS == 0 && (RT_KC * EB) % RT_THREADS == 0, "staging split");
-
-    // The next slab is fetched into registers (from clamped, always valid addresses) while the current one
-    // is consumed; masking and conversion to fp32 happen when it is written to LDS.
-    uint4 xr[XPT];
-    XT wr[WPT];
-    auto fetch = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < XPT; ++i) {
-            const int c = tid + i * RT_THREADS;
-            const int tt = c / CH_PER_TOK, kc = (c % CH_PER_TOK) * VN;
-            xr[i] = *reinterpret_cast<const uint4*>(x + (size_t)min(t0 + tt, T - 1) * H + min(k0 + kc, H - VN));
-        }
-#pragma unroll
-        for (int i = 0; i < WPT; ++i) {
-            const int c = tid + i * RT_THREADS;
-            wr[i] = w[(size_t)min(k0 + c / EB, H - 1) * E + min(e0 + c % EB, E - 1)];
-        }
-    };
-    auto stash = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < XPT; ++i) {
-            const int c = tid + i * RT_THREADS;
-            const int tt = c / CH_PER_TOK, kc = (c % CH_PER_TOK) * VN;
-            const bool ok = t0 + tt < T && k0 + kc < H;
-            float v[VN];
-            VecLoad<XT>::unpack(xr[i], v);
-#pragma unroll
-            for (int j = 0; j < VN; ++j) xs[kc + j][tt] = ok ? v[j] : 0.0f;
-        }
-#pragma unroll
-        for (int i = 0; i < WPT; ++i) {
-            const int c = tid + i * RT_THREADS;
-            const bool ok = k0 + c / EB < H && e0 + c % EB < E;
-            ws[c / EB][c % EB] = ok ? load_f32<XT>(&wr[i]) : 0.0f;
-        }
-    };
-
-    constexpr int UK = 8;  // h per inner step: all LDS reads of the step are issued before its fmaf chains
-    fetch(0);
-    for (int k0 = 0; k0 < H; k0 += RT_KC) {
-        stash(k0);
-        __syncthreads();
-        if (k0 + RT_KC < H) fetch(k0 + RT_KC);
-        const int kmax = min(RT_KC, H - k0);
-        int kk = 0;
-        for (; kk + UK <= kmax; kk += UK) {
-            float xv[UK][TT], wv[UK][EE];
-#pragma unroll
-            for (int u = 0; u < UK; ++u) {
-#pragma unroll
-                for (int i = 0; i < TT; ++i) xv[u][i] = xs[kk + u][ty * TT + i];
-#pragma unroll
-                for (int j = 0; j < EE; ++j) wv[u][j] = ws[kk + u][tx * EE + j];
-            }
-#pragma unroll
-            for (int u = 0; u < UK; ++u)
-#pragma unroll
-                for (int i = 0; i < TT; ++i)
-#pragma unroll
-                    for (int j = 0; j < EE; ++j) acc[i][j] = fmaf(xv[u][i], wv[u][j], acc[i][j]);
-        }
-        for (; kk < kmax; ++kk) {
-#pragma unroll
-            for (int i = 0; i < TT; ++i)
-#pragma unroll
-                for (int j = 0; j < EE; ++j) acc[i][j] = fmaf(xs[kk][ty * TT + i], ws[kk][tx * EE + j], acc[i][j]);
-        }
-        __syncthreads();
-    }
-#pragma unroll
-    for (int i = 0; i < TT; ++i) {
-        const int t = t0 + ty * TT + i;
-        if (t >= T) continue;
-#pragma unroll
-        for (int j = 0; j < EE; ++j) {
-            const int e = e0 + tx * EE + j;
-            if (e < E) logits[(size_t)t * E + e] = bias ? __fadd_rn(acc[i][j], bias[e]) : acc[i][j];
-        }
-    }
-}
-
-// Few experts (E <= 16): one thread per (token, EE experts).  Lane = token (64 tokens per block), wave w
-// owns experts [w*EE, w*EE+EE).  x goes through LDS in its storage type (the lane reads its own row 16
-// bytes at a time); the router slab is converted to fp32 once per slab and read back with broadcast
-// 128-bit LDS reads.  The next slab is fetched into registers while the current one is consumed.
-// Same reduction order as above: one fmaf chain per (t,e), ascending h.
-constexpr int RS_KC = 128;
-
-template <typename XT, int EE>
-__global__ __launch_bounds__(RT_THREADS) void route_logits_small_kernel(const XT* __restrict__ x, const XT* __restrict__ w,
-                                                                         const float* __restrict__ bias,
-                                                                         float* __restrict__ logits, int T, int H, int E) {
-    constexpr int VN = VecLoad<XT>::N;          // elements per 16 bytes
-    constexpr int XS = RS_KC + VN;              // padded row (16 bytes of padding: conflict-free b128 rows)
-    constexpr int XCH = RT_TB * (RS_KC / VN);   // 16-byte chunks of an x slab
-    constexpr int XPT = XCH / RT_THREADS;       // per thread
-    constexpr int WPT = 16 * RS_KC / RT_THREADS;  // router elements per thread per slab (16 expert rows)
+template <typename XT, int SHAPE, int NWV>
+__global__ __launch_bounds__(NWV * WAVE) void route_logits_mfma_kernel(const XT* __restrict__ x, const XT* __restrict__ w,
+                                                                        const float* __restrict__ bias,
+                                                                        float* __restrict__ logits, int T, int H, int E) {
+    static_assert(SHAPE == 4 || SHAPE == 16, "experts per MFMA");
+    constexpr int NTH = NWV * WAVE;
+    constexpr int EB = NWV * SHAPE;            // experts per block
+    constexpr int VN = VecLoad<XT>::N;         // elements per 16 bytes
+    constexpr int KC = 16 * VN;                // h per slab: 256 bytes of every token row
+    constexpr int XS = KC + VN;                // padded row (conflict-free 128-bit row reads)
+    constexpr int XPT = RT_TB * 16 / NTH;      // 16-byte x chunks per thread and slab
+    constexpr int WQ = KC * EB / (4 * NTH);    // groups of four h of one expert per thread and slab
+    // slabs in flight per block: one block holds D x 16 KB of token rows in registers, which is what hides the
+    // memory latency when there is only one block of 64 tokens per compute unit
+    constexpr int D = NWV == 1 ? 2 : 4;
+    constexpr int NACC = SHAPE == 16 ? 16 : 4;
+    typedef typename std::conditional<SHAPE == 16, rt_f16, rt_f4>::type acc_t;
+    static_assert((KC * EB) % (4 * NTH) == 0, "router slab split");
     __shared__ __align__(16) XT xs[RT_TB][XS];
-    __shared__ __align__(16) float wsT[16][RS_KC + 4];
+    __shared__ __align__(16) float wsT[EB][KC + 4];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int t0 = blockIdx.x * RT_TB;
-    const int e0 = wave * EE;
-    float acc[EE];
+    const int t0 = blockIdx.x * RT_TB, eb0 = blockIdx.y * EB;
+    const float* wrow = &wsT[wave * SHAPE + lane % SHAPE][0];
+    const XT* xrow = &xs[lane][0];
+    acc_t acc;
 #pragma unroll
-    for (int j = 0; j < EE; ++j) acc[j] = 0.f;
+    for (int v = 0; v < NACC; ++v) acc[v] = 0.f;
 
-    // raw slab data held in registers while the previous slab is consumed; masking and conversion
-    // happen when it is written to LDS, so nothing waits on these loads until then
-    uint4 xr[XPT];
-    XT wr[WPT];
-    auto fetch = [&](int k0) {
+    // Slab s covers h in [ks, ks + KC), ks = min(s * KC, H - KC) (0 when H < KC): the last slab of a row whose
+    // length is no multiple of KC overlaps its predecessor and is consumed from offset s * KC - ks on; slabs past
+    // the end repeat it and are not consumed at all.  So every slab is a full, in-bounds fetch from a block-uniform
+    // base plus lane offsets that never change (the clamps below only matter for H < KC, T and E tails).
+    const int ks_max = max(H - KC, 0);
+    int xoff[XPT], woff[WQ][4];
 #pragma unroll
-        for (int i = 0; i < XPT; ++i) {
-            const int c = tid + i * RT_THREADS;
-            const int row = c / (RS_KC / VN), col = (c % (RS_KC / VN)) * VN;
-            // clamped (always valid) address: no divergent branch, all loads of a slab in flight together
-            xr[i] = *reinterpret_cast<const uint4*>(x + (size_t)min(t0 + row, T - 1) * H + min(k0 + col, H - VN));
-        }
+    for (int i = 0; i < XPT; ++i) {
+        const int c = tid + i * NTH;
+        xoff[i] = min(c / 16, T - 1 - t0) * H + min((c % 16) * VN, H - VN);
+    }
 #pragma unroll
-        for (int i = 0; i < WPT; ++i) {
-            const int c = tid + i * RT_THREADS;
-            wr[i] = w[(size_t)min(k0 + c / 16, H - 1) * E + min(c % 16, E - 1)];
-        }
-    };
-    auto stash = [&](int k0) {
+    for (int i = 0; i < WQ; ++i) {
+        const int c = tid + i * NTH;  // expert c % EB, h 4 * (c / EB) .. + 3 of the slab
 #pragma unroll
-        for (int i = 0; i < XPT; ++i) {
-            const int c = tid + i * RT_THREADS;
-            const int row = c / (RS_KC / VN), col = (c % (RS_KC / VN)) * VN;
-            const bool ok = t0 + row < T && k0 + col < H;
-            *reinterpret_cast<uint4*>(&xs[row][col]) =
-                make_uint4(ok ? xr[i].x : 0u, ok ? xr[i].y : 0u, ok ? xr[i].z : 0u, ok ? xr[i].w : 0u);
-        }
-#pragma unroll
-        for (int i = 0; i < WPT; ++i) {
-            const int c = tid + i * RT_THREADS;
-            const bool ok = k0 + c / 16 < H && c % 16 < E;
-            wsT[c % 16][c / 16] = ok ? load_f32<XT>(&wr[i]) : 0.f;
-        }
-    };
+        for (int q = 0; q < 4; ++q) woff[i][q] = min(4 * (c / EB) + q, H - 1) * E + min(eb0 + c % EB, E - 1);
+    }
+    const XT* xblk = x + (size_t)t0 * H;
 
-    constexpr int UN = 4;  // 16-byte x chunks consumed per inner step
-    fetch(0);
-    for (int k0 = 0; k0 < H; k0 += RS_KC) {
-        stash(k0);
-        __syncthreads();
-        if (k0 + RS_KC < H) fetch(k0 + RS_KC);
-        const int kmax = min(RS_KC, H - k0);
-        int kk = 0;
-        for (; kk + UN * VN <= kmax; kk += UN * VN) {
-            // all LDS reads of the step first, then the fmaf chains in ascending h
-            uint4 xraw[UN];
-            float4 wv[EE][UN * VN / 4];
+    // slabs wait in registers until their turn in LDS
+    rt_u4 xr[D][XPT];  // (vector types, not HIP's uint4 struct: the arrays must stay in registers)
+    XT wr[D][WQ][4];
+#define RT_FETCH(d, k0)                                                                                      \
+    do {                                                                                                     \
+        const int ks_ = min((k0), ks_max);                                                                   \
+        const XT* xb_ = xblk + ks_;                                                                          \
+        const XT* wb_ = w + (size_t)ks_ * E;                                                                 \
+        _Pragma("unroll") for (int i = 0; i < XPT; ++i) xr[d][i] = *reinterpret_cast<const rt_u4*>(xb_ + xoff[i]); \
+        _Pragma("unroll") for (int i = 0; i < WQ; ++i)                                                        \
+            _Pragma("unroll") for (int q = 0; q < 4; ++q) wr[d][i][q] = wb_[woff[i][q]];                      \
+    } while (0)
+    // registers -> LDS: token rows as they are, the router slab as fp32, transposed (one 128-bit write per four h)
+#define RT_STASH(d)                                                                                                  \
+    do {                                                                                                             \
+        _Pragma("unroll") for (int i = 0; i < XPT; ++i) {                                                             \
+            const int c = tid + i * NTH;                                                                             \
+            *reinterpret_cast<rt_u4*>(&xs[c / 16][(c % 16) * VN]) = xr[d][i];                                        \
+        }                                                                                                            \
+        _Pragma("unroll") for (int i = 0; i < WQ; ++i) {                                                              \
+            const int c = tid + i * NTH;                                                                             \
+            const rt_f4 v = {load_f32<XT>(&wr[d][i][0]), load_f32<XT>(&wr[d][i][1]), load_f32<XT>(&wr[d][i][2]),     \
+                             load_f32<XT>(&wr[d][i][3])};                                                            \
+            *reinterpret_cast<rt_f4*>(&wsT[c % EB][4 * (c / EB)]) = v;                                               \
+        }                                                                                                            \
+    } while (0)
+
+    // One chunk = VN consecutive h (16 bytes of the lane's token row): VN chained MFMAs.  Within one wave a
+    // vector instruction does not overlap the chain (measured: one VALU between two dependent MFMAs adds 12 to 14
+    // cycles, a second one 8 more), so the conversions and LDS reads are not spread between the MFMAs but issued
+    // as one group ahead of them: token bytes are read two chunks ahead and converted one chunk ahead, router
+    // values are read one chunk ahead, and nothing in the chain waits for LDS.
+#define RT_MFMA(XV, WV, u)                                                                                           \
+    do {                                                                                                             \
+        if constexpr (SHAPE == 16) acc = __builtin_amdgcn_mfma_f32_16x16x1f32(XV[u], WV[(u) / 4][(u) % 4], acc, 0, 0, 0); \
+        else acc = __builtin_amdgcn_mfma_f32_4x4x1f32(XV[u], WV[(u) / 4][(u) % 4], acc, 0, 0, 0);                    \
+        __builtin_amdgcn_sched_barrier(0);                                                                           \
+    } while (0)
+    // (an empty asm statement that "modifies" a value keeps its computation where it is written: it would
+    // otherwise sink to its first use, out of the shadow of the MFMAs)
+#define RT_PIN(a) asm volatile("" : "+v"(a))
+    // element u of a 16-byte piece of a token row as fp32
+#define RT_CVT(RAW, u) (VN == 8 ? __uint_as_float(((u) & 1) ? (RAW[(u) / 2] & 0xffff0000u) : (RAW[(u) / 2] << 16)) : __uint_as_float(RAW[(u) & 3]))
+    // chunk c: MFMAs on XV / WV; meanwhile RAWN (chunk c+1, read one chunk ago) is converted into XN, the router
+    // values of chunk c+1 are read into WN and the token bytes of chunk c+2 into RAWF
+#define RT_CHUNK(XV, WV, XN, WN, RAWN, RAWF, nxt1, nxt2)                                                             \
+    do {                                                                                                             \
+        RAWF = *reinterpret_cast<const rt_u4*>(xrow + (nxt2));                                                       \
+        WN[0] = *reinterpret_cast<const rt_f4*>(wrow + (nxt1));                                                      \
+        if constexpr (VN == 8) WN[1] = *reinterpret_cast<const rt_f4*>(wrow + (nxt1) + 4);                           \
+        _Pragma("unroll") for (int u_ = 0; u_ < VN; ++u_) { XN[u_] = RT_CVT(RAWN, u_); RT_PIN(XN[u_]); }             \
+        __builtin_amdgcn_sched_barrier(0);                                                                           \
+        RT_MFMA(XV, WV, 0); RT_MFMA(XV, WV, 1); RT_MFMA(XV, WV, 2); RT_MFMA(XV, WV, 3);                              \
+        if constexpr (VN == 8) { RT_MFMA(XV, WV, 4); RT_MFMA(XV, WV, 5); RT_MFMA(XV, WV, 6); RT_MFMA(XV, WV, 7); }   \
+    } while (0)
+
+    // Every slab slot is fetched and stashed unconditionally (no branch around a load: the compiler then knows how
+    // many younger loads are in flight at each stash and waits only for the slab it needs).  The fences keep the
+    // first loads in slab order: the scheduler would otherwise issue them last slab first.
 #pragma unroll
-            for (int u = 0; u < UN; ++u) xraw[u] = *reinterpret_cast<const uint4*>(&xs[lane][kk + u * VN]);
+    for (int d = 0; d < D; ++d) {
+        RT_FETCH(d, d * KC);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    for (int kb = 0; kb < H; kb += D * KC) {
 #pragma unroll
-            for (int j = 0; j < EE; ++j)
+        for (int d = 0; d < D; ++d) {
+            const int k0 = kb + d * KC;
+            RT_STASH(d);
+            __syncthreads();
+            RT_FETCH(d, k0 + D * KC);
+            // only the h that exist take part: a padded step would add +0 and could turn a -0 chain into +0
+            const int sh = k0 - min(k0, ks_max);        // where h = k0 sits in the slab
+            const int kend = sh + max(min(KC, H - k0), 0);
+            if (sh < kend) {
+                float xa[VN], xb[VN];
+                rt_f4 wa[2], wb[2];
+                rt_u4 ra, rb;
+                {
+                    ra = *reinterpret_cast<const rt_u4*>(xrow + sh);
+                    rb = *reinterpret_cast<const rt_u4*>(xrow + min(sh + VN, KC - VN));
 #pragma unroll
-                for (int q = 0; q < UN * VN / 4; ++q) wv[j][q] = *reinterpret_cast<const float4*>(&wsT[e0 + j][kk + 4 * q]);
+                    for (int q = 0; q < VN / 4; ++q) wa[q] = *reinterpret_cast<const rt_f4*>(wrow + sh + 4 * q);
 #pragma unroll
-            for (int u = 0; u < UN; ++u) {
-                float xv[VN];
-                VecLoad<XT>::unpack(xraw[u], xv);
-#pragma unroll
-                for (int q = 0; q < VN; q += 4) {
-#pragma unroll
-                    for (int j = 0; j < EE; ++j) {
-                        const float4 wq = wv[j][(u * VN + q) / 4];
-                        acc[j] = fmaf(xv[q + 0], wq.x, acc[j]);
-                        acc[j] = fmaf(xv[q + 1], wq.y, acc[j]);
-                        acc[j] = fmaf(xv[q + 2], wq.z, acc[j]);
-                        acc[j] = fmaf(xv[q + 3], wq.w, acc[j]);
+                    for (int u = 0; u < VN; ++u) xa[u] = RT_CVT(ra, u);
+                }
+                if (sh == 0 && kend == KC) {
+                    // a whole slab: sixteen chunks of straight-line code (reads past the last chunk repeat it)
+#define RT_PAIR(c) /* chunks c (even) and c + 1 */                                                                    \
+    RT_CHUNK(xa, wa, xb, wb, rb, ra, ((c) + 1) * VN, ((c) + 2 < 16 ? (c) + 2 : 15) * VN);                              \
+    RT_CHUNK(xb, wb, xa, wa, ra, rb, ((c) + 2 < 16 ? (c) + 2 : 15) * VN, ((c) + 3 < 16 ? (c) + 3 : 15) * VN)
+                    RT_PAIR(0); RT_PAIR(2); RT_PAIR(4); RT_PAIR(6); RT_PAIR(8); RT_PAIR(10); RT_PAIR(12); RT_PAIR(14);
+#undef RT_PAIR
+                } else {
+                    for (int kk = sh; kk < kend; kk += 2 * VN) {
+                        // chunks past the last one are read from a clamped (valid) place and never used
+                        RT_CHUNK(xa, wa, xb, wb, rb, ra, min(kk + VN, KC - VN), min(kk + 2 * VN, KC - VN));
+                        if (kk + VN < kend) RT_CHUNK(xb, wb, xa, wa, ra, rb, min(kk + 2 * VN, KC - VN), min(kk + 3 * VN, KC - VN));
                     }
                 }
             }
+            __syncthreads();
         }
-        for (; kk < kmax; kk += VN) {
-            float xv[VN];
-            VecLoad<XT>::load(&xs[lane][kk], xv);
-#pragma unroll
-            for (int q = 0; q < VN; q += 4) {
-#pragma unroll
-                for (int j = 0; j < EE; ++j) {
-                    const float4 wq = *reinterpret_cast<const float4*>(&wsT[e0 + j][kk + q]);
-                    acc[j] = fmaf(xv[q + 0], wq.x, acc[j]);
-                    acc[j] = fmaf(xv[q + 1], wq.y, acc[j]);
-                    acc[j] = fmaf(xv[q + 2], wq.z, acc[j]);
-                    acc[j] = fmaf(xv[q + 3], wq.w, acc[j]);
-                }
-            }
-        }
-        __syncthreads();
     }
-    const int t = t0 + lane;
-    if (t < T) {
+#undef RT_CHUNK
+#undef RT_CVT
+#undef RT_PIN
+#undef RT_MFMA
+#undef RT_STASH
+#undef RT_FETCH
+    const int e = eb0 + wave * SHAPE + lane % SHAPE;
+    if (e < E) {
+        const float bv = bias ? bias[e] : 0.f;
 #pragma unroll
-        for (int j = 0; j < EE; ++j) {
-            const int e = e0 + j;
-            if (e < E) logits[(size_t)t * E + e] = bias ? __fadd_rn(acc[j], bias[e]) : acc[j];
+        for (int v = 0; v < NACC; ++v) {
+            const int t = t0 + (SHAPE == 16 ? 16 * (v / 4) + 4 * (lane / 16) + v % 4 : 4 * (lane / 4) + v);
+            if (t < T) logits[(size_t)t * E + e] = bias ? __fadd_rn(acc[v], bv) : acc[v];
         }
     }
 }
@@ -347,25 +299,19 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict_
     }
 }
 
+template <typename XT, int SHAPE>
+void launch_logits_mfma(const XT* x, const XT* w, const float* bias, float* logits, int T, int H, int E, hipStream_t s) {
+    const int gx = ceil_div(T, RT_TB), groups = ceil_div(E, SHAPE);
+    if (groups == 1) route_logits_mfma_kernel<XT, SHAPE, 1><<<dim3(gx, 1), WAVE, 0, s>>>(x, w, bias, logits, T, H, E);
+    else if (groups == 2) route_logits_mfma_kernel<XT, SHAPE, 2><<<dim3(gx, 1), 2 * WAVE, 0, s>>>(x, w, bias, logits, T, H, E);
+    else route_logits_mfma_kernel<XT, SHAPE, 4><<<dim3(gx, ceil_div(groups, 4)), 4 * WAVE, 0, s>>>(x, w, bias, logits, T, H, E);
+}
+
 template <typename XT>
 int launch_logits(const XT* x, const XT* w, const float* bias, float* logits, int T, int H, int E, hipStream_t s) {
-    const int gx = ceil_div(T, RT_TB);
-    if (E <= 4) {
-        route_logits_small_kernel<XT, 1><<<gx, RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
-    } else if (E <= 8) {
-        route_logits_small_kernel<XT, 2><<<gx, RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
-    } else if (E <= 12) {
-        route_logits_small_kernel<XT, 3><<<gx, RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
-    } else if (E <= 16) {
-        route_logits_small_kernel<XT, 4><<<gx, RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
-    } else if (E <= 32) {
-        route_logits_kernel<XT, 2, 4, 8><<<dim3(gx, 1), RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
-    } else if (gx * ceil_div(E, 64) < 2 * 256) {
-        // too few 64 x 64 blocks to give every SIMD two waves: halve the expert tile instead
-        route_logits_kernel<XT, 2, 4, 8><<<dim3(gx, ceil_div(E, 32)), RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
-    } else {
-        route_logits_kernel<XT, 4, 4, 16><<<dim3(gx, ceil_div(E, 64)), RT_THREADS, 0, s>>>(x, w, bias, logits, T, H, E);
-    }
+    // 16 experts per instruction when that alone gives every SIMD of the chip a wave, else 4 (four times the waves)
+    if (E > 8 && ceil_div(T, RT_TB) * ceil_div(E, 16) >= 1024) launch_logits_mfma<XT, 16>(x, w, bias, logits, T, H, E, s);
+    else launch_logits_mfma<XT, 4>(x, w, bias, logits, T, H, E, s);
     return moe_check_launch("route_logits");
 }
 
