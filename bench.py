@@ -141,7 +141,9 @@ def main():
     else:
         ms_graph, stream_ms_per_step = None, ms_per_step
 
-    stage_ms = {n: sum(e[n][0].elapsed_time(e[n][1]) for e in events) / len(events) for n in STAGES}
+    per_stage = {n: sorted(e[n][0].elapsed_time(e[n][1]) for e in events) for n in STAGES}
+    stage_ms = {n: sum(v) / len(v) for n, v in per_stage.items()}
+    stage_spread = {n: (v[0], v[len(v) // 2]) for n, v in per_stage.items()}  # (min, median) over the timed steps
     work = pipe.work()
     stages = {}
     for n, wk in work.items():
@@ -158,8 +160,8 @@ def main():
             ach = wk["amount"] / (ms * 1e-3) / 1e12
             peak = PEAK["mfma_fp8"] if cfg.quant == "fp8" else (PEAK["fp32"] if cfg.dtype == "f32" else PEAK["mfma_bf16"])
             unit = "TFLOP/s"
-        stages[n] = {"ms": round(ms, 4), "bound": wk["bound"], "achieved": round(ach, 2), "peak": peak, "unit": unit,
-                     "frac": round(ach / peak, 4)}
+        stages[n] = {"ms": round(ms, 4), "ms_min": round(stage_spread[n][0], 4), "ms_median": round(stage_spread[n][1], 4),
+                     "bound": wk["bound"], "achieved": round(ach, 2), "peak": peak, "unit": unit, "frac": round(ach / peak, 4)}
     # HBM traffic per launch of the dominant kernel, from the FETCH_SIZE / WRITE_SIZE runs summarised in
     # profiles/mixtral_hbm_traffic.txt (bytes; only measured for the default workload)
     measured_traffic = {"mixtral": 12.52e9}

@@ -92,6 +92,33 @@ def test_route_ties_prefer_lower_expert():
     assert (cls == cls[:, :1]).all() and (np.diff(o_idx, axis=1) == 4).all()
 
 
+@pytest.mark.parametrize("kind", ["wide", "subnormal", "cancel"])
+@pytest.mark.parametrize("E", [8, 20, 200])
+def test_route_logits_rounding_matches_fmaf_chain(kind, E):
+    """The logits run on K = 1 fp32 matrix instructions; every step must round exactly like fmaf (one rounding,
+    subnormals kept): operands spread over 40 binades, products in the subnormal range, and sums that cancel
+    would each expose a multiply-then-add, a flush to zero or another summation order."""
+    T, H, k = 130, 200, 3
+    g = torch.Generator().manual_seed(E * 7 + len(kind))
+    x = torch.randn(T, H, generator=g)
+    w = torch.randn(H, E, generator=g)
+    if kind == "wide":
+        x = x * torch.pow(2.0, torch.randint(-20, 21, (T, H), generator=g).float())
+        w = w * torch.pow(2.0, torch.randint(-20, 21, (H, E), generator=g).float())
+    elif kind == "subnormal":
+        x = x * 2.0 ** -70
+        w = w * 2.0 ** -62
+    else:
+        x[:, 1::2] = -x[:, 0::2]  # consecutive terms nearly cancel
+        w[1::2] = w[0::2] * (1 + 2.0 ** -12)
+    idx, gate, logits = ops.route_topk(x.to(DEV), w.to(DEV).contiguous(), k)
+    o_idx, _, o_logits = O.route(x.numpy(), w.numpy(), k)
+    if kind == "subnormal":
+        assert np.abs(o_logits).max() < 2.0 ** -126 and np.count_nonzero(o_logits) > o_logits.size // 2
+    assert_bits_equal(logits, o_logits, f"logits ({kind})")
+    assert_bits_equal(idx, o_idx, f"top-k ({kind})")
+
+
 @pytest.mark.parametrize("E,k,W", [(8, 8, 4), (512, 16, 64), (6, 1, 3), (60, 7, 1)])
 def test_route_edge_shapes(E, k, W):
     T, H = 77, 72
