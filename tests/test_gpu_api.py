@@ -121,3 +121,16 @@ def test_expert_layer_signature():
     want = O.grouped_gemm(x, w, cnt, "f32")
     np.testing.assert_allclose(to_np(out), want, rtol=1e-2, atol=1e-3)  # the reference's intended rtol (unit_tests.py:237)
     np.testing.assert_allclose(to_np(out), want, rtol=1e-4, atol=1e-4)
+
+
+def test_benchmark_driver_point_and_overflow_report(capsys):
+    """The environment-variable driver (the reference's benchmark.py knobs): one point with a CAPACITY smaller
+    than the largest per-expert count prints the skip notice, still times, and its correctness report (fixed-M
+    route against the padding-free flat route into token_buf) passes."""
+    from iris_testing_amd import benchmark
+    res = benchmark.run_point({"WORLD_SIZE": 4, "BATCH": 1, "SEQ": 320, "HIDDEN": 256, "TOPK": 2, "E_LOCAL": 3,
+                               "CAPACITY": 8, "SEED": 7})
+    out = capsys.readouterr().out
+    assert "[SKIP] max_recv_count=" in out and "=== Correctness Report ===" in out and out.rstrip().endswith("PASS")
+    assert res["ok"] and res["world"] == 4 and res["e_local"] == 3 and res["cap"] > 8
+    assert res["source_ms"] > 0 and res["dest_ms"] > 0 and res["dest_direct_ms"] > 0
