@@ -191,14 +191,21 @@ int moe_grouped_mlp_fp8(const void* tokens_bf16, const int32_t* expert_cnt, int 
  *   moe_grouped_gemm_mapped moe_grouped_gemm_packed with row indirection: logical row r is read from row
  *                           a_row_map[r] of a_base (a_rows rows of K, under 4 GiB) and written to row
  *                           c_row_map[r] of out (out_rows rows of N); either map may be NULL (identity).
- *                           Map entries must lie inside their buffers.
+ *                           Map entries must lie inside their buffers.  part_ws (nullable, part_ws_bytes
+ *                           bytes, moe_gemm_part_workspace_bytes() for the full benefit): scratch for fp32
+ *                           partial sums; with it, when the last round of the persistent grid holds at most
+ *                           a quarter of a grid of tiles, those tiles are cut along K over the idle compute
+ *                           units and summed in a fixed order by a second kernel (same result for the same
+ *                           shapes and counts on every call; last-bit differences against the unsplit sum).
  *   moe_zero_padding_rows   rows [sum_e recv_counts[s,e], M) of every slot s of buf [W,M,H] <- 0: what
  *                           moe_return_pack writes besides the result rows. */
 int moe_recv_row_map(const int32_t* recv_counts, int W, int E_l, int M, int n_rows, int32_t* row_map,
                      int32_t* expert_cnt, int32_t* map_ws, moe_stream_t stream);
 int moe_grouped_gemm_mapped(const void* a_base, int a_rows, const int32_t* a_row_map, const void* packed,
                             const int32_t* expert_cnt, int S_rows, int K, int N, int E_l, int act, void* out,
-                            int out_rows, const int32_t* c_row_map, moe_stream_t stream);
+                            int out_rows, const int32_t* c_row_map, void* part_ws, size_t part_ws_bytes,
+                            moe_stream_t stream);
+size_t moe_gemm_part_workspace_bytes(void);
 int moe_zero_padding_rows(void* buf, int dtype, int W, int M, int H, const int32_t* recv_counts, int E_l,
                           moe_stream_t stream);
 /* moe_grouped_mlp_fp8 with the same row indirection: the row quantisation reads input row r from row

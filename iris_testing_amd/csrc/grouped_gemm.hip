@@ -16,6 +16,7 @@
 //   * the tile walk is XCD-aware: the 32 workgroups that share an L2 take a compact 4 x 8 patch of
 //     a 16 x 16 super-tile.
 #include "common.h"
+#include <algorithm>
 #include <type_traits>
 
 namespace moe_gg {
@@ -46,7 +47,38 @@ struct GemmParams {
     const int32_t* a_map;     // optional: logical row -> row of A (gather while loading), else A is row r itself
     const int32_t* c_map;     // optional: logical row -> row of C (scatter while storing)
     int E_l, K, N, Npad, ldc, S_rows, ncs;
+    // Optional split of the last, partly filled round of the persistent grid along K: when that round holds at
+    // most a quarter of a grid of tiles, each of them is cut into P parts of the K range, one per otherwise idle
+    // workgroup, which store their fp32 partial sums here (max_units part tiles of BM x 256 floats); a second
+    // kernel adds the parts of a tile in part order and applies the epilogue.  NULL: no split.
+    float* part_ws;
+    int max_units;
 };
+
+constexpr int GG_MAX_PARTS = 16;   // parts per tile at most
+constexpr int GG_MIN_PART_STAGES = 8;  // K stages per part at least (64 bytes of K each)
+
+// stages per part when nk stages (even) are cut into P parts: even, and P of them cover nk
+__host__ __device__ inline int gg_part_stages(int nk, int P) { return ((nk + P - 1) / P + 1) & ~1; }
+
+// How the tiles of a launch are walked: tiles [0, full) whole, tiles [full, total) in P parts each.
+struct GgPlan {
+    int total, full, P, nkp, units;
+};
+__host__ __device__ inline GgPlan gg_plan(int total, int grid, int nk, bool split, int max_units) {
+    GgPlan pl;
+    pl.total = total; pl.full = total; pl.P = 1; pl.nkp = nk;
+    const int tail = total % grid;
+    if (split && tail > 0 && 4 * tail <= grid) {
+        int P = grid / tail;
+        if (P > GG_MAX_PARTS) P = GG_MAX_PARTS;
+        if (P > max_units / tail) P = max_units / tail;
+        while (P > 1 && (gg_part_stages(nk, P) < GG_MIN_PART_STAGES || (P - 1) * gg_part_stages(nk, P) >= nk)) --P;
+        if (P > 1) { pl.P = P; pl.full = total - tail; pl.nkp = gg_part_stages(nk, P); }
+    }
+    pl.units = pl.full + (total - pl.full) * pl.P;
+    return pl;
+}
 
 // x * sigmoid(x) with the hardware reciprocal (1 ulp) instead of an IEEE division: the SwiGLU epilogue of a
 // 128 x 128 wave tile evaluates this 8192 times per lane-row, and the division was most of its cost
@@ -91,6 +123,8 @@ enum { EPI_NONE = 0, EPI_GELU = 1, EPI_SILU = 2, EPI_SWIGLU = 3 };
 // One output tile of the walk: group g, n tile nt, first row row0, rv valid rows (rv <= 0: none).
 struct GgTile {
     int g, nt, row0, rv;
+    int ks0, nks;   // first K stage and number of K stages this workgroup multiplies (the whole K range, or a part)
+    int unit;       // part tile index in the partial-sum workspace, or -1 for a whole tile
 };
 
 // lin -> tile: group-major, 16-row bands, 16-column super-columns (see the XCD-aware walk above)
@@ -114,17 +148,27 @@ __device__ __forceinline__ GgTile gg_decode(const int* g_tile_start, const int* 
 }
 
 // next non-empty tile of this workgroup at or after round `base` (base is advanced past it)
-template <int BM>
+// SPLIT = false walks the whole tiles [0, full); SPLIT = true walks the parts of the tiles [full, total): unit q
+// is part q % P of tile full + q / P.
+template <int BM, bool SPLIT>
 __device__ __forceinline__ GgTile gg_next_tile(const int* g_tile_start, const int* g_row_start, int E_l, int Nt, int S_rows,
-                                               int total, int my, int stride, int& base) {
+                                               const GgPlan& pl, int nk, int my, int stride, int& base) {
     GgTile t;
     t.g = t.nt = t.row0 = 0;
     t.rv = 0;
-    while (base < total) {
+    t.ks0 = 0; t.nks = nk; t.unit = -1;
+    const int n = SPLIT ? pl.units - pl.full : pl.full;
+    while (base < n) {
         const int lin = base + my;
         base += stride;
-        if (lin < total) {
-            t = gg_decode<BM>(g_tile_start, g_row_start, E_l, Nt, S_rows, lin);
+        if (lin < n) {
+            t = gg_decode<BM>(g_tile_start, g_row_start, E_l, Nt, S_rows, SPLIT ? pl.full + lin / pl.P : lin);
+            t.ks0 = 0; t.nks = nk; t.unit = -1;
+            if constexpr (SPLIT) {
+                t.ks0 = (lin % pl.P) * pl.nkp;
+                t.nks = min(pl.nkp, nk - t.ks0);
+                t.unit = lin;
+            }
             if (t.rv > 0) break;
         }
     }
@@ -163,7 +207,7 @@ __device__ __forceinline__ void gg_wait() {
 // wave holds the last fragments of stage s in registers, and are spread over the two MFMA blocks that
 // follow, so the load pipe sees a steady stream instead of a burst and every load has two full stages
 // of MFMA work to land.
-template <int BM, int NWM, int EPI, bool FP8>
+template <int BM, int NWM, int EPI, bool FP8, bool SPLIT>
 __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const GemmParams p) {
     constexpr int BN = GG_BN;
     constexpr int ES = FP8 ? 1 : 2;
@@ -215,8 +259,9 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         g_row_start[p.E_l] = rs;
     }
     __syncthreads();
-    const int total = g_tile_start[p.E_l];
     const int nk = (p.K * ES) / ROWB;  // ring stages per tile; even (K * ES is a multiple of 2 * ROWB)
+    const GgPlan plan = gg_plan(g_tile_start[p.E_l], (int)gridDim.x, nk, p.part_ws != nullptr, p.max_units);
+    if (SPLIT && plan.P == 1) return;  // nothing was left over for this launch
 
     // XCD-aware position inside a round of gridDim.x tiles: workgroups b, b+8, b+16, ... share an L2.
     int my = blockIdx.x;
@@ -247,8 +292,8 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     for (int r = 0; r < RB; ++r) b_off[r] = (uint32_t)(r * LR + lrow) * ROWB + lchunk * 16;
 
 #define GG_TILE_PTRS(t, Ab_, Bb_, aoff_)                                                                   \
-    const uint8_t* Ab_ = p.a_map ? p.A : p.A + (size_t)(t).row0 * p.K * ES;                                 \
-    const uint8_t* Bb_ = p.B + (size_t)(t).g * p.Npad * p.K * ES + (size_t)(t).nt * BN * ROWB;               \
+    const uint8_t* Ab_ = (p.a_map ? p.A : p.A + (size_t)(t).row0 * p.K * ES) + (size_t)(t).ks0 * ROWB;      \
+    const uint8_t* Bb_ = p.B + (size_t)(t).g * p.Npad * p.K * ES + (size_t)(t).nt * BN * ROWB + (size_t)(t).ks0 * b_slab; \
     uint32_t aoff_[RA];                                                                                     \
     _Pragma("unroll") for (int r = 0; r < RA; ++r) {                                                         \
         const int lr_ = max(min(r * LR + lrow, (t).rv - 1), 0);  /* tile row this lane fetches, clamped */     \
@@ -262,13 +307,13 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     } while (0)
     // loads [first, first + count) of stage `st` (clamped to the last stage: the ring never holds data
     // of another tile, and a repeated load of the last stage lands in a slot nobody reads again)
-#define GG_STAGE_PTRS(Ab_, Bb_, st, ap_, bp_)                                                  \
-    const int st_ = min((st), nk - 1);                                                         \
+#define GG_STAGE_PTRS(Ab_, Bb_, st, ap_, bp_, nks_)                                            \
+    const int st_ = min((st), (nks_) - 1);                                                     \
     const uint8_t* ap_ = gg_uniform(Ab_ + (size_t)st_ * ROWB);                                 \
     const uint8_t* bp_ = gg_uniform(Bb_ + (size_t)st_ * b_slab);
-#define GG_ISSUE_RANGE(Ab_, Bb_, aoff_, st, slot, first, count)                                \
+#define GG_ISSUE_RANGE(Ab_, Bb_, aoff_, st, slot, first, count, nks_)                          \
     do {                                                                                       \
-        GG_STAGE_PTRS(Ab_, Bb_, st, ap_i, bp_i)                                                \
+        GG_STAGE_PTRS(Ab_, Bb_, st, ap_i, bp_i, nks_)                                          \
         if constexpr ((first) + 0 < (first) + (count)) GG_LD((first) + 0 < LPS ? (first) + 0 : 0, ap_i, bp_i, aoff_, slot); \
         if constexpr ((first) + 1 < (first) + (count)) GG_LD((first) + 1 < LPS ? (first) + 1 : 0, ap_i, bp_i, aoff_, slot); \
         if constexpr ((first) + 2 < (first) + (count)) GG_LD((first) + 2 < LPS ? (first) + 2 : 0, ap_i, bp_i, aoff_, slot); \
@@ -280,16 +325,16 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         static_assert((count) <= 8, "GG_ISSUE_RANGE is unrolled for eight loads");             \
     } while (0)
     // what a tile has in flight before its first MFMA: its first four stages, one per ring slot
-#define GG_PROLOGUE(Ab_, Bb_, aoff_)                          \
+#define GG_PROLOGUE(Ab_, Bb_, aoff_, nks_)                    \
     do {                                                      \
-        GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 0, 0, 0, LPS);        \
-        GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 1, 1, 0, LPS);        \
-        GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 2, 2, 0, LPS);        \
-        GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 3, 3, 0, LPS);        \
+        GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 0, 0, 0, LPS, nks_);  \
+        GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 1, 1, 0, LPS, nks_);  \
+        GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 2, 2, 0, LPS, nks_);  \
+        GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 3, 3, 0, LPS, nks_);  \
     } while (0)
 
     int base = 0;
-    GgTile cur = gg_next_tile<BM>(g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, total, my, gridDim.x, base);
+    GgTile cur = gg_next_tile<BM, SPLIT>(g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, plan, nk, my, gridDim.x, base);
     uint32_t a_off[RA];
     const uint8_t *Ab = p.A, *Bb = p.B;
     if (cur.rv > 0) {
@@ -298,11 +343,13 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         Bb = Bb0;
 #pragma unroll
         for (int r = 0; r < RA; ++r) a_off[r] = a_off0[r];
-        GG_PROLOGUE(Ab, Bb, a_off);
+        GG_PROLOGUE(Ab, Bb, a_off, (SPLIT ? cur.nks : nk));
     }
     while (cur.rv > 0) {
         const int g = __builtin_amdgcn_readfirstlane(cur.g), nt = __builtin_amdgcn_readfirstlane(cur.nt);
         const int row0 = __builtin_amdgcn_readfirstlane(cur.row0), rv = __builtin_amdgcn_readfirstlane(cur.rv);
+        const int nks = SPLIT ? __builtin_amdgcn_readfirstlane(cur.nks) : nk;
+        const int unit = SPLIT ? __builtin_amdgcn_readfirstlane(cur.unit) : -1;
 
         typedef typename std::conditional<FP8, floatx16, floatx4>::type acc_t;
         acc_t acc[TM][TN];
@@ -351,7 +398,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     GG_ML((I) + 6, FA_, FB_, NA_, NB_, slot); GG_ML((I) + 7, FA_, FB_, NA_, NB_, slot)
 #define GG_STAGE(FA_, FB_, NA_, NB_, SL, s, last)                                                        \
     do {                                                                                                 \
-        GG_STAGE_PTRS(Ab, Bb, (s) + 4, ap_, bp_)                                                         \
+        GG_STAGE_PTRS(Ab, Bb, (s) + 4, ap_, bp_, nks)                                                    \
         const uint4* nfa_ = fa + (((SL) + 1) & 3) * ASLOT;                                               \
         const uint4* nfb_ = fb + (((SL) + 1) & 3) * BSLOT;                                               \
         __builtin_amdgcn_sched_barrier(0);                                                               \
@@ -387,13 +434,13 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             int ks = 0;
             do {
                 GG_STAGE(fA0, fB0, fA1, fB1, 0, ks, false);
-                GG_STAGE(fA1, fB1, fA0, fB0, 1, ks + 1, ks + 2 >= nk);
-                if (ks + 2 < nk) {
+                GG_STAGE(fA1, fB1, fA0, fB0, 1, ks + 1, ks + 2 >= nks);
+                if (ks + 2 < nks) {
                     GG_STAGE(fA0, fB0, fA1, fB1, 2, ks + 2, false);
-                    GG_STAGE(fA1, fB1, fA0, fB0, 3, ks + 3, ks + 4 >= nk);
+                    GG_STAGE(fA1, fB1, fA0, fB0, 3, ks + 3, ks + 4 >= nks);
                 }
                 ks += 4;
-            } while (ks < nk);
+            } while (ks < nks);
         }
 #undef GG_STAGE
 #undef GG_ML8
@@ -402,11 +449,40 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 
         // ---- next tile: decode it and request its first stages now (every slot is free once all waves
         // have passed the barrier: the last fragments of this tile are already in registers)
-        const GgTile nxt = gg_next_tile<BM>(g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, total, my, gridDim.x, base);
+        const GgTile nxt = gg_next_tile<BM, SPLIT>(g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, plan, nk, my, gridDim.x, base);
         GG_TILE_PTRS(nxt, Ab_n, Bb_n, a_off_n);
         if (nxt.rv > 0) {
             __syncthreads();
-            GG_PROLOGUE(Ab_n, Bb_n, a_off_n);
+            GG_PROLOGUE(Ab_n, Bb_n, a_off_n, (SPLIT ? nxt.nks : nk));
+        }
+
+        // ---- a part of a tile: its fp32 partial sums go to the workspace as they are (tile row major, 256
+        // columns; the lane's runs of four columns as 16-byte stores); the reduction kernel does the rest
+        if constexpr (SPLIT) {  // (every tile of this instantiation is a part; the epilogue below is the other one's)
+            float* wsT = p.part_ws + (size_t)unit * (BM * BN);
+            constexpr int NQp = FP8 ? 4 : 1;
+            const int clp = FP8 ? (lane >> 5) * 4 : (lane >> 4) * 4;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int r = wm * (BM / NWM) + i * MT + (lane & (MT - 1));
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+#pragma unroll
+                    for (int q = 0; q < NQp; ++q) {
+                        const int c = wn * (BN / 2) + j * MT + 8 * q + clp;
+                        const float4 v = make_float4(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                                                     acc[i][j][4 * q + 3]);
+                        if (r < rv) *(float4*)(wsT + (size_t)r * BN + c) = v;
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            cur = nxt;
+            Ab = Ab_n;
+            Bb = Bb_n;
+#pragma unroll
+            for (int r = 0; r < RA; ++r) a_off[r] = a_off_n[r];
+            continue;
         }
 
         // ---- epilogue: acc -> (scales) -> activation -> bf16 -> C
@@ -511,6 +587,94 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 #undef GG_STAGE_PTRS
 #undef GG_ISSUE_RANGE
 #undef GG_PROLOGUE
+}
+
+// ---- second half of a K-split tile: add its parts in part order, then the epilogue of the GEMM kernel ------------
+// Same tile tables and the same plan as the GEMM launch it follows (gemm_grid = that launch's grid).  A block takes
+// BM / 8 rows of one split tile; a thread takes four consecutive output columns of a row (for SwiGLU the gate
+// columns and, 32 packed columns further, their up columns).
+template <int BM, int EPI, bool FP8>
+__global__ __launch_bounds__(256) void gg_reduce_parts_kernel(const GemmParams p, int gemm_grid) {
+    constexpr int BN = GG_BN;
+    constexpr int ES = FP8 ? 1 : 2;
+    constexpr int RSL = 8;  // row slabs (blocks) per tile
+    __shared__ int g_tile_start[GG_MAXG + 1];
+    __shared__ int g_row_start[GG_MAXG + 1];
+    const int Nt = p.Npad / BN;
+    if (threadIdx.x == 0) {
+        int ts = 0, rs = 0;
+        for (int g = 0; g < p.E_l; ++g) {
+            g_tile_start[g] = ts;
+            g_row_start[g] = rs;
+            const int c = max(p.cnt[g], 0);
+            ts += ((c + BM - 1) / BM) * Nt;
+            rs += c;
+        }
+        g_tile_start[p.E_l] = ts;
+        g_row_start[p.E_l] = rs;
+    }
+    __syncthreads();
+    const int nk = (p.K * ES) / ROWB;
+    const GgPlan plan = gg_plan(g_tile_start[p.E_l], gemm_grid, nk, true, p.max_units);
+    if (plan.P == 1) return;
+    const int ti = blockIdx.x / RSL, slab = blockIdx.x % RSL;
+    if (ti >= plan.total - plan.full) return;
+    const GgTile t = gg_decode<BM>(g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, plan.full + ti);
+    if (t.rv <= 0) return;
+    const float* ws = p.part_ws + (size_t)ti * plan.P * (BM * BN);
+    constexpr int OC4 = (EPI == EPI_SWIGLU ? BN / 2 : BN) / 4;  // groups of four output columns per tile row
+    constexpr int RPP = 256 / OC4;                               // rows per pass of the block
+    const int oc = (threadIdx.x % OC4) * 4;                      // first output column of the thread inside the tile
+    const int pc = EPI == EPI_SWIGLU ? (oc / 32) * 64 + oc % 32 : oc;  // its packed column inside the tile
+    const int gp = t.nt * BN + pc;                               // packed column of the launch
+    const int col = EPI == EPI_SWIGLU ? (gp / 64) * 32 + gp % 32 : gp;  // output column
+    float4 sc0 = make_float4(1.f, 1.f, 1.f, 1.f), sc1 = sc0;
+    if (FP8 && col < p.N) {
+        sc0 = *(const float4*)(p.col_scale + (size_t)t.g * p.ncs + col);
+        if constexpr (EPI == EPI_SWIGLU) sc1 = *(const float4*)(p.col_scale2 + (size_t)t.g * p.ncs + col);
+    }
+    bf16_t* C = (bf16_t*)p.C;
+    const int r_end = min((slab + 1) * (BM / RSL), t.rv);
+    for (int r = slab * (BM / RSL) + threadIdx.x / OC4; r < r_end; r += RPP) {
+        const float* w = ws + (size_t)r * BN + pc;
+        float4 a = *(const float4*)w, b = make_float4(0.f, 0.f, 0.f, 0.f);
+        if constexpr (EPI == EPI_SWIGLU) b = *(const float4*)(w + 32);
+        for (int part = 1; part < plan.P; ++part) {
+            const float* wp = w + (size_t)part * (BM * BN);
+            const float4 v = *(const float4*)wp;
+            a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w;
+            if constexpr (EPI == EPI_SWIGLU) {
+                const float4 u = *(const float4*)(wp + 32);
+                b.x += u.x; b.y += u.y; b.z += u.z; b.w += u.w;
+            }
+        }
+        const size_t grow = (size_t)(t.row0 + r);
+        float rs = 1.f;
+        if constexpr (FP8) rs = p.row_scale[grow];
+        float av[4] = {a.x, a.y, a.z, a.w}, bv[4] = {b.x, b.y, b.z, b.w};
+        const float c0[4] = {sc0.x, sc0.y, sc0.z, sc0.w}, c1[4] = {sc1.x, sc1.y, sc1.z, sc1.w};
+        float x[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if constexpr (EPI == EPI_SWIGLU) {
+                float gv = av[e], uv = bv[e];
+                if constexpr (FP8) { gv *= c0[e] * rs; uv *= c1[e] * rs; }
+                x[e] = act_silu_fast(gv) * uv;
+            } else {
+                float v = av[e];
+                if constexpr (FP8) v *= c0[e] * rs;
+                if constexpr (EPI == EPI_GELU) v = act_gelu(v);
+                if constexpr (EPI == EPI_SILU) v = act_silu_fast(v);
+                x[e] = v;
+            }
+        }
+        if (col < p.N) {
+            uint2 o;
+            o.x = gg_pack_bf16(x[0], x[1]);
+            o.y = gg_pack_bf16(x[2], x[3]);
+            *(uint2*)(C + (p.c_map ? (size_t)p.c_map[grow] : grow) * p.ldc + col) = o;
+        }
+    }
 }
 
 // ---- one-time weight re-tiling: w [E_l,K,N] (N contiguous) -> out [E_l][K/SK][Npad][SK], SK = one LDS
@@ -725,15 +889,32 @@ int num_cus() {
 int round_up(int a, int b) { return (a + b - 1) / b * b; }
 
 template <bool FP8>
-int launch_gemm(const GemmParams& p, int epi, hipStream_t s) {
+int launch_gemm(const GemmParams& p_in, int epi, hipStream_t s, void* part_ws = nullptr, size_t part_ws_bytes = 0) {
     const int grid = num_cus();
+    GemmParams p = p_in;
     // 256-row or 128-row tiles: the host knows only the total row count, so it compares the estimated number
     // of rounds of the persistent grid (every group adds about half a tile of ragged tail); a 128-row tile
     // costs about 0.62 of a 256-row one
     const int nt = p.Npad / GG_BN;
     const double t256 = ((double)p.S_rows / 256 + 0.5 * p.E_l) * nt, t128 = ((double)p.S_rows / 128 + 0.5 * p.E_l) * nt;
     const bool small_m = 0.62 * ceil(t128 / grid) < ceil(t256 / grid);
-#define GG_LAUNCH(BMv, NWMv, EPIv) grouped_gemm_kernel<BMv, NWMv, EPIv, FP8><<<grid, NWMv * 2 * WAVE, 0, s>>>(p)
+    // with a workspace, the tiles of a last round that fills at most a quarter of the grid are split along K
+    // (decided on the device from the row counts); the reduction kernel finds nothing to do otherwise
+    p.part_ws = nullptr;
+    p.max_units = 0;
+    if (part_ws) {
+        p.max_units = (int)std::min<size_t>(part_ws_bytes / ((size_t)(small_m ? 128 : 256) * GG_BN * sizeof(float)), (size_t)grid);
+        if (p.max_units >= 2) p.part_ws = (float*)part_ws;
+    }
+    const int red_blocks = (grid / 4) * 8;
+#define GG_LAUNCH(BMv, NWMv, EPIv)                                                                        \
+    do {                                                                                                  \
+        grouped_gemm_kernel<BMv, NWMv, EPIv, FP8, false><<<grid, NWMv * 2 * WAVE, 0, s>>>(p);              \
+        if (p.part_ws && red_blocks > 0) {                                                                \
+            grouped_gemm_kernel<BMv, NWMv, EPIv, FP8, true><<<grid, NWMv * 2 * WAVE, 0, s>>>(p);           \
+            gg_reduce_parts_kernel<BMv, EPIv, FP8><<<red_blocks, 256, 0, s>>>(p, grid);                    \
+        }                                                                                                 \
+    } while (0)
 #define GG_EPI(EPIv)                          \
     do {                                      \
         if (small_m) GG_LAUNCH(128, 2, EPIv); \
@@ -832,9 +1013,12 @@ extern "C" int moe_grouped_gemm_packed(const void* tokens, const void* packed, c
     return launch_gemm<false>(p, act, (hipStream_t)stream);
 }
 
+extern "C" size_t moe_gemm_part_workspace_bytes(void) { return (size_t)num_cus() * 256 * GG_BN * sizeof(float); }
+
 extern "C" int moe_grouped_gemm_mapped(const void* a_base, int a_rows, const int32_t* a_row_map, const void* packed,
                                        const int32_t* expert_cnt, int S_rows, int K, int N, int E_l, int act, void* out,
-                                       int out_rows, const int32_t* c_row_map, moe_stream_t stream) {
+                                       int out_rows, const int32_t* c_row_map, void* part_ws, size_t part_ws_bytes,
+                                       moe_stream_t stream) {
     MOE_REQUIRE(S_rows >= 0 && K > 0 && N > 0 && E_l > 0 && E_l <= GG_MAXG, MOE_ERR_INVALID, "grouped_gemm_mapped: bad shape");
     MOE_REQUIRE(act >= EPI_NONE && act <= EPI_SWIGLU, MOE_ERR_INVALID, "grouped_gemm_mapped: activation %d", act);
     MOE_REQUIRE(K % 64 == 0 && N % 8 == 0, MOE_ERR_UNSUPPORTED, "grouped_gemm_mapped: needs K %% 64 == 0 and N %% 8 == 0 (K=%d N=%d)", K, N);
@@ -849,7 +1033,7 @@ extern "C" int moe_grouped_gemm_mapped(const void* a_base, int a_rows, const int
     p.a_map = a_row_map; p.c_map = c_row_map;
     p.E_l = E_l; p.K = K; p.N = N; p.ldc = N; p.S_rows = S_rows;
     p.Npad = round_up(act == EPI_SWIGLU ? 2 * N : N, GG_BN);
-    return launch_gemm<false>(p, act, (hipStream_t)stream);
+    return launch_gemm<false>(p, act, (hipStream_t)stream, part_ws, part_ws_bytes);
 }
 
 extern "C" int moe_grouped_mlp(const void* tokens, const int32_t* expert_cnt, int dtype, int S_rows, int H, int F, int E_l,

@@ -363,9 +363,10 @@ def recv_row_map(recv_counts: torch.Tensor, M: int, n_rows: int, row_map: Option
 
 def grouped_gemm_mapped(a_base: torch.Tensor, a_row_map: Optional[torch.Tensor], packed: torch.Tensor,
                         expert_cnt: torch.Tensor, S_rows: int, N: int, act: str, out: torch.Tensor,
-                        c_row_map: Optional[torch.Tensor] = None) -> torch.Tensor:
+                        c_row_map: Optional[torch.Tensor] = None, part_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
     """grouped_gemm_packed with row indirection on the way in (a_base rows a_row_map[r]) and / or on the
-    way out (out rows c_row_map[r]).  a_base and out are 2-D views [rows, K] / [rows, N]."""
+    way out (out rows c_row_map[r]).  a_base and out are 2-D views [rows, K] / [rows, N].  part_ws: optional
+    scratch (gemm_part_workspace) that lets an under-filled last round of tiles be split along K."""
     _req_cuda(a_base, "a_base")
     _req_i32(expert_cnt, "expert_cnt")
     assert a_base.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and a_base.dim() == 2 and out.dim() == 2
@@ -377,8 +378,16 @@ def grouped_gemm_mapped(a_base: torch.Tensor, a_row_map: Optional[torch.Tensor],
     L.check(L.lib().moe_grouped_gemm_mapped(L.ptr(a_base), a_base.shape[0], L.ptr(a_row_map) if a_row_map is not None else None,
                                             L.ptr(packed), L.ptr(expert_cnt), S_rows, a_base.shape[1], N, expert_cnt.numel(),
                                             L.ACT[act], L.ptr(out), out.shape[0],
-                                            L.ptr(c_row_map) if c_row_map is not None else None, L.stream_ptr()))
+                                            L.ptr(c_row_map) if c_row_map is not None else None,
+                                            L.ptr(part_ws) if part_ws is not None else None,
+                                            part_ws.numel() * part_ws.element_size() if part_ws is not None else 0,
+                                            L.stream_ptr()))
     return out
+
+
+def gemm_part_workspace(device) -> torch.Tensor:
+    """fp32 scratch for the K-split of grouped_gemm_mapped, sized for any launch."""
+    return torch.empty(L.lib().moe_gemm_part_workspace_bytes() // 4, dtype=torch.float32, device=device)
 
 
 def zero_padding_rows(buf: torch.Tensor, recv_counts: torch.Tensor) -> torch.Tensor:

@@ -62,6 +62,9 @@ class DispatchPipeline:
         self.ret = torch.empty((W, M, H), dtype=dt, device=dev)
         self.ret_map = i32(lib.moe_recv_map_ints(W, E_l, W * M))
         self.row_map = i32(max(S, 1))
+        # scratch for the K-split of an under-filled last round of GEMM tiles (bf16 experts)
+        self.part_ws_bytes = lib.moe_gemm_part_workspace_bytes() if weights.dtype == torch.bfloat16 else 0
+        self.part_ws = torch.empty(self.part_ws_bytes // 4, dtype=torch.float32, device=dev) if self.part_ws_bytes else None
         if weights.dtype == torch.uint8:
             self.xq = torch.empty((S, H), dtype=torch.uint8, device=dev)
             self.xs = torch.empty((S,), dtype=torch.float32, device=dev)
@@ -128,10 +131,11 @@ class DispatchPipeline:
             w = self.world
             L.check(lib.moe_grouped_gemm_mapped(self._p(w.recv), c.world * w.M, self._p(self.row_map), self._p(ew.w1),
                                                 self._p(self.expert_cnt), self.S, c.hidden, c.ffn, c.e_local, L.ACT[ew.act],
-                                                self._p(self.hidden), self.S, None, s))
+                                                self._p(self.hidden), self.S, None, self._p(self.part_ws), self.part_ws_bytes, s))
         else:
-            L.check(lib.moe_grouped_gemm_packed(self._p(self.rows), self._p(ew.w1), self._p(self.expert_cnt), self.S, c.hidden,
-                                                c.ffn, c.e_local, L.ACT[ew.act], self._p(self.hidden), s))
+            L.check(lib.moe_grouped_gemm_mapped(self._p(self.rows), self.S, None, self._p(ew.w1), self._p(self.expert_cnt),
+                                                self.S, c.hidden, c.ffn, c.e_local, L.ACT[ew.act], self._p(self.hidden),
+                                                self.S, None, self._p(self.part_ws), self.part_ws_bytes, s))
 
     def mlp_down(self, s):
         c, ew = self.cfg, self.weights
@@ -139,10 +143,11 @@ class DispatchPipeline:
             w = self.world
             L.check(L.lib().moe_grouped_gemm_mapped(self._p(self.hidden), self.S, None, self._p(ew.w2), self._p(self.expert_cnt),
                                                     self.S, c.ffn, c.hidden, c.e_local, 0, self._p(self.ret), c.world * w.M,
-                                                    self._p(self.row_map), s))
+                                                    self._p(self.row_map), self._p(self.part_ws), self.part_ws_bytes, s))
         elif ew.dtype == torch.bfloat16:
-            L.check(L.lib().moe_grouped_gemm_packed(self._p(self.hidden), self._p(ew.w2), self._p(self.expert_cnt), self.S,
-                                                    c.ffn, c.hidden, c.e_local, 0, self._p(self.y), s))
+            L.check(L.lib().moe_grouped_gemm_mapped(self._p(self.hidden), self.S, None, self._p(ew.w2), self._p(self.expert_cnt),
+                                                    self.S, c.ffn, c.hidden, c.e_local, 0, self._p(self.y), self.S, None,
+                                                    self._p(self.part_ws), self.part_ws_bytes, s))
 
     def return_pack(self, s):
         c, w = self.cfg, self.world

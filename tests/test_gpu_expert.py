@@ -150,11 +150,51 @@ def test_grouped_gemm_mapped(E_l, K, N, S, act):
     # argument checks happen before any launch
     lib = L.lib()
     rc = lib.moe_grouped_gemm_mapped(L.ptr(base_t), n_in, None, L.ptr(packed), L.ptr(cnt_t), S_tot, K + 8, N, E_l, 0,
-                                     L.ptr(out), n_out, None, L.stream_ptr())
+                                     L.ptr(out), n_out, None, None, 0, L.stream_ptr())
     assert rc != 0 and b"K" in lib.moe_last_error()
     rc = lib.moe_grouped_gemm_mapped(L.ptr(base_t), 1 << 30, L.ptr(torch.from_numpy(a_map).to(DEV)), L.ptr(packed),
-                                     L.ptr(cnt_t), S_tot, K, N, E_l, 0, L.ptr(out), n_out, None, L.stream_ptr())
+                                     L.ptr(cnt_t), S_tot, K, N, E_l, 0, L.ptr(out), n_out, None, None, 0, L.stream_ptr())
     assert rc != 0 and b"4 GiB" in lib.moe_last_error()
+
+
+@pytest.mark.parametrize("E_l,K,N,rows,act", [(2, 512, 1024, (200, 150), "none"), (2, 2048, 4096, (230, 213), "silu"),
+                                              (3, 1024, 512, (300, 0, 77), "swiglu"), (1, 4096, 2048, (443,), "gelu"),
+                                              (1, 1024, 4096, (20836,), "swiglu")])
+def test_grouped_gemm_k_split_of_the_last_round(E_l, K, N, rows, act):
+    """With a partial-sum workspace the tiles of an under-filled last round are cut along K and summed by a second
+    kernel.  The result must be the oracle's within the bf16 bar, within a bf16 rounding step of the unsplit kernel's
+    (only the fp32 summation order differs), identical from call to call, and rows outside the map stay untouched."""
+    rng = np.random.default_rng(K + N + len(rows))
+    cnt = np.array(rows, dtype=np.int32)
+    S_tot = int(cnt.sum())
+    x = _randn(rng, S_tot, K)
+    w = _randn(rng, E_l, K, N, scale=K ** -0.5)
+    wu = _randn(rng, E_l, K, N, scale=K ** -0.5) if act == "swiglu" else None
+    packed = ops.prepack_weights(_t(w, "bf16"), None if wu is None else _t(wu, "bf16"))
+    cnt_t, x_t = torch.from_numpy(cnt).to(DEV), _t(x, "bf16")
+    c_map = torch.from_numpy(rng.permutation(S_tot + 64)[:S_tot].astype(np.int32)).to(DEV)
+    ws = ops.gemm_part_workspace(DEV)
+    ws.fill_(float("nan"))  # stale contents must not matter
+    plain = torch.full((S_tot + 64, N), -7.0, dtype=torch.bfloat16, device=DEV)
+    ops.grouped_gemm_mapped(x_t, None, packed, cnt_t, S_tot, N, act, plain, c_map)
+    split = torch.full((S_tot + 64, N), -7.0, dtype=torch.bfloat16, device=DEV)
+    ops.grouped_gemm_mapped(x_t, None, packed, cnt_t, S_tot, N, act, split, c_map, part_ws=ws)
+    again = torch.full((S_tot + 64, N), -7.0, dtype=torch.bfloat16, device=DEV)
+    ws.fill_(3.0)
+    ops.grouped_gemm_mapped(x_t, None, packed, cnt_t, S_tot, N, act, again, c_map, part_ws=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(split.view(torch.int16), again.view(torch.int16)), "the K split is not reproducible"
+    a, b = split.float(), plain.float()
+    assert bool(torch.isfinite(a).all())
+    step = 2.0 ** -7 * torch.maximum(a.abs(), b.abs()) + 1e-6  # one bf16 rounding step either way
+    assert bool(((a - b).abs() <= 2 * step).all()), "split and unsplit sums differ by more than a rounding step"
+    untouched = np.setdiff1d(np.arange(S_tot + 64), to_np(c_map))
+    assert bool((split[torch.from_numpy(untouched).to(DEV)] == -7.0).all()), "rows outside the map were written"
+    got = to_np(split[c_map.long()])
+    if act == "none":
+        _check(got, O.grouped_gemm(x, w, cnt, "bf16"), BF16_RTOL, BF16_ATOL, "K-split GEMM")
+    differs = int((split.view(torch.int16) != plain.view(torch.int16)).sum().item())
+    print(f"K split: {differs} of {split.numel()} outputs differ in the last bits from the unsplit kernel", flush=True)
 
 
 @pytest.mark.parametrize("W,E_l,M,H,F,fill", [(4, 3, 300, 128, 256, "ragged"), (8, 5, 64, 256, 128, "empty"),
