@@ -725,15 +725,19 @@ __global__ void zero_pad_rows_kernel(T* __restrict__ out, int K, int Nreal, int 
 }
 
 // ---- fp32 path: plain tiled FMA kernel, weights in the reference layout ------------------------------
-// C[rows of g] = epi(A[rows of g] @ W[g] (, A @ Wup[g])); 64x64 tiles, 16x16 threads, 4x4 per thread.
+// C[rows of g] = epi(A[rows of g] @ W[g] (, A @ Wup[g])); 64x64 tiles, 16x16 threads, 4x4 per thread; K in slabs
+// of 64 through LDS, the next slab fetched into registers while the current one is multiplied (the workloads of
+// this path are small: what counts is that no memory latency is left exposed per slab).
 template <int EPI>
 __global__ __launch_bounds__(256) void grouped_gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ Wt,
                                                                 const float* __restrict__ Wup, float* __restrict__ C,
                                                                 const int32_t* __restrict__ cnt, int E_l, int K, int N,
                                                                 int S_rows) {
-    __shared__ float As[16][64 + 4];
-    __shared__ float Bs[16][64];
-    __shared__ float Us[EPI == EPI_SWIGLU ? 16 : 1][64];
+    constexpr int KC = 64;                       // K per slab
+    constexpr int PT = 64 * KC / 256;            // elements of each operand per thread and slab
+    __shared__ float As[KC][64 + 4];
+    __shared__ float Bs[KC][64];
+    __shared__ float Us[EPI == EPI_SWIGLU ? KC : 1][64];
     __shared__ int s_g, s_row0, s_rv;
     if (threadIdx.x == 0) {
         int mt = blockIdx.y, rs = 0, g = 0, found = 0;
@@ -754,20 +758,33 @@ __global__ __launch_bounds__(256) void grouped_gemm_f32_kernel(const float* __re
     const float* U = EPI == EPI_SWIGLU ? Wup + (size_t)g * K * N : nullptr;
     const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
     float acc[4][4] = {}, acu[4][4] = {};
-    for (int k0 = 0; k0 < K; k0 += 16) {
-        for (int i = threadIdx.x; i < 64 * 16; i += 256) {
-            const int r = i / 16, kk = i % 16;
-            As[kk][r] = (r < rv && k0 + kk < K) ? A[(size_t)(row0 + r) * K + k0 + kk] : 0.f;
+    float ra[PT], rb[PT], ru[EPI == EPI_SWIGLU ? PT : 1];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int q = 0; q < PT; ++q) {
+            const int i = threadIdx.x + q * 256;
+            const int r = i / KC, kk = i % KC;          // A: consecutive threads walk K
+            ra[q] = (r < rv && k0 + kk < K) ? A[(size_t)(row0 + r) * K + k0 + kk] : 0.f;
+            const int kb = i / 64, nn = i % 64;          // W: consecutive threads walk N
+            const bool ok = k0 + kb < K && n0 + nn < N;
+            rb[q] = ok ? W[(size_t)(k0 + kb) * N + n0 + nn] : 0.f;
+            if constexpr (EPI == EPI_SWIGLU) ru[q] = ok ? U[(size_t)(k0 + kb) * N + n0 + nn] : 0.f;
         }
-        for (int i = threadIdx.x; i < 16 * 64; i += 256) {
-            const int kk = i / 64, nn = i % 64;
-            const bool ok = k0 + kk < K && n0 + nn < N;
-            Bs[kk][nn] = ok ? W[(size_t)(k0 + kk) * N + n0 + nn] : 0.f;
-            if constexpr (EPI == EPI_SWIGLU) Us[kk][nn] = ok ? U[(size_t)(k0 + kk) * N + n0 + nn] : 0.f;
+    };
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += KC) {
+#pragma unroll
+        for (int q = 0; q < PT; ++q) {
+            const int i = threadIdx.x + q * 256;
+            As[i % KC][i / KC] = ra[q];
+            Bs[i / 64][i % 64] = rb[q];
+            if constexpr (EPI == EPI_SWIGLU) Us[i / 64][i % 64] = ru[q];
         }
         __syncthreads();
-#pragma unroll
-        for (int kk = 0; kk < 16; ++kk) {
+        if (k0 + KC < K) fetch(k0 + KC);
+        // slab positions past K hold zeros: adding +0 products leaves every sum as it is
+#pragma unroll 8
+        for (int kk = 0; kk < KC; ++kk) {
             float a[4], b[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
