@@ -84,3 +84,14 @@ def test_graph_replay_equals_eager(name, fused):
             assert torch.equal(getattr(pipe, n), eager[n]), f"replay {rep}: {n} differs from the eager step"
         pipe.step()  # eager work between replays
         torch.cuda.synchronize()
+
+
+def test_entry_point_smoke_runs():
+    """The smoke check of the repository's entry module (one small step against the oracle) must keep passing."""
+    import importlib
+    import os
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    if root not in sys.path:
+        sys.path.insert(0, root)
+    importlib.import_module("__graft_entry__").smoke()
