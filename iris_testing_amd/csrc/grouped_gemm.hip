@@ -56,6 +56,7 @@ struct GemmParams {
 };
 
 constexpr int GG_MAX_PARTS = 16;   // parts per tile at most
+constexpr int GG_RED_SLABS = 32;   // blocks per tile in the reduction of the parts
 constexpr int GG_MIN_PART_STAGES = 8;  // K stages per part at least (64 bytes of K each)
 
 // stages per part when nk stages (even) are cut into P parts: even, and P of them cover nk
@@ -591,13 +592,13 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 
 // ---- second half of a K-split tile: add its parts in part order, then the epilogue of the GEMM kernel ------------
 // Same tile tables and the same plan as the GEMM launch it follows (gemm_grid = that launch's grid).  A block takes
-// BM / 8 rows of one split tile; a thread takes four consecutive output columns of a row (for SwiGLU the gate
+// BM / GG_RED_SLABS rows of one split tile (many small blocks: the partial sums of a few tiles are tens of MB); a thread takes four consecutive output columns of a row (for SwiGLU the gate
 // columns and, 32 packed columns further, their up columns).
 template <int BM, int EPI, bool FP8>
 __global__ __launch_bounds__(256) void gg_reduce_parts_kernel(const GemmParams p, int gemm_grid) {
     constexpr int BN = GG_BN;
     constexpr int ES = FP8 ? 1 : 2;
-    constexpr int RSL = 8;  // row slabs (blocks) per tile
+    constexpr int RSL = GG_RED_SLABS;  // row slabs (blocks) per tile
     __shared__ int g_tile_start[GG_MAXG + 1];
     __shared__ int g_row_start[GG_MAXG + 1];
     const int Nt = p.Npad / BN;
@@ -923,7 +924,7 @@ int launch_gemm(const GemmParams& p_in, int epi, hipStream_t s, void* part_ws = 
         p.max_units = (int)std::min<size_t>(part_ws_bytes / ((size_t)(small_m ? 128 : 256) * GG_BN * sizeof(float)), (size_t)grid);
         if (p.max_units >= 2) p.part_ws = (float*)part_ws;
     }
-    const int red_blocks = (grid / 4) * 8;
+    const int red_blocks = (grid / 4) * GG_RED_SLABS;
 #define GG_LAUNCH(BMv, NWMv, EPIv)                                                                        \
     do {                                                                                                  \
         grouped_gemm_kernel<BMv, NWMv, EPIv, FP8, false><<<grid, NWMv * 2 * WAVE, 0, s>>>(p);              \
