@@ -63,12 +63,11 @@ __global__ __launch_bounds__(WAVE) void scan_blocks_kernel(const int32_t* __rest
 }
 
 // ---- 3. expert prefix -> all count/offset outputs (one wave) ---------------------------------------
-__global__ __launch_bounds__(WAVE) void offsets_kernel(const int32_t* __restrict__ counts, int E, int W,
-                                                        int32_t* __restrict__ expert_start /*[E+1]*/,
-                                                        int32_t* __restrict__ send_counts, int32_t* __restrict__ expert_offs,
-                                                        int32_t* __restrict__ dst_sizes, int32_t* __restrict__ dst_offsets,
-                                                        int32_t* __restrict__ caps) {
-    __shared__ int32_t es[MOE_MAX_EXPERTS + 1];
+// (every wave of the calling block runs this with the same inputs and writes the same values: es is shared)
+__device__ __forceinline__ void offsets_body(const int32_t* counts, int E, int W, int32_t* es /*[E+1], LDS*/,
+                                             int32_t* expert_start /*[E+1]*/, int32_t* __restrict__ send_counts,
+                                             int32_t* __restrict__ expert_offs, int32_t* __restrict__ dst_sizes,
+                                             int32_t* __restrict__ dst_offsets, int32_t* __restrict__ caps) {
     const int lane = lane_id();
     const int per = (E + WAVE - 1) / WAVE;
     const int lo = min(lane * per, E), hi = min(lo + per, E);
@@ -99,14 +98,21 @@ __global__ __launch_bounds__(WAVE) void offsets_kernel(const int32_t* __restrict
     if (lane == 0) { caps[0] = max(mmax, 1); caps[1] = max(cmax, 1); }
 }
 
+__global__ __launch_bounds__(WAVE) void offsets_kernel(const int32_t* __restrict__ counts, int E, int W,
+                                                        int32_t* __restrict__ expert_start /*[E+1]*/,
+                                                        int32_t* __restrict__ send_counts, int32_t* __restrict__ expert_offs,
+                                                        int32_t* __restrict__ dst_sizes, int32_t* __restrict__ dst_offsets,
+                                                        int32_t* __restrict__ caps) {
+    __shared__ int32_t es[MOE_MAX_EXPERTS + 1];
+    offsets_body(counts, E, W, es, expert_start, send_counts, expert_offs, dst_sizes, dst_offsets, caps);
+}
+
 // ---- 4. stable positions: one wave per 64-token block ----------------------------------------------
-__global__ __launch_bounds__(256) void rank_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ base,
-                                                    const int32_t* __restrict__ expert_start, int32_t* __restrict__ pos,
-                                                    int32_t* __restrict__ row_token, int T, int k, int E, int NB) {
-    const int wave = threadIdx.x / WAVE;
+// one wave ranks the slots of token block b
+__device__ __forceinline__ void rank_block(const int32_t* __restrict__ idx, const int32_t* base, const int32_t* expert_start,
+                                           int32_t* __restrict__ pos, int32_t* __restrict__ row_token, int T, int k, int E,
+                                           int NB, int b) {
     const int lane = lane_id();
-    const int b = blockIdx.x * 4 + wave;
-    if (b >= NB) return;
     const int t = b * CB + lane;
     const bool live = t < T;
     int mine[MOE_MAX_TOPK];
@@ -134,6 +140,52 @@ __global__ __launch_bounds__(256) void rank_kernel(const int32_t* __restrict__ i
             }
         }
     }
+}
+
+__global__ __launch_bounds__(256) void rank_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ base,
+                                                    const int32_t* __restrict__ expert_start, int32_t* __restrict__ pos,
+                                                    int32_t* __restrict__ row_token, int T, int k, int E, int NB) {
+    const int b = blockIdx.x * 4 + threadIdx.x / WAVE;
+    if (b >= NB) return;
+    rank_block(idx, base, expert_start, pos, row_token, T, k, E, NB, b);
+}
+
+// ---- the four steps above in one block, for few tokens (NB <= CS_MAXNB blocks of 64): launch latency is all that
+// such a count costs, so one launch instead of four.  Same arithmetic, tables in LDS instead of the workspace.
+constexpr int CS_MAXNB = 16;
+constexpr int CS_MAXCELLS = 4096;  // E * NB histogram cells held in LDS (twice: counts and prefixes)
+
+__global__ __launch_bounds__(256) void count_small_kernel(const int32_t* __restrict__ idx, int T, int k, int E, int W, int NB,
+                                                           int32_t* __restrict__ send_counts, int32_t* __restrict__ expert_offs,
+                                                           int32_t* __restrict__ dst_sizes, int32_t* __restrict__ dst_offsets,
+                                                           int32_t* __restrict__ caps, int32_t* __restrict__ pos,
+                                                           int32_t* __restrict__ row_token) {
+    __shared__ int32_t hist[CS_MAXCELLS];   // [e][b]
+    __shared__ int32_t base[CS_MAXCELLS];   // [e][b] rows of e in earlier blocks
+    __shared__ int32_t counts[MOE_MAX_EXPERTS];
+    __shared__ int32_t es[MOE_MAX_EXPERTS + 1];
+    __shared__ int32_t expert_start[MOE_MAX_EXPERTS + 1];
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    for (int i = threadIdx.x; i < E * NB; i += blockDim.x) hist[i] = 0;
+    __syncthreads();
+    for (int b = wave; b < NB; b += 4) {
+        const int t = b * CB + lane;
+        if (t < T)
+            for (int j = 0; j < k; ++j) {
+                const int e = idx[(size_t)t * k + j];
+                if ((unsigned)e < (unsigned)E) atomicAdd(&hist[e * NB + b], 1);
+            }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
+        int run = 0;
+        for (int b = 0; b < NB; ++b) { base[e * NB + b] = run; run += hist[e * NB + b]; }
+        counts[e] = run;
+    }
+    __syncthreads();
+    offsets_body(counts, E, W, es, expert_start, send_counts, expert_offs, dst_sizes, dst_offsets, caps);
+    __syncthreads();
+    for (int b = wave; b < NB; b += 4) rank_block(idx, base, expert_start, pos, row_token, T, k, E, NB, b);
 }
 
 // ---- small integer helpers --------------------------------------------------------------------------
@@ -545,6 +597,11 @@ extern "C" int moe_count_and_offsets(const int32_t* topk_idx, int T, int k, int 
     int32_t* base = hist + (size_t)E * NB;
     int32_t* counts = base + (size_t)E * NB;
     int32_t* expert_start = counts + E;
+    if (T > 0 && NB <= CS_MAXNB && E * NB <= CS_MAXCELLS) {
+        count_small_kernel<<<1, 256, 0, s>>>(topk_idx, T, k, E, W, NB, send_counts, expert_offs, dst_sizes, dst_offsets, caps, pos,
+                                             row_token);
+        return moe_check_launch("count_and_offsets");
+    }
     block_hist_kernel<<<ceil_div(NB, 4), 256, 4 * E * sizeof(int32_t), s>>>(topk_idx, hist, T, k, E, NB);
     scan_blocks_kernel<<<E, WAVE, 0, s>>>(hist, base, counts, NB);
     offsets_kernel<<<1, WAVE, 0, s>>>(counts, E, W, expert_start, send_counts, expert_offs, dst_sizes, dst_offsets, caps);
