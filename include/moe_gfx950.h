@@ -206,6 +206,11 @@ int moe_grouped_gemm_mapped(const void* a_base, int a_rows, const int32_t* a_row
                             int out_rows, const int32_t* c_row_map, void* part_ws, size_t part_ws_bytes,
                             moe_stream_t stream);
 size_t moe_gemm_part_workspace_bytes(void);
+/* How a launch with total_tiles output tiles, a persistent grid of `grid` workgroups, k_stages 64-byte stages of K
+ * (even) and room for max_units part tiles in the workspace is walked: out[0] = tiles taken whole, out[1] = parts
+ * per remaining tile (1: no split), out[2] = K stages per part, out[3] = work units in all.  Host-only arithmetic
+ * (the kernels evaluate the same function); no counterpart in the reference. */
+int moe_gemm_split_plan(int total_tiles, int grid, int k_stages, int max_units, int32_t* out);
 int moe_zero_padding_rows(void* buf, int dtype, int W, int M, int H, const int32_t* recv_counts, int E_l,
                           moe_stream_t stream);
 /* moe_grouped_mlp_fp8 with the same row indirection: the row quantisation reads input row r from row

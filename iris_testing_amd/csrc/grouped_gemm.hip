@@ -1031,6 +1031,16 @@ extern "C" int moe_grouped_gemm_packed(const void* tokens, const void* packed, c
     return launch_gemm<false>(p, act, (hipStream_t)stream);
 }
 
+// The tile walk of a launch as the kernels compute it (host side of the same function; no GPU needed):
+// out = {full, P, stages per part, work units}.  For callers that size workspaces and for tests.
+extern "C" int moe_gemm_split_plan(int total_tiles, int grid, int k_stages, int max_units, int32_t* out) {
+    MOE_REQUIRE(total_tiles >= 0 && grid > 0 && k_stages >= 2 && k_stages % 2 == 0 && max_units >= 0 && out, MOE_ERR_INVALID,
+                "gemm_split_plan: bad arguments");
+    const GgPlan pl = gg_plan(total_tiles, grid, k_stages, max_units >= 2, max_units);
+    out[0] = pl.full; out[1] = pl.P; out[2] = pl.nkp; out[3] = pl.units;
+    return MOE_OK;
+}
+
 extern "C" size_t moe_gemm_part_workspace_bytes(void) { return (size_t)num_cus() * 256 * GG_BN * sizeof(float); }
 
 extern "C" int moe_grouped_gemm_mapped(const void* a_base, int a_rows, const int32_t* a_row_map, const void* packed,

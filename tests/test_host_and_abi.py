@@ -75,3 +75,39 @@ def test_configs_and_generators_are_deterministic():
     assert abs(float(torch.exp(z).sum()) - 1) < 1e-5
     for name, c in CONFIGS.items():
         assert c.experts % c.world == 0 and c.topk <= c.experts, name
+
+
+def test_gemm_split_plan_covers_every_tile_and_every_k_stage_once():
+    """The walk of a grouped-GEMM launch (whole tiles, then the tiles of an under-filled last round cut along K) is
+    one host/device function; here its host side: every tile appears, the parts of a split tile tile its K range
+    exactly, every part has an even, non-zero number of stages, and the part tiles fit the workspace."""
+    import ctypes
+    import random
+    from iris_testing_amd import _lib as L
+    lib = L.lib()
+    out = (ctypes.c_int32 * 4)()
+    rnd = random.Random(3)
+    split_seen = 0
+    for _ in range(3000):
+        grid = rnd.choice([256, 256, 304, 64, 8])
+        total = rnd.randint(0, 4 * grid + 5)
+        nk = 2 * rnd.randint(1, 400)
+        max_units = rnd.choice([grid, grid // 2, 3, 1, 0])
+        assert lib.moe_gemm_split_plan(total, grid, nk, max_units, out) == 0
+        full, P, nkp, units = out[0], out[1], out[2], out[3]
+        tail = total - full
+        assert 0 <= full <= total and P >= 1 and units == full + tail * P
+        if P == 1:
+            assert full == total
+            continue
+        split_seen += 1
+        assert tail == total % grid and 4 * tail <= grid and tail * P <= min(grid, max_units) and P <= 16
+        assert nkp % 2 == 0 and nkp >= 8
+        stages = [min(nkp, nk - part * nkp) for part in range(P)]
+        assert sum(stages) == nk and all(s >= 2 and s % 2 == 0 for s in stages)
+    assert split_seen > 100
+    # the shapes of the bench workloads: Mixtral-style down GEMM (2064 tiles, 448 stages) and the small config's GEMMs
+    for total, nk, want in [(2064, 448, (2048, 16, 28)), (14448, 128, (14448, 1, 128)), (64, 64, (0, 4, 16)), (32, 128, (0, 8, 16))]:
+        lib.moe_gemm_split_plan(total, 256, nk, 256, out)
+        assert (out[0], out[1], out[2]) == want
+    assert lib.moe_gemm_split_plan(10, 0, 8, 4, out) != 0 and lib.moe_gemm_split_plan(10, 8, 7, 4, out) != 0
