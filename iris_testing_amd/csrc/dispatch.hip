@@ -108,46 +108,46 @@ __global__ __launch_bounds__(WAVE) void offsets_kernel(const int32_t* __restrict
 }
 
 // ---- 4. stable positions: one wave per 64-token block ----------------------------------------------
-// one wave ranks the slots of token block b
+// One wave ranks the slots of token block b: the rank of a slot among the block's slots of the same expert is the
+// number of lower lanes that hold that expert (a token holds an expert at most once), read off a 64-bit lane
+// mask per expert that the wave builds in LDS with one atomic OR per slot.  Called by every thread of a block
+// (it contains block barriers); waves without a block pass active = false.
 __device__ __forceinline__ void rank_block(const int32_t* __restrict__ idx, const int32_t* base, const int32_t* expert_start,
                                            int32_t* __restrict__ pos, int32_t* __restrict__ row_token, int T, int k, int E,
-                                           int NB, int b) {
+                                           int NB, int b, bool active, unsigned long long* mask /*[E], LDS, per wave*/) {
     const int lane = lane_id();
     const int t = b * CB + lane;
-    const bool live = t < T;
+    const bool live = active && t < T;
     int mine[MOE_MAX_TOPK];
 #pragma unroll
     for (int j = 0; j < MOE_MAX_TOPK; ++j) mine[j] = (live && j < k) ? idx[(size_t)t * k + j] : -1;
-    const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (WAVE - lane));
-    for (int e0 = 0; e0 < E; e0 += WAVE) {
-        // lane l prefetches the start row of expert e0+l for this block
-        const int el = e0 + lane;
-        const int start_l = el < E ? expert_start[el] + base[(size_t)el * NB + b] : 0;
-        const int n = min(WAVE, E - e0);
-        for (int i = 0; i < n; ++i) {
-            const int e = e0 + i;
-            int jm = -1;
+    if (active)
+        for (int e = lane; e < E; e += WAVE) mask[e] = 0ull;
+    __syncthreads();
 #pragma unroll
-            for (int j = 0; j < MOE_MAX_TOPK; ++j)
-                if (mine[j] == e) jm = j;
-            const unsigned long long m = __ballot(jm >= 0);
-            if (m == 0ull) continue;
-            const int start = __shfl(start_l, i, WAVE);
-            if (jm >= 0) {
-                const int p = start + __popcll(m & lt_mask);
-                pos[(size_t)t * k + jm] = p;
-                row_token[p] = t;
-            }
+    for (int j = 0; j < MOE_MAX_TOPK; ++j)
+        if ((unsigned)mine[j] < (unsigned)E) atomicOr(&mask[mine[j]], 1ull << lane);
+    __syncthreads();
+    const unsigned long long lt_mask = (lane == 0) ? 0ull : (~0ull >> (WAVE - lane));
+#pragma unroll
+    for (int j = 0; j < MOE_MAX_TOPK; ++j) {
+        const int e = mine[j];
+        if ((unsigned)e < (unsigned)E) {
+            const int p = expert_start[e] + base[(size_t)e * NB + b] + __popcll(mask[e] & lt_mask);
+            pos[(size_t)t * k + j] = p;
+            row_token[p] = t;
         }
     }
+    __syncthreads();  // the masks are reused by the caller's next block
 }
 
 __global__ __launch_bounds__(256) void rank_kernel(const int32_t* __restrict__ idx, const int32_t* __restrict__ base,
                                                     const int32_t* __restrict__ expert_start, int32_t* __restrict__ pos,
                                                     int32_t* __restrict__ row_token, int T, int k, int E, int NB) {
-    const int b = blockIdx.x * 4 + threadIdx.x / WAVE;
-    if (b >= NB) return;
-    rank_block(idx, base, expert_start, pos, row_token, T, k, E, NB, b);
+    __shared__ unsigned long long masks[4][MOE_MAX_EXPERTS];
+    const int wave = threadIdx.x / WAVE;
+    const int b = blockIdx.x * 4 + wave;
+    rank_block(idx, base, expert_start, pos, row_token, T, k, E, NB, b, b < NB, masks[wave]);
 }
 
 // ---- the four steps above in one block, for few tokens (NB <= CS_MAXNB blocks of 64): launch latency is all that
@@ -165,6 +165,7 @@ __global__ __launch_bounds__(256) void count_small_kernel(const int32_t* __restr
     __shared__ int32_t counts[MOE_MAX_EXPERTS];
     __shared__ int32_t es[MOE_MAX_EXPERTS + 1];
     __shared__ int32_t expert_start[MOE_MAX_EXPERTS + 1];
+    __shared__ unsigned long long masks[4][MOE_MAX_EXPERTS];
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     for (int i = threadIdx.x; i < E * NB; i += blockDim.x) hist[i] = 0;
     __syncthreads();
@@ -185,7 +186,8 @@ __global__ __launch_bounds__(256) void count_small_kernel(const int32_t* __restr
     __syncthreads();
     offsets_body(counts, E, W, es, expert_start, send_counts, expert_offs, dst_sizes, dst_offsets, caps);
     __syncthreads();
-    for (int b = wave; b < NB; b += 4) rank_block(idx, base, expert_start, pos, row_token, T, k, E, NB, b);
+    for (int b0 = 0; b0 < NB; b0 += 4)  // (uniform trip count: rank_block holds block barriers)
+        rank_block(idx, base, expert_start, pos, row_token, T, k, E, NB, b0 + wave, b0 + wave < NB, masks[wave]);
 }
 
 // ---- small integer helpers --------------------------------------------------------------------------
