@@ -1,4 +1,4 @@
-"""The three large workloads at their full BASELINE sizes, through the pipeline the benchmark times.
+"""The three large workloads at their full published sizes, through the pipeline the benchmark times.
 What the oracle can finish in seconds is compared directly (shard-0 routing, counts, the packed send
 buffer, sampled expert rows); the rest is pinned by size-independent properties: the return pack is the
 exact inverse of the unpack, every received row appears exactly once, combine is linear under exact
