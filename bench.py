@@ -212,7 +212,7 @@ def main():
         else:
             w_np = tuple(to_np(t) for t in raw)
         flops_per_token = 2 * cfg.hidden * cfg.ffn * cfg.n_mat * cfg.topk
-        sample = args.cpu_sample_tokens or max(64, min(cfg.tokens, int(4e12 / flops_per_token)))
+        sample = args.cpu_sample_tokens or max(64, min(cfg.tokens, int(1.2e13 / flops_per_token)))
         v, secs, threads, desc = cpu_baseline(cfg, (x_np, router_np, bias_np, w_np), sample)
         out["cpu_baseline"] = {"value": round(v, 1), "unit": "tokens/s", "cores": threads, "kind": "port",
                                "sample": desc, "seconds": round(secs, 2)}
