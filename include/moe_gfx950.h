@@ -213,6 +213,11 @@ size_t moe_gemm_part_workspace_bytes(void);
 int moe_gemm_split_plan(int total_tiles, int grid, int k_stages, int max_units, int32_t* out);
 int moe_zero_padding_rows(void* buf, int dtype, int W, int M, int H, const int32_t* recv_counts, int E_l,
                           moe_stream_t stream);
+/* Gradient of moe_shuffle (the reference leaves TokenShuffle.backward empty, token_shuffle.py:58-60):
+ * grad_token_buf[e,s,j,:] = grad_rows[off[e,s]+j,:] for j < pca[e,s], zeros in the padding; off as in moe_shuffle.
+ * map_ws >= moe_recv_map_ints(W,E_l,0) ints. */
+int moe_shuffle_backward(const void* grad_rows, int dtype, int E_l, int W, int CAP, int H, const int32_t* pca,
+                         void* grad_token_buf, int32_t* map_ws, moe_stream_t stream);
 /* moe_grouped_mlp_fp8 with the same row indirection: the row quantisation reads input row r from row
  * a_row_map[r] of a_base_bf16 (a_rows rows of H), the down GEMM writes result row r to row c_row_map[r]
  * of out (out_rows rows of H); either map may be NULL. */

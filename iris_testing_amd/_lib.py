@@ -44,6 +44,7 @@ _SIGNATURES = {
     "moe_unpack_token_buf": (c_int, [P, c_int, c_int, c_int, c_int, P, c_int, c_int, P, P, P, P, P]),
     "moe_reorder_flat_to_token_buf": (c_int, [P, c_int, c_int, c_int, P, c_int, c_int, c_int, P, P, P, P]),
     "moe_shuffle": (c_int, [P, c_int, c_int, c_int, c_int, c_int, P, P, c_int, P, P, P]),
+    "moe_shuffle_backward": (c_int, [P, c_int, c_int, c_int, c_int, c_int, P, P, P, P]),
     "moe_unpack_expert_major": (c_int, [P, c_int, c_int, c_int, c_int, P, c_int, P, c_int, P, P, P]),
     "moe_prepack_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "moe_prepack_weights": (c_int, [P, P, c_int, c_int, c_int, c_int, P, P]),

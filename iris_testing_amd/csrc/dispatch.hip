@@ -276,7 +276,8 @@ enum {
     SRC_TOKBUF = 3,   // token_buf row (e,s,j) -> recv row       (recv [W,M,H] -> [E_l,W,CAP,H])
     SRC_RETURN = 4,   // return slot (s,m) -> expert-major row   ([S,H] -> [W,M,H])
     SRC_REORDER = 5,  // token_buf row (e,s,j) -> flat row       (flat payload -> [E_l,W,CAP,H])
-    SRC_SHUFFLE = 6   // expert-major row r -> token_buf row     ([E_l,W,CAP,H] -> [S,H])
+    SRC_SHUFFLE = 6,  // expert-major row r -> token_buf row     ([E_l,W,CAP,H] -> [S,H])
+    SRC_UNSHUFFLE = 7 // token_buf row (e,s,j) -> expert-major row ([S,H] -> [E_l,W,CAP,H]; the shuffle's gradient)
 };
 
 struct RowSource {
@@ -325,6 +326,10 @@ __device__ __forceinline__ int source_row(const RowSource& a, int r) {
             if (j == 0 && c > a.CAP && a.status && lane_id() == 0) *a.status = 1;
             if (j >= c) return -1;
             return a.mode == SRC_TOKBUF ? s * a.M + a.src_off[s * a.E_l + e] + j : a.flat_off[s * a.E_l + e] + j;
+        }
+        case SRC_UNSHUFFLE: {
+            const int j = r % a.CAP, s = (r / a.CAP) % a.W, e = r / (a.CAP * a.W);
+            return j < a.rc[s * a.E_l + e] ? a.row_off[e * a.W + s] + j : -1;
         }
         default: {  // SRC_RETURN
             const int s = r / a.M, m = r % a.M;
@@ -690,7 +695,8 @@ static int recv_driven(const char* who, int mode, const void* src, void* dst, in
     int32_t* flat_off = tables + 2 * (n + 1);
     recv_tables_kernel<<<1, WAVE, 0, s>>>(rc_dev, W, E_l, src_off, row_off, flat_off, pca, expert_cnt);
     if (n_out == 0) return moe_check_launch(who);
-    MOE_REQUIRE(dst && (src || mode == SRC_REORDER), MOE_ERR_INVALID, "%s: null pointer", who);  // an empty flat payload has no storage
+    // (an empty flat payload or gradient has no storage: every output row is then padding and the source is never read)
+    MOE_REQUIRE(dst && (src || mode == SRC_REORDER || mode == SRC_UNSHUFFLE), MOE_ERR_INVALID, "%s: null pointer", who);
     RowSource a{};
     a.mode = mode;
     a.rc = rc_dev; a.src_off = src_off; a.row_off = row_off; a.flat_off = flat_off;
@@ -775,6 +781,19 @@ extern "C" int moe_shuffle(const void* token_buf, int dtype, int E_l, int W, int
     transpose_counts_kernel<<<ceil_div(W * E_l, 256), 256, 0, s>>>(pca, E_l, W, rc_t);
     return recv_driven("shuffle", SRC_SHUFFLE, token_buf, shuffled, dtype, H, rc_t, W, E_l, 1, CAP, S_rows, nullptr, expert_cnt,
                        map_ws, nullptr, s);
+}
+
+// gradient of moe_shuffle: grad_token_buf[e,s,j,:] = grad_rows[off[e,s] + j,:] for j < pca[e,s], zeros elsewhere
+extern "C" int moe_shuffle_backward(const void* grad_rows, int dtype, int E_l, int W, int CAP, int H, const int32_t* pca,
+                                    void* grad_token_buf, int32_t* map_ws, moe_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    MOE_REQUIRE(W > 0 && E_l > 0 && W * E_l <= MOE_MAX_EXPERTS && CAP >= 1 && pca && map_ws, MOE_ERR_INVALID,
+                "shuffle_backward: bad arguments");
+    MOE_REQUIRE((long long)E_l * W * CAP < (1ll << 31), MOE_ERR_UNSUPPORTED, "shuffle_backward: too many rows");
+    int32_t* rc_t = map_ws + 3 * (W * E_l + 1);  // recv_counts[s,e] = pca[e,s], kept behind the tables
+    transpose_counts_kernel<<<ceil_div(W * E_l, 256), 256, 0, s>>>(pca, E_l, W, rc_t);
+    return recv_driven("shuffle_backward", SRC_UNSHUFFLE, grad_rows, grad_token_buf, dtype, H, rc_t, W, E_l, 1, CAP, E_l * W * CAP,
+                       nullptr, nullptr, map_ws, nullptr, s);
 }
 
 extern "C" int moe_return_pack(const void* y, int dtype, int S_rows, int H, const int32_t* recv_counts, int W, int E_l,

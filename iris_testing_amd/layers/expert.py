@@ -21,11 +21,39 @@ class Expert(torch.autograd.Function):
         assert tokens.is_cuda, "tokens must be CUDA"
         _assert_cuda_int32(local_expert_cnt, "local_expert_cnt")
         assert weights.shape[0] == local_expert_cnt.numel(), "one row count per local expert"
+        ctx.save_for_backward(tokens, weights, local_expert_cnt)
         return ops.grouped_gemm(tokens.contiguous(), weights.contiguous(), local_expert_cnt.contiguous())
 
     @staticmethod
     def backward(ctx, do):
-        raise NotImplementedError("Backward pass not implemented yet.")
+        """Gradients of out[rows of g] = tokens[rows of g] @ weights[g] (not implemented in the reference,
+        layers/expert.py:62-64), both on the grouped GEMM kernel:
+          d tokens[rows of g] = do[rows of g] @ weights[g]^T        one grouped launch over the transposed weights
+          d weights[g]        = tokens[rows of g]^T @ do[rows of g]  one launch per expert: the reduction runs over
+                                                                      the expert's rows, zero padded to 64
+        Rows past the counted total get a zero gradient."""
+        tokens, weights, cnt = ctx.saved_tensors
+        do = do.contiguous()
+        E_l, H, F = weights.shape
+        d_tokens = ops.grouped_gemm(do, weights.transpose(1, 2).contiguous(), cnt.contiguous())
+        counts = [max(int(c), 0) for c in cnt.cpu().tolist()]
+        total = min(sum(counts), tokens.shape[0])
+        if total < tokens.shape[0]:
+            d_tokens[total:].zero_()
+        d_weights = torch.zeros_like(weights)
+        h_rows = torch.full((1,), H, dtype=torch.int32, device=tokens.device)
+        row0 = 0
+        for g, c in enumerate(counts):
+            c = min(c, tokens.shape[0] - row0)
+            if c > 0:
+                pad = (c + 63) // 64 * 64
+                xt = torch.zeros((H, pad), dtype=tokens.dtype, device=tokens.device)
+                xt[:, :c] = tokens[row0:row0 + c].t()
+                dy = torch.zeros((1, pad, F), dtype=do.dtype, device=do.device)
+                dy[0, :c] = do[row0:row0 + c]
+                d_weights[g] = ops.grouped_gemm(xt, dy, h_rows)
+            row0 += c
+        return d_tokens, d_weights, None, None
 
 
 expert = Expert.apply

@@ -26,11 +26,17 @@ class TokenShuffle(torch.autograd.Function):
                 raise RuntimeError("token_sync shows an incomplete transfer (expected >= world_size)")
         total = int(pca.sum().item())
         out, _ = ops.shuffle_rows(dispatched_tokens.contiguous(), pca.contiguous(), total)
+        ctx.save_for_backward(pca)
+        ctx.capacity = dispatched_tokens.shape[2]
         return out
 
     @staticmethod
-    def backward(ctx, *grad_outputs):
-        raise NotImplementedError("Backward pass not implemented yet.")
+    def backward(ctx, grad_shuffled):
+        """The shuffle is a row permutation that drops the padding, so its gradient puts row off[e,src] + j back
+        at [e, src, j] and leaves zeros in the padding (empty in the reference, token_shuffle.py:58-60)."""
+        (pca,) = ctx.saved_tensors
+        grad = ops.shuffle_rows_backward(grad_shuffled.contiguous(), pca.contiguous(), ctx.capacity)
+        return grad, None, None
 
 
 shuffle = TokenShuffle.apply

@@ -199,6 +199,19 @@ def shuffle_rows(token_buf: torch.Tensor, pca: torch.Tensor, S_rows: int, out: O
     return out, expert_cnt
 
 
+def shuffle_rows_backward(grad_rows: torch.Tensor, pca: torch.Tensor, capacity: int) -> torch.Tensor:
+    """Gradient of shuffle_rows: [S,H] expert-major rows back into the zero-padded [E_l,W,CAP,H] layout."""
+    _req_cuda(grad_rows, "grad_rows")
+    _req_i32(pca, "pca")
+    E_l, W = pca.shape
+    H = grad_rows.shape[1]
+    out = torch.empty((E_l, W, capacity, H), dtype=grad_rows.dtype, device=grad_rows.device)
+    ws = _map_ws(W, E_l, 0, grad_rows.device)
+    L.check(L.lib().moe_shuffle_backward(L.ptr(grad_rows), L.dtype_code(grad_rows.dtype), E_l, W, capacity, H, L.ptr(pca),
+                                         L.ptr(out), L.ptr(ws), L.stream_ptr()))
+    return out
+
+
 def unpack_expert_major(recv: torch.Tensor, recv_counts: torch.Tensor, S_rows: int,
                         out: Optional[torch.Tensor] = None, expert_cnt: Optional[torch.Tensor] = None,
                         map_ws=None) -> Tuple[torch.Tensor, torch.Tensor]:

@@ -134,3 +134,64 @@ def test_benchmark_driver_point_and_overflow_report(capsys):
     assert "[SKIP] max_recv_count=" in out and "=== Correctness Report ===" in out and out.rstrip().endswith("PASS")
     assert res["ok"] and res["world"] == 4 and res["e_local"] == 3 and res["cap"] > 8
     assert res["source_ms"] > 0 and res["dest_ms"] > 0 and res["dest_direct_ms"] > 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_shuffle_backward_puts_rows_back_and_zeroes_the_padding(dtype):
+    """Gradient of the expert-major unpack (empty in the reference, token_shuffle.py:58-60): the shuffle is a row
+    permutation that drops the padding, so the gradient of token_buf[e, src, j] is the gradient of the row it
+    went to, and zero in the padding -- exact, whatever the dtype."""
+    rng = np.random.default_rng(11)
+    E_l, W, CAP, H = 3, 4, 9, 64
+    pca = rng.integers(0, CAP + 1, size=(E_l, W)).astype(np.int32)
+    pca[1, 2] = 0
+    S = int(pca.sum())
+    tb = torch.from_numpy(rng.standard_normal((E_l, W, CAP, H)).astype(np.float32)).to(DEV).to(dtype).requires_grad_(True)
+    out = shuffle(tb, torch.from_numpy(pca).to(DEV), None)
+    assert out.shape == (S, H)
+    g = torch.from_numpy(rng.standard_normal((S, H)).astype(np.float32)).to(DEV).to(dtype)
+    out.backward(g)
+    want = np.zeros((E_l, W, CAP, H), np.float32)
+    gn, r = to_np(g), 0
+    for e in range(E_l):
+        for s in range(W):
+            want[e, s, :pca[e, s]] = gn[r:r + pca[e, s]]
+            r += pca[e, s]
+    assert_bits_equal(tb.grad, want if dtype == torch.float32 else torch.from_numpy(want).to(dtype), "grad of token_buf")
+    # nothing received: the gradient is all padding
+    tb0 = torch.zeros((2, 2, 3, 64), device=DEV, dtype=dtype, requires_grad=True)
+    out0 = shuffle(tb0, torch.zeros((2, 2), dtype=torch.int32, device=DEV), None)
+    out0.backward(torch.zeros_like(out0))
+    assert out0.shape == (0, 64) and bool((tb0.grad == 0).all())
+
+
+@pytest.mark.parametrize("dtype,H,F,cnt", [(torch.float32, 96, 72, (70, 0, 45)), (torch.bfloat16, 128, 192, (70, 0, 45)),
+                                           (torch.bfloat16, 256, 320, (300, 17, 0, 129))])
+def test_expert_backward_matches_float64_autograd(dtype, H, F, cnt):
+    """Gradients of the grouped GEMM layer (not implemented in the reference, layers/expert.py:62-64) against
+    float64 autograd of  out[rows of g] = tokens[rows of g] @ weights[g]  on the CPU -- parity unpinned by the
+    reference, pinned by the mathematics.  Rows past the counted total take no part and get a zero gradient."""
+    rng = np.random.default_rng(H + F)
+    cnt = np.array(cnt, dtype=np.int32)
+    S = int(cnt.sum()) + 5
+    x = torch.from_numpy(rng.standard_normal((S, H)).astype(np.float32)).to(dtype)
+    w = torch.from_numpy((rng.standard_normal((len(cnt), H, F)) * H ** -0.5).astype(np.float32)).to(dtype)
+    g = torch.from_numpy(rng.standard_normal((S, F)).astype(np.float32)).to(dtype)
+    xd, wd = x.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+    out = expert(xd, wd, torch.from_numpy(cnt).to(DEV), int(cnt.sum()))
+    out.backward(g.to(DEV))
+    x64, w64 = x.double().requires_grad_(True), w.double().requires_grad_(True)
+    parts, r = [], 0
+    for e, c in enumerate(cnt):
+        parts.append(x64[r:r + c] @ w64[e])
+        r += c
+    ref = torch.cat(parts + [torch.zeros((S - r, F), dtype=torch.float64)])
+    ref.backward(g.double())
+    tol = 1e-4 if dtype == torch.float32 else 2.0 ** -6
+    for name, got, want in (("d tokens", xd.grad, x64.grad), ("d weights", wd.grad, w64.grad)):
+        got, want = got.double().cpu(), want
+        scale = float(want.abs().max()) + 1e-30
+        err = float((got - want).abs().max()) / scale
+        print(f"{name}: max error / max |gradient| = {err:.2e}", flush=True)
+        assert err < tol, f"{name}: {err}"
+    assert bool((xd.grad[int(cnt.sum()):] == 0).all()) and bool((wd.grad[cnt == 0] == 0).all())
