@@ -14,7 +14,9 @@
 //     MFMA operands are read as 128-bit fragments;
 //   * ragged group tails are masked (the reference assumes full tiles, kernels.py:270,282);
 //   * the tile walk is XCD-aware: the 32 workgroups that share an L2 take a compact 4 x 8 patch of
-//     a 16 x 16 super-tile.
+//     a 16 x 16 super-tile;
+//   * a last round of the persistent grid that would leave most compute units idle is split along K over all
+//     of them (second launch + a reduction kernel that applies the epilogue), given a workspace.
 #include "common.h"
 #include <algorithm>
 #include <type_traits>
@@ -203,11 +205,13 @@ __device__ __forceinline__ void gg_wait() {
 
 // NWM x 2 wave64s per workgroup; every wave owns a (BM/NWM) x 128 block of the tile.
 //
-// K moves through LDS in a ring of NRING stages of ROWB bytes per tile row.  A stage is two MFMA
-// blocks (one per 32 bytes of K).  The loads of stage s+4 go into the slot of stage s as soon as every
-// wave holds the last fragments of stage s in registers, and are spread over the two MFMA blocks that
-// follow, so the load pipe sees a steady stream instead of a burst and every load has two full stages
-// of MFMA work to land.
+// K moves through LDS in a ring of NRING stages of ROWB bytes per tile row.  A stage is one MFMA block
+// (one 16x16x32 bf16 or 32x32x64 fp8 MFMA per pair of fragments).  The loads of stage s+4 go into the slot of
+// stage s during block s -- every wave took the fragments of stage s into registers one block earlier -- spread
+// over the block, so the load pipe sees a steady stream instead of a burst and every load has more than two
+// blocks of MFMA work to land.
+// SPLIT = false: the launch that takes whole tiles.  SPLIT = true: the launch that takes the tiles of an
+// under-filled last round in parts of the K range and leaves fp32 partial sums in the workspace (GemmParams).
 template <int BM, int NWM, int EPI, bool FP8, bool SPLIT>
 __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const GemmParams p) {
     constexpr int BN = GG_BN;
