@@ -9,7 +9,7 @@
 // Order of rows inside a (dst, el) bucket is ascending token index (utils.py:210-219).  An
 // atomic-counter scatter would not reproduce that, so the position of every routed slot is
 // computed as   expert_start[ex] + (rows of ex in earlier 64-token blocks) + (rows of ex in
-// earlier lanes of this block),  with LDS histograms, a wave prefix scan and wave ballots.
+// earlier lanes of this block),  with LDS histograms, a wave prefix scan and per-expert lane masks.
 // All integer work: results are bit-exact by construction.
 #include "common.h"
 
