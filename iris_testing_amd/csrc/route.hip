@@ -51,9 +51,9 @@ struct VecLoad<float> {
 //   B operand: lane l holds w[h][e0 + l % SHAPE]         (the SHAPE experts, repeated across the lanes)
 //   D, SHAPE = 16: register v holds token t0 + 16 * (v / 4) + 4 * (l / 16) + v % 4, expert e0 + l % 16
 //   D, SHAPE = 4:  register v holds token t0 + 4 * (l / 4) + v,                     expert e0 + l % 4
-// Block = NWV waves on the same 64 tokens, wave i on experts [e0 + i * SHAPE, + SHAPE).  x goes through LDS in
-// its storage type (the lane reads its own row, 16 bytes at a time), the router slab is converted to fp32 and
-// transposed on its way into LDS (the lane reads four consecutive h of its expert with one 128-bit read).
+// Block = NWV waves on the same 64 tokens, wave i on experts [e0 + i * SHAPE, + SHAPE).  Both operands are converted
+// to fp32 on their way into LDS (the lane reads four consecutive h of its own token row, and of its expert in the
+// transposed router slab, with one 128-bit read each).
 typedef float rt_f4 __attribute__((ext_vector_type(4)));
 typedef float rt_f16 __attribute__((ext_vector_type(16)));
 typedef unsigned int rt_u4 __attribute__((ext_vector_type(4)));
@@ -67,7 +67,7 @@ __global__ __launch_bounds__(NWV * WAVE) void route_logits_mfma_kernel(const XT*
     constexpr int EB = NWV * SHAPE;            // experts per block
     constexpr int VN = VecLoad<XT>::N;         // elements per 16 bytes
     constexpr int KC = 16 * VN;                // h per slab: 256 bytes of every token row
-    constexpr int XS = KC + VN;                // padded row (conflict-free 128-bit row reads)
+    constexpr int XS = KC + 4;                 // padded fp32 row (conflict-free 128-bit row reads)
     constexpr int XPT = RT_TB * 16 / NTH;      // 16-byte x chunks per thread and slab
     constexpr int WQ = KC * EB / (4 * NTH);    // groups of four h of one expert per thread and slab
     // slabs in flight per block: one block holds D x 16 KB of token rows in registers, which is what hides the
@@ -76,13 +76,13 @@ __global__ __launch_bounds__(NWV * WAVE) void route_logits_mfma_kernel(const XT*
     constexpr int NACC = SHAPE == 16 ? 16 : 4;
     typedef typename std::conditional<SHAPE == 16, rt_f16, rt_f4>::type acc_t;
     static_assert((KC * EB) % (4 * NTH) == 0, "router slab split");
-    __shared__ __align__(16) XT xs[RT_TB][XS];
+    __shared__ __align__(16) float xs[RT_TB][XS];
     __shared__ __align__(16) float wsT[EB][KC + 4];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int t0 = blockIdx.x * RT_TB, eb0 = blockIdx.y * EB;
     const float* wrow = &wsT[wave * SHAPE + lane % SHAPE][0];
-    const XT* xrow = &xs[lane][0];
+    const float* xrow = &xs[lane][0];
     acc_t acc;
 #pragma unroll
     for (int v = 0; v < NACC; ++v) acc[v] = 0.f;
@@ -118,12 +118,23 @@ __global__ __launch_bounds__(NWV * WAVE) void route_logits_mfma_kernel(const XT*
         _Pragma("unroll") for (int i = 0; i < WQ; ++i)                                                        \
             _Pragma("unroll") for (int q = 0; q < 4; ++q) wr[d][i][q] = wb_[woff[i][q]];                      \
     } while (0)
-    // registers -> LDS: token rows as they are, the router slab as fp32, transposed (one 128-bit write per four h)
+    // registers -> LDS: token rows as fp32 (converted here, once per block, and not by every wave in its MFMA chain),
+    // the router slab as fp32, transposed (one 128-bit write per four h)
 #define RT_STASH(d)                                                                                                  \
     do {                                                                                                             \
         _Pragma("unroll") for (int i = 0; i < XPT; ++i) {                                                             \
             const int c = tid + i * NTH;                                                                             \
-            *reinterpret_cast<rt_u4*>(&xs[c / 16][(c % 16) * VN]) = xr[d][i];                                        \
+            if constexpr (VN == 8) {                                                                                 \
+                const rt_u4 r_ = xr[d][i];                                                                           \
+                const rt_f4 lo_ = {__uint_as_float(r_.x << 16), __uint_as_float(r_.x & 0xffff0000u),                 \
+                                   __uint_as_float(r_.y << 16), __uint_as_float(r_.y & 0xffff0000u)};                \
+                const rt_f4 hi_ = {__uint_as_float(r_.z << 16), __uint_as_float(r_.z & 0xffff0000u),                 \
+                                   __uint_as_float(r_.w << 16), __uint_as_float(r_.w & 0xffff0000u)};                \
+                *reinterpret_cast<rt_f4*>(&xs[c / 16][(c % 16) * VN]) = lo_;                                         \
+                *reinterpret_cast<rt_f4*>(&xs[c / 16][(c % 16) * VN + 4]) = hi_;                                     \
+            } else {                                                                                                 \
+                *reinterpret_cast<rt_u4*>(&xs[c / 16][(c % 16) * VN]) = xr[d][i];                                    \
+            }                                                                                                        \
         }                                                                                                            \
         _Pragma("unroll") for (int i = 0; i < WQ; ++i) {                                                              \
             const int c = tid + i * NTH;                                                                             \
@@ -133,30 +144,24 @@ __global__ __launch_bounds__(NWV * WAVE) void route_logits_mfma_kernel(const XT*
         }                                                                                                            \
     } while (0)
 
-    // One chunk = VN consecutive h (16 bytes of the lane's token row): VN chained MFMAs.  Within one wave a
-    // vector instruction does not overlap the chain (measured: one VALU between two dependent MFMAs adds 12 to 14
-    // cycles, a second one 8 more), so the conversions and LDS reads are not spread between the MFMAs but issued
-    // as one group ahead of them: token bytes are read two chunks ahead and converted one chunk ahead, router
-    // values are read one chunk ahead, and nothing in the chain waits for LDS.
+    // One chunk = VN consecutive h of the lane's token row: VN chained MFMAs.  Within one wave a vector
+    // instruction does not overlap the chain (measured: one VALU between two dependent MFMAs adds 12 to 14 cycles,
+    // a second one 8 more), so the chain's wave does no arithmetic of its own: the operands of the next chunk come
+    // out of LDS ready made (token values converted at the stash), read as one group ahead of the chunk's MFMAs.
 #define RT_MFMA(XV, WV, u)                                                                                           \
     do {                                                                                                             \
-        if constexpr (SHAPE == 16) acc = __builtin_amdgcn_mfma_f32_16x16x1f32(XV[u], WV[(u) / 4][(u) % 4], acc, 0, 0, 0); \
-        else acc = __builtin_amdgcn_mfma_f32_4x4x1f32(XV[u], WV[(u) / 4][(u) % 4], acc, 0, 0, 0);                    \
+        if constexpr (SHAPE == 16)                                                                                   \
+            acc = __builtin_amdgcn_mfma_f32_16x16x1f32(XV[(u) / 4][(u) % 4], WV[(u) / 4][(u) % 4], acc, 0, 0, 0);    \
+        else acc = __builtin_amdgcn_mfma_f32_4x4x1f32(XV[(u) / 4][(u) % 4], WV[(u) / 4][(u) % 4], acc, 0, 0, 0);     \
         __builtin_amdgcn_sched_barrier(0);                                                                           \
     } while (0)
-    // (an empty asm statement that "modifies" a value keeps its computation where it is written: it would
-    // otherwise sink to its first use, out of the shadow of the MFMAs)
-#define RT_PIN(a) asm volatile("" : "+v"(a))
-    // element u of a 16-byte piece of a token row as fp32
-#define RT_CVT(RAW, u) (VN == 8 ? __uint_as_float(((u) & 1) ? (RAW[(u) / 2] & 0xffff0000u) : (RAW[(u) / 2] << 16)) : __uint_as_float(RAW[(u) & 3]))
-    // chunk c: MFMAs on XV / WV; meanwhile RAWN (chunk c+1, read one chunk ago) is converted into XN, the router
-    // values of chunk c+1 are read into WN and the token bytes of chunk c+2 into RAWF
-#define RT_CHUNK(XV, WV, XN, WN, RAWN, RAWF, nxt1, nxt2)                                                             \
+    // chunk c: MFMAs on XV / WV, behind the LDS reads of chunk c+1 (at slab offset nxt) into XN / WN
+#define RT_CHUNK(XV, WV, XN, WN, nxt)                                                                                \
     do {                                                                                                             \
-        RAWF = *reinterpret_cast<const rt_u4*>(xrow + (nxt2));                                                       \
-        WN[0] = *reinterpret_cast<const rt_f4*>(wrow + (nxt1));                                                      \
-        if constexpr (VN == 8) WN[1] = *reinterpret_cast<const rt_f4*>(wrow + (nxt1) + 4);                           \
-        _Pragma("unroll") for (int u_ = 0; u_ < VN; ++u_) { XN[u_] = RT_CVT(RAWN, u_); RT_PIN(XN[u_]); }             \
+        _Pragma("unroll") for (int q_ = 0; q_ < VN / 4; ++q_) {                                                       \
+            XN[q_] = *reinterpret_cast<const rt_f4*>(xrow + (nxt) + 4 * q_);                                         \
+            WN[q_] = *reinterpret_cast<const rt_f4*>(wrow + (nxt) + 4 * q_);                                         \
+        }                                                                                                            \
         __builtin_amdgcn_sched_barrier(0);                                                                           \
         RT_MFMA(XV, WV, 0); RT_MFMA(XV, WV, 1); RT_MFMA(XV, WV, 2); RT_MFMA(XV, WV, 3);                              \
         if constexpr (VN == 8) { RT_MFMA(XV, WV, 4); RT_MFMA(XV, WV, 5); RT_MFMA(XV, WV, 6); RT_MFMA(XV, WV, 7); }   \
@@ -181,29 +186,24 @@ __global__ __launch_bounds__(NWV * WAVE) void route_logits_mfma_kernel(const XT*
             const int sh = k0 - min(k0, ks_max);        // where h = k0 sits in the slab
             const int kend = sh + max(min(KC, H - k0), 0);
             if (sh < kend) {
-                float xa[VN], xb[VN];
-                rt_f4 wa[2], wb[2];
-                rt_u4 ra, rb;
-                {
-                    ra = *reinterpret_cast<const rt_u4*>(xrow + sh);
-                    rb = *reinterpret_cast<const rt_u4*>(xrow + min(sh + VN, KC - VN));
+                rt_f4 xa[2], xb[2], wa[2], wb[2];
 #pragma unroll
-                    for (int q = 0; q < VN / 4; ++q) wa[q] = *reinterpret_cast<const rt_f4*>(wrow + sh + 4 * q);
-#pragma unroll
-                    for (int u = 0; u < VN; ++u) xa[u] = RT_CVT(ra, u);
+                for (int q = 0; q < VN / 4; ++q) {
+                    xa[q] = *reinterpret_cast<const rt_f4*>(xrow + sh + 4 * q);
+                    wa[q] = *reinterpret_cast<const rt_f4*>(wrow + sh + 4 * q);
                 }
                 if (sh == 0 && kend == KC) {
-                    // a whole slab: sixteen chunks of straight-line code (reads past the last chunk repeat it)
-#define RT_PAIR(c) /* chunks c (even) and c + 1 */                                                                    \
-    RT_CHUNK(xa, wa, xb, wb, rb, ra, ((c) + 1) * VN, ((c) + 2 < 16 ? (c) + 2 : 15) * VN);                              \
-    RT_CHUNK(xb, wb, xa, wa, ra, rb, ((c) + 2 < 16 ? (c) + 2 : 15) * VN, ((c) + 3 < 16 ? (c) + 3 : 15) * VN)
+                    // a whole slab: sixteen chunks of straight-line code (the read past the last chunk repeats it)
+#define RT_PAIR(c) /* chunks c (even) and c + 1 */                                         \
+    RT_CHUNK(xa, wa, xb, wb, ((c) + 1) * VN);                                              \
+    RT_CHUNK(xb, wb, xa, wa, ((c) + 2 < 16 ? (c) + 2 : 15) * VN)
                     RT_PAIR(0); RT_PAIR(2); RT_PAIR(4); RT_PAIR(6); RT_PAIR(8); RT_PAIR(10); RT_PAIR(12); RT_PAIR(14);
 #undef RT_PAIR
                 } else {
                     for (int kk = sh; kk < kend; kk += 2 * VN) {
-                        // chunks past the last one are read from a clamped (valid) place and never used
-                        RT_CHUNK(xa, wa, xb, wb, rb, ra, min(kk + VN, KC - VN), min(kk + 2 * VN, KC - VN));
-                        if (kk + VN < kend) RT_CHUNK(xb, wb, xa, wa, ra, rb, min(kk + 2 * VN, KC - VN), min(kk + 3 * VN, KC - VN));
+                        // the chunk past the last one is read from a clamped (valid) place and never used
+                        RT_CHUNK(xa, wa, xb, wb, min(kk + VN, KC - VN));
+                        if (kk + VN < kend) RT_CHUNK(xb, wb, xa, wa, min(kk + 2 * VN, KC - VN));
                     }
                 }
             }
@@ -211,8 +211,6 @@ __global__ __launch_bounds__(NWV * WAVE) void route_logits_mfma_kernel(const XT*
         }
     }
 #undef RT_CHUNK
-#undef RT_CVT
-#undef RT_PIN
 #undef RT_MFMA
 #undef RT_STASH
 #undef RT_FETCH
