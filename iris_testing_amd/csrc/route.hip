@@ -330,8 +330,9 @@ extern "C" int moe_route_topk(const void* x, const void* router, const float* bi
                  ? launch_logits<float>((const float*)x, (const float*)router, bias, logits_ws, T, H, E, s)
                  : launch_logits<bf16_t>((const bf16_t*)x, (const bf16_t*)router, bias, logits_ws, T, H, E, s);
     if (rc) return rc;
+    // lanes per token: the fewest that hold all experts at TK_MAXV per lane (more tokens per wave, fewer shuffles)
     int G = 8;
-    while (G < 64 && G < E) G *= 2;
+    while (G < 64 && TK_MAXV * G < E) G *= 2;
     if (E > 8 * G) return moe_fail(MOE_ERR_UNSUPPORTED, "route_topk: E=%d too large", E);
     const int tpw = WAVE / G;
     const int waves = ceil_div(T, tpw);
