@@ -229,3 +229,39 @@ def test_capacity_overflow_flag_on_unpack():
     tb, pca = ops.unpack_token_buf(recv, rc, 3, status=status)
     assert int(status.item()) == 0
     assert_bits_equal(tb, O.recv_to_token_buf(to_np(recv), to_np(rc), 3)[0], "token_buf")
+
+
+def test_kernels_reproduce_the_frozen_dispatch_vectors():
+    """The committed vectors of tests/golden (every intermediate of route -> count -> pack -> unpack -> return ->
+    combine on a tiny case) against the kernels, with no oracle call in between."""
+    import os
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "dispatch_small.npz"))
+    W, E, k = 3, 12, 3
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(DEV)  # noqa: E731
+    router, bias = dev(g["router"]), dev(g["bias"])
+    M, CAP = int(g["M"]), int(g["CAP"])
+    for s in range(W):
+        x = dev(g[f"x{s}"])
+        idx, gate, logits = ops.route_topk(x, router, k, bias)
+        assert_bits_equal(logits, g[f"logits{s}"], f"logits of shard {s}")
+        assert_bits_equal(idx, g[f"idx{s}"], f"top-k of shard {s}")
+        np.testing.assert_allclose(to_np(gate), g[f"gate{s}"], rtol=1e-5)
+        c = ops.count_and_offsets(idx, E, W)
+        assert_bits_equal(c.send_counts, g[f"counts{s}"], "send_counts")
+        assert_bits_equal(c.pos, g[f"pos{s}"], "pos")
+        assert_bits_equal(c.row_token, g[f"row_token{s}"], "row_token")
+        if s == 0:
+            assert_bits_equal(ops.pack_tokens(x, idx, c.pos, c.dst_sizes, c.dst_offsets, E // W, M), g["send0"], "send [W,M,H]")
+            assert_bits_equal(ops.pack_fixed_m(x, c.row_token, c.dst_sizes, c.dst_offsets, M), g["send0"], "send [W,M,H]")
+            c0, idx0 = c, idx
+    recv, rc = dev(g["recv"]), dev(g["recv_counts"])
+    tb, pca = ops.unpack_token_buf(recv, rc, CAP)
+    assert_bits_equal(tb, g["token_buf"], "token_buf")
+    assert_bits_equal(pca, g["pca"], "pca")
+    S = int(g["rows"].shape[0])
+    rows, _ = ops.unpack_expert_major(recv, rc, S)
+    assert_bits_equal(rows, g["rows"], "expert-major rows")
+    assert_bits_equal(ops.shuffle_rows(tb, pca, S)[0], g["rows"], "shuffled rows")
+    assert_bits_equal(ops.return_pack(rows * 2.0, rc, M), g["ret"], "return buffer")
+    out = ops.combine(dev(g["send0"]) * 2.0, idx0, c0.pos, dev(g["gate0"]), c0.dst_offsets, E // W)
+    assert_bits_equal(out, g["combined"], "combined output")

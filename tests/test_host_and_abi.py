@@ -111,3 +111,11 @@ def test_gemm_split_plan_covers_every_tile_and_every_k_stage_once():
         lib.moe_gemm_split_plan(total, 256, nk, 256, out)
         assert (out[0], out[1], out[2]) == want
     assert lib.moe_gemm_split_plan(10, 0, 8, 4, out) != 0 and lib.moe_gemm_split_plan(10, 8, 7, 4, out) != 0
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """This build has no collectives: bench.py --gpus 2 must say so and exit non-zero without touching a GPU."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2 and "--gpus must be 1" in r.stderr and r.stdout.strip() == ""

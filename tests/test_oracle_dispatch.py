@@ -181,3 +181,25 @@ def test_combine_closed_forms():
             d = idx[t, kk] // E_l
             acc = acc + gate[t, kk] * send[d, pos[t, kk] - offs[d]]
         assert np.array_equal(O.combine(send, idx, pos, gate, offs, E_l, "bf16")[t], O.bf16_round(acc))
+
+
+def test_oracle_reproduces_the_frozen_dispatch_vectors():
+    """tests/golden/dispatch_small.npz freezes every intermediate of the dispatch path on a tiny seeded case;
+    regenerating it from the oracle must give the same bits (a change of the oracle shows up here first)."""
+    import importlib.util
+    import os
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_fixtures", os.path.join(here, "make_fixtures.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    frozen = np.load(os.path.join(here, "dispatch_small.npz"))
+    fresh = mod.build()
+    assert sorted(frozen.keys()) == sorted(fresh.keys())
+    for k in frozen.keys():
+        a, b = np.asarray(frozen[k]), np.asarray(fresh[k])
+        assert a.dtype == b.dtype and a.shape == b.shape, k
+        assert np.array_equal(a.view(np.uint8) if a.dtype.kind == "f" and a.ndim else a,
+                              b.view(np.uint8) if b.dtype.kind == "f" and b.ndim else b), f"{k} drifted"
+    # a few facts that must hold for the vectors to mean anything
+    assert int(frozen["M"]) == max(int(frozen[f"counts{s}"].sum(1).max()) for s in range(3))
+    assert int(frozen["recv_counts"].sum()) == frozen["rows"].shape[0] and (frozen["pca"] == frozen["recv_counts"].T).all()
