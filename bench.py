@@ -56,8 +56,51 @@ def cpu_baseline(cfg, world_np, budget_tokens: int):
     out = O.combine(ret, idx, pos, gate, offs, E_l, cfg.dtype)
     dt = time.perf_counter() - t0
     assert out.shape == xs.shape and send.shape[1] == M
-    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    return Ts / dt, dt, threads, f"first {Ts} tokens of shard 0 ({rows.shape[0]} routed rows), all stages, numpy/C oracle"
+    return Ts / dt, dt, blas_threads(), f"first {Ts} tokens of shard 0 ({rows.shape[0]} routed rows), all stages, numpy/C oracle"
+
+
+def blas_threads() -> int:
+    """Threads the BLAS behind numpy's matmul actually runs (where the CPU baseline spends its time)."""
+    try:
+        from threadpoolctl import threadpool_info
+        n = [int(p["num_threads"]) for p in threadpool_info() if p.get("user_api") == "blas"]
+        if n:
+            return max(n)
+    except Exception:
+        pass
+    return 1
+
+
+def per_element_loop_baseline():
+    """The reference's own host algorithm, one Python iteration per routed slot (utils.py:213-219), on the
+    CPU-runnable plumbing workload (256 tokens, top-2): timed for the record, one thread."""
+    from iris_testing_amd.configs import CONFIGS, gen_router, gen_shard_tokens
+    from oracle import moe_oracle as O
+    cfg = CONFIGS["plumbing"]
+    x, router = gen_shard_tokens(cfg, 0).numpy(), gen_router(cfg).numpy()
+    t0 = time.perf_counter()
+    idx = O.route(x, router, cfg.topk)[0]
+    payload, counts, offs, sizes = O.bucket_loop_pack(x, idx, cfg.world, cfg.experts)
+    dt = time.perf_counter() - t0
+    assert payload.shape[0] == cfg.tokens * cfg.topk
+    return {"value": round(cfg.tokens / dt, 1), "unit": "tokens/s", "cores": 1, "seconds": round(dt, 4),
+            "sample": "plumbing workload, route + per-slot Python bucket loop + payload (the reference's host routine)"}
+
+
+def profiled_traffic(workload: str, stage: str):
+    """HBM bytes per launch of a stage's kernel as summarised under profiles/ from separate rocprofv3 --pmc runs
+    (FETCH_SIZE, WRITE_SIZE): the line `TRAFFIC_BYTES <stage> <bytes>` of profiles/<workload>_hbm_traffic.txt.
+    (None, None) when no such summary exists: this run itself measures no counters."""
+    path = os.path.join(ROOT, "profiles", f"{workload}_hbm_traffic.txt")
+    try:
+        with open(path) as f:
+            for line in f:
+                p = line.split()
+                if len(p) >= 3 and p[0] == "TRAFFIC_BYTES" and p[1] == stage:
+                    return float(p[2]), f"profiles/{workload}_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, separate runs)"
+    except OSError:
+        pass
+    return None, None
 
 
 def main():
@@ -162,10 +205,8 @@ def main():
             unit = "TFLOP/s"
         stages[n] = {"ms": round(ms, 4), "ms_min": round(stage_spread[n][0], 4), "ms_median": round(stage_spread[n][1], 4),
                      "bound": wk["bound"], "achieved": round(ach, 2), "peak": peak, "unit": unit, "frac": round(ach / peak, 4)}
-    # HBM traffic per launch of the dominant kernel, from the FETCH_SIZE / WRITE_SIZE runs summarised in
-    # profiles/mixtral_hbm_traffic.txt (bytes; only measured for the default workload)
-    measured_traffic = {"mixtral": 12.52e9}
     dom = "mlp_up"  # the gate/up grouped GEMM: most of the flops of a step
+    traffic, traffic_source = profiled_traffic(cfg.name, dom)
     if cfg.quant == "fp8":
         kname = "moe_grouped_mlp_fp8 (row quantisation + gate/up GEMM + SwiGLU + re-quantisation + down GEMM)"
     elif cfg.dtype == "f32":
@@ -174,8 +215,8 @@ def main():
         kname = "grouped_gemm_kernel (gate/up + SwiGLU epilogue)" if cfg.act == "swiglu" else "grouped_gemm_kernel (up + activation)"
     roofline = {"kernel": kname,
                 "bound": "mfma", "achieved": stages[dom]["achieved"], "peak": stages[dom]["peak"], "unit": "TFLOP/s",
-                "frac": stages[dom]["frac"], "traffic": measured_traffic.get(cfg.name), "avg_launch_ms": stages[dom]["ms"],
-                "flops_per_launch": work[dom]["amount"]}
+                "frac": stages[dom]["frac"], "traffic": traffic, "traffic_source": traffic_source,
+                "avg_launch_ms": stages[dom]["ms"], "flops_per_launch": work[dom]["amount"]}
 
     out = {
         "metric": "routed tokens/sec (dispatch+expert+combine) at 1 MI355X",
@@ -215,7 +256,8 @@ def main():
         sample = args.cpu_sample_tokens or max(64, min(cfg.tokens, int(1.2e13 / flops_per_token)))
         v, secs, threads, desc = cpu_baseline(cfg, (x_np, router_np, bias_np, w_np), sample)
         out["cpu_baseline"] = {"value": round(v, 1), "unit": "tokens/s", "cores": threads, "kind": "port",
-                               "sample": desc, "seconds": round(secs, 2)}
+                               "sample": desc, "seconds": round(secs, 2), "host_cpus": os.cpu_count(),
+                               "per_element_loop_config1": per_element_loop_baseline()}
     print(json.dumps(out), flush=True)
 
 

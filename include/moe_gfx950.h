@@ -105,7 +105,8 @@ int moe_pack_tokens(const void* x, int dtype, int T, int H, const int32_t* topk_
  * recv [W,M,H]: slot s holds what source s sent to this rank ((el, token) order, zero padded);
  * recv_counts [W,E_l]: recv_counts[s,e] rows from source s for local expert e.
  * token_buf[e,s,j,:] = recv[s, expert_offs_s[e]+j, :] for j < recv_counts[s,e], else zeros;
- * pca[e,s] = recv_counts[s,e].  status (nullable): 1 on count > CAP.
+ * pca[e,s] = recv_counts[s,e].  status (nullable): 1 on count > CAP, or when a counted row lies at or
+ * past row M of its slot (the sender's pack dropped it: it reads as zeros).
  * map_ws (here and in every entry point below that takes one): int32 scratch of
  * moe_recv_map_ints(W, E_l, n_out) elements (prefix tables over the counts; n_out = rows of the
  * output buffer, which no longer enters the size). */
@@ -128,7 +129,8 @@ int moe_reorder_flat_to_token_buf(const void* flat, int dtype, int R, int H, con
 int moe_shuffle(const void* token_buf, int dtype, int E_l, int W, int CAP, int H, const int32_t* pca,
                 void* shuffled, int S_rows, int32_t* expert_cnt, int32_t* map_ws, moe_stream_t stream);
 
-/* recv [W,M,H] -> shuffled [S_rows,H] directly (token_buf never materialised). */
+/* recv [W,M,H] -> shuffled [S_rows,H] directly (token_buf never materialised).  A counted row that lies at
+ * or past row M of its slot was dropped by the sender's pack and reads as zeros. */
 int moe_unpack_expert_major(const void* recv, int dtype, int W, int M, int H, const int32_t* recv_counts,
                             int E_l, void* shuffled, int S_rows, int32_t* expert_cnt, int32_t* map_ws,
                             moe_stream_t stream);
@@ -185,13 +187,15 @@ int moe_grouped_mlp_fp8(const void* tokens_bf16, const int32_t* expert_cnt, int 
  * can read its input rows where the transfer left them and write its result rows where the way back
  * wants them.  Three entry points make that path:
  *   moe_recv_row_map        row_map[r] = row of the [W,M,H] receive buffer that holds expert-major row r
- *                           (r < n_rows; rows past the received total map to row 0), expert_cnt (nullable)
+ *                           (r < n_rows; rows past the received total map to row 0; rows dropped by the
+ *                           sender's pack, at or past row M of their slot, map to -1), expert_cnt (nullable)
  *                           as in moe_unpack_expert_major; map_ws >= moe_recv_map_ints(W,E_l,n_rows) ints.
  *                           The same map is the destination of result row r in the returned buffer.
  *   moe_grouped_gemm_mapped moe_grouped_gemm_packed with row indirection: logical row r is read from row
  *                           a_row_map[r] of a_base (a_rows rows of K, under 4 GiB) and written to row
  *                           c_row_map[r] of out (out_rows rows of N); either map may be NULL (identity).
- *                           Map entries must lie inside their buffers.  part_ws (nullable, part_ws_bytes
+ *                           Map entries must lie inside their buffers or be negative: a negative a_row_map
+ *                           entry reads row 0, a negative c_row_map entry stores nothing.  part_ws (nullable, part_ws_bytes
  *                           bytes, moe_gemm_part_workspace_bytes() for the full benefit): scratch for fp32
  *                           partial sums; with it, when the last round of the persistent grid holds at most
  *                           a quarter of a grid of tiles, those tiles are cut along K over the idle compute
@@ -234,10 +238,12 @@ int moe_return_pack(const void* y, int dtype, int S_rows, int H, const int32_t* 
                     int M, void* ret, int32_t* map_ws, moe_stream_t stream);
 
 /* out[t,:] = sum_kk gate[t,kk] * ret[dst, pos[t,kk]-dst_offsets[dst], :], dst = idx[t,kk]/E_l;
- * fp32 multiply then add in ascending kk (no fma), one rounding to `dtype`. */
+ * fp32 multiply then add in ascending kk (no fma), one rounding to `dtype`.  A slot whose dst lies
+ * outside [0,W) or whose row lies outside [0,M) -- a row the pack dropped because the pair capacity
+ * was exceeded -- has no returned row: it is skipped and *status (nullable) is set to 1. */
 int moe_combine(const void* ret, int dtype, int W, int M, int H, const int32_t* topk_idx, const int32_t* pos,
                 const float* gate, const int32_t* dst_offsets, int T, int k, int E_l, void* out,
-                moe_stream_t stream);
+                int32_t* status, moe_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -317,7 +317,14 @@ __device__ __forceinline__ int source_row(const RowSource& a, int r) {
             if (r >= a.row_off[n]) return -1;
             const int seg = wave_seg(a.row_off, n + 1, r);  // seg = e*W + s
             const int e = seg / a.W, s = seg % a.W, j = r - a.row_off[seg];
-            return a.mode == SRC_UNPACK ? s * a.M + a.src_off[s * a.E_l + e] + j : (e * a.W + s) * a.CAP + j;
+            if (a.mode == SRC_SHUFFLE) return (e * a.W + s) * a.CAP + j;
+            // a row past the pair capacity never reached the slot (the pack dropped it): it reads as zeros
+            const int m = a.src_off[s * a.E_l + e] + j;
+            if (m >= a.M) {
+                if (a.status && lane_id() == 0) *a.status = 1;
+                return -1;
+            }
+            return s * a.M + m;
         }
         case SRC_TOKBUF:
         case SRC_REORDER: {
@@ -325,7 +332,13 @@ __device__ __forceinline__ int source_row(const RowSource& a, int r) {
             const int c = a.rc[s * a.E_l + e];
             if (j == 0 && c > a.CAP && a.status && lane_id() == 0) *a.status = 1;
             if (j >= c) return -1;
-            return a.mode == SRC_TOKBUF ? s * a.M + a.src_off[s * a.E_l + e] + j : a.flat_off[s * a.E_l + e] + j;
+            if (a.mode == SRC_REORDER) return a.flat_off[s * a.E_l + e] + j;
+            const int m = a.src_off[s * a.E_l + e] + j;  // row inside the sender's slot; past M it was dropped by the pack
+            if (m >= a.M) {
+                if (a.status && lane_id() == 0) *a.status = 1;
+                return -1;
+            }
+            return s * a.M + m;
         }
         case SRC_UNSHUFFLE: {
             const int j = r % a.CAP, s = (r / a.CAP) % a.W, e = r / (a.CAP * a.W);
@@ -463,20 +476,29 @@ template <typename XT, int KT, int WPB>
 __global__ __launch_bounds__(WPB * WAVE) void combine_kernel(const uint4* __restrict__ ret, const int32_t* __restrict__ idx,
                                                               const int32_t* __restrict__ pos, const float* __restrict__ gate,
                                                               const int32_t* __restrict__ dst_offsets, int T, int k_rt, int E_l,
-                                                              int M, int row_vec, uint4* __restrict__ out) {
+                                                              int W, int M, int row_vec, uint4* __restrict__ out,
+                                                              int32_t* __restrict__ status) {
     constexpr int N = Vec16<XT>::N;
     constexpr int KMAX = KT ? KT : MOE_MAX_TOPK;
     const int k = KT ? KT : k_rt;
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     for (int t = blockIdx.x * WPB + wave; t < T; t += gridDim.x * WPB) {
+        // a slot whose destination or row lies outside the [W,M] layout was dropped by the pack (pair capacity
+        // exceeded) and has no returned row: it is skipped, like the pack skipped it, and the status word is raised
         size_t rows[KMAX];
         float g[KMAX];
+        bool have[KMAX];
 #pragma unroll
         for (int j = 0; j < KMAX; ++j) {
+            have[j] = false;
             if (j < k) {
                 const int d = idx[(size_t)t * k + j] / E_l;
-                rows[j] = ((size_t)d * M + (pos[(size_t)t * k + j] - dst_offsets[d])) * row_vec;
+                const bool d_ok = (unsigned)d < (unsigned)W;
+                const int m = pos[(size_t)t * k + j] - dst_offsets[d_ok ? d : 0];
+                have[j] = d_ok && (unsigned)m < (unsigned)M;
+                rows[j] = have[j] ? ((size_t)d * M + m) * row_vec : 0;
                 g[j] = gate[(size_t)t * k + j];
+                if (!have[j] && status && lane == 0) *status = 1;
             }
         }
 #pragma unroll 2
@@ -484,7 +506,7 @@ __global__ __launch_bounds__(WPB * WAVE) void combine_kernel(const uint4* __rest
             uint4 v[KMAX];
 #pragma unroll
             for (int j = 0; j < KMAX; ++j)
-                if (j < k) {
+                if (j < k && have[j]) {
                     // every returned row is read once: no cache retention wanted
                     const u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(ret + rows[j] + c));
                     v[j] = make_uint4(raw.x, raw.y, raw.z, raw.w);
@@ -494,7 +516,7 @@ __global__ __launch_bounds__(WPB * WAVE) void combine_kernel(const uint4* __rest
             for (int i = 0; i < N; ++i) acc[i] = 0.f;
 #pragma unroll
             for (int j = 0; j < KMAX; ++j) {
-                if (j < k) {
+                if (j < k && have[j]) {
                     float f[N];
                     Vec16<XT>::unpack(v[j], f);
 #pragma unroll
@@ -510,10 +532,10 @@ __global__ __launch_bounds__(WPB * WAVE) void combine_kernel(const uint4* __rest
 
 template <typename XT>
 int launch_combine(const void* ret, const int32_t* idx, const int32_t* pos, const float* gate, const int32_t* dst_offsets, int T,
-                   int k, int E_l, int M, int row_vec, void* out, hipStream_t s) {
+                   int k, int E_l, int W, int M, int row_vec, void* out, int32_t* status, hipStream_t s) {
     const int blocks = min(ceil_div(T, 4), 65535 * 8);
 #define MOE_COMBINE(KT) \
-    combine_kernel<XT, KT, 4><<<blocks, 4 * WAVE, 0, s>>>((const uint4*)ret, idx, pos, gate, dst_offsets, T, k, E_l, M, row_vec, (uint4*)out)
+    combine_kernel<XT, KT, 4><<<blocks, 4 * WAVE, 0, s>>>((const uint4*)ret, idx, pos, gate, dst_offsets, T, k, E_l, W, M, row_vec, (uint4*)out, status)
     switch (k) {
         case 1: MOE_COMBINE(1); break;
         case 2: MOE_COMBINE(2); break;
@@ -534,7 +556,9 @@ int gather_rows(const void* src, void* dst, const RowSource& a, int n_rows, int 
 
 // Expert-major row r of the receive side -> row of the [W,M,H] buffer that holds it (one thread per row,
 // binary search in the (expert, source)-major prefix).  The same index serves the way back: the result
-// row of r returns to the slot its input came from.  Rows past the received total map to row 0.
+// row of r returns to the slot its input came from.  Rows past the received total map to row 0; rows the pack
+// dropped (position in the sender's slot at or past the pair capacity M) map to -1: the GEMMs read row 0 for them
+// and store nothing.
 __global__ __launch_bounds__(256) void row_map_kernel(const int32_t* __restrict__ row_off, const int32_t* __restrict__ src_off,
                                                        int W, int E_l, int M, int n_rows, int32_t* __restrict__ map) {
     const int r = blockIdx.x * blockDim.x + threadIdx.x;
@@ -548,7 +572,7 @@ __global__ __launch_bounds__(256) void row_map_kernel(const int32_t* __restrict_
     }
     const int e = lo / W, s = lo % W;
     const int m = src_off[s * E_l + e] + (r - row_off[lo]);
-    map[r] = s * M + min(m, M - 1);
+    map[r] = m < M ? s * M + m : -1;
 }
 
 // rows [size_s, M) of every slot s of a [W,M,row] buffer <- 0, size_s = sum over e of rc[s,e] (one wave per row)
@@ -807,7 +831,7 @@ extern "C" int moe_return_pack(const void* y, int dtype, int S_rows, int H, cons
 
 extern "C" int moe_combine(const void* ret, int dtype, int W, int M, int H, const int32_t* topk_idx, const int32_t* pos,
                            const float* gate, const int32_t* dst_offsets, int T, int k, int E_l, void* out,
-                           moe_stream_t stream) {
+                           int32_t* status, moe_stream_t stream) {
     hipStream_t s = (hipStream_t)stream;
     int rc = check_rows("combine", dtype, H);
     if (rc) return rc;
@@ -816,6 +840,6 @@ extern "C" int moe_combine(const void* ret, int dtype, int W, int M, int H, cons
     if (T == 0) return MOE_OK;
     MOE_REQUIRE(ret && topk_idx && pos && gate && dst_offsets && out, MOE_ERR_INVALID, "combine: null pointer");
     const int row_vec = H * dtype_size(dtype) / 16;
-    if (dtype == MOE_F32) return launch_combine<float>(ret, topk_idx, pos, gate, dst_offsets, T, k, E_l, M, row_vec, out, s);
-    return launch_combine<bf16_t>(ret, topk_idx, pos, gate, dst_offsets, T, k, E_l, M, row_vec, out, s);
+    if (dtype == MOE_F32) return launch_combine<float>(ret, topk_idx, pos, gate, dst_offsets, T, k, E_l, W, M, row_vec, out, status, s);
+    return launch_combine<bf16_t>(ret, topk_idx, pos, gate, dst_offsets, T, k, E_l, W, M, row_vec, out, status, s);
 }

@@ -302,7 +302,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     uint32_t aoff_[RA];                                                                                     \
     _Pragma("unroll") for (int r = 0; r < RA; ++r) {                                                         \
         const int lr_ = max(min(r * LR + lrow, (t).rv - 1), 0);  /* tile row this lane fetches, clamped */     \
-        aoff_[r] = (uint32_t)(p.a_map ? p.a_map[(t).row0 + lr_] : lr_) * ldk + lchunk * 16;                   \
+        aoff_[r] = (uint32_t)(p.a_map ? max(p.a_map[(t).row0 + lr_], 0) : lr_) * ldk + lchunk * 16;           \
     }
     // load d (0 .. LPS-1) of one stage: A rounds first, then B rounds
 #define GG_LD(d, ap_, bp_, aoff_, slot)                                                                       \
@@ -513,7 +513,9 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             const size_t grow = (size_t)(row0 + (ok[i] ? r : 0));
             rs[i] = 1.f;
             if constexpr (FP8) rs[i] = p.row_scale[grow];
-            crow[i] = C + (p.c_map ? (size_t)p.c_map[grow] : grow) * p.ldc;
+            const int crow_i = p.c_map ? p.c_map[grow] : 0;
+            ok[i] = ok[i] && crow_i >= 0;  // a negative map entry: the row has no place in the output
+            crow[i] = C + (p.c_map ? (size_t)max(crow_i, 0) : grow) * p.ldc;
         }
         float4 sc0[NQ], sc1[NQ];  // fp8: channel scales of the lane's columns (gate / only; up)
 #pragma unroll
@@ -673,11 +675,12 @@ __global__ __launch_bounds__(256) void gg_reduce_parts_kernel(const GemmParams p
                 x[e] = v;
             }
         }
-        if (col < p.N) {
+        const int crow = p.c_map ? p.c_map[grow] : 0;
+        if (col < p.N && crow >= 0) {
             uint2 o;
             o.x = gg_pack_bf16(x[0], x[1]);
             o.y = gg_pack_bf16(x[2], x[3]);
-            *(uint2*)(C + (p.c_map ? (size_t)p.c_map[grow] : grow) * p.ldc + col) = o;
+            *(uint2*)(C + (p.c_map ? (size_t)crow : grow) * p.ldc + col) = o;
         }
     }
 }
@@ -865,7 +868,7 @@ __global__ __launch_bounds__(256) void quantize_rows_fp8_kernel(const bf16_t* __
     const int limit = n_rows_dev ? min(rows, *n_rows_dev) : rows;
     const int nv = cols / 8;
     for (int r = blockIdx.x * 4 + wave; r < limit; r += gridDim.x * 4) {
-        const uint4* src = (const uint4*)(x + (size_t)(src_map ? src_map[r] : r) * cols);
+        const uint4* src = (const uint4*)(x + (size_t)(src_map ? max(src_map[r], 0) : r) * cols);
         uint4 held[NV > 0 ? NV : 1];
         float amax = 0.f;
         if constexpr (NV > 0) {

@@ -12,6 +12,46 @@ from .. import ops
 from ..utils import _assert_cuda_int32
 
 
+# Re-tiled copies of weight tensors the operator has seen, keyed on the tensor's storage and version counter, so that
+# a weight that did not change between calls is re-tiled once, not on every forward (the re-tiling reads and writes the
+# whole tensor).  Entries die with their tensors (weak references); an in-place update bumps the version and re-tiles.
+_PACKED = {}
+_PART_WS = {}
+
+
+def _packed_weights(w: torch.Tensor) -> torch.Tensor:
+    import weakref
+    key = (w.data_ptr(), w._version, tuple(w.shape), w.dtype, w.device)
+    hit = _PACKED.get(key)
+    if hit is not None and hit[0]() is w:
+        return hit[1]
+    for k in [k for k, v in _PACKED.items() if v[0]() is None or (v[0]() is w and k != key)]:
+        del _PACKED[k]
+    packed = ops.prepack_weights(w)
+    _PACKED[key] = (weakref.ref(w), packed)
+    return packed
+
+
+def _part_ws(device) -> torch.Tensor:
+    """One partial-sum workspace per device for the K split of an under-filled last round of GEMM tiles."""
+    ws = _PART_WS.get(device)
+    if ws is None:
+        ws = _PART_WS[device] = ops.gemm_part_workspace(device)
+    return ws
+
+
+def _grouped_gemm(tokens: torch.Tensor, weights: torch.Tensor, cnt: torch.Tensor) -> torch.Tensor:
+    """out[rows of g] = tokens[rows of g] @ weights[g]; rows past sum(cnt) are zero."""
+    if tokens.dtype != torch.bfloat16 or weights.shape[1] % 64 or weights.shape[2] % 8:
+        return ops.grouped_gemm(tokens, weights, cnt)
+    S, N = tokens.shape[0], weights.shape[2]
+    out = torch.zeros((S, N), dtype=tokens.dtype, device=tokens.device)
+    if S:
+        ops.grouped_gemm_mapped(tokens, None, _packed_weights(weights), cnt, S, N, "none", out,
+                                part_ws=_part_ws(tokens.device))
+    return out
+
+
 class Expert(torch.autograd.Function):
 
     @staticmethod
@@ -22,7 +62,7 @@ class Expert(torch.autograd.Function):
         _assert_cuda_int32(local_expert_cnt, "local_expert_cnt")
         assert weights.shape[0] == local_expert_cnt.numel(), "one row count per local expert"
         ctx.save_for_backward(tokens, weights, local_expert_cnt)
-        return ops.grouped_gemm(tokens.contiguous(), weights.contiguous(), local_expert_cnt.contiguous())
+        return _grouped_gemm(tokens.contiguous(), weights.contiguous(), local_expert_cnt.contiguous())
 
     @staticmethod
     def backward(ctx, do):

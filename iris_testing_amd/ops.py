@@ -414,7 +414,10 @@ def zero_padding_rows(buf: torch.Tensor, recv_counts: torch.Tensor) -> torch.Ten
 
 
 def combine(ret: torch.Tensor, topk_idx: torch.Tensor, pos: torch.Tensor, gate: torch.Tensor,
-            dst_offsets: torch.Tensor, e_local: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+            dst_offsets: torch.Tensor, e_local: int, out: Optional[torch.Tensor] = None,
+            status: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = sum_kk gate[t,kk] * ret[slot of (t,kk)].  Slots the pack dropped (row at or past M) are skipped
+    and raise ``status`` (int32 [1], optional)."""
     _req_cuda(ret, "ret")
     _req_i32(topk_idx, "topk_idx")
     _req_i32(pos, "pos")
@@ -426,7 +429,7 @@ def combine(ret: torch.Tensor, topk_idx: torch.Tensor, pos: torch.Tensor, gate: 
     if out is None:
         out = torch.empty((T, H), dtype=ret.dtype, device=ret.device)
     L.check(L.lib().moe_combine(L.ptr(ret), L.dtype_code(ret.dtype), W, M, H, L.ptr(topk_idx), L.ptr(pos), L.ptr(gate),
-                                L.ptr(dst_offsets), T, k, e_local, L.ptr(out), L.stream_ptr()))
+                                L.ptr(dst_offsets), T, k, e_local, L.ptr(out), L.ptr(status), L.stream_ptr()))
     return out
 
 

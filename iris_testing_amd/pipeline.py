@@ -162,7 +162,7 @@ class DispatchPipeline:
         c, w = self.cfg, self.world
         L.check(L.lib().moe_combine(self._p(self.returned), self.code, c.world, w.M, c.hidden, self._p(self.idx),
                                     self._p(self.pos), self._p(self.gate), self._p(self.dst_offsets), c.tokens, c.topk,
-                                    c.e_local, self._p(self.out), s))
+                                    c.e_local, self._p(self.out), self._p(self.status), s))
 
     def step(self, events: Optional[List[Dict[str, tuple]]] = None):
         """One pass of the hot path.  With ``events`` (a list), per-stage (start, end) torch.cuda.Event

@@ -298,6 +298,34 @@ def send_payload(x: np.ndarray, row_token: np.ndarray) -> np.ndarray:
     return x[row_token.astype(np.int64)]
 
 
+def bucket_loop_pack(x: np.ndarray, top_idxs: np.ndarray, world_size: int, num_experts_total: int):
+    """The reference's host algorithm as it is written, one Python iteration per routed slot (utils.py:204-246):
+    append each token row to bucket[dst][el] in (token, slot) order, then concatenate the buckets in (dst, el)
+    order.  Returns (send_payload, send_counts, dst_offsets, dst_sizes).  Slow by construction; the vectorised
+    functions above are held to it in the tests, and the benchmark times it on the smallest workload."""
+    e_local = num_experts_total // world_size
+    buckets = [[[] for _ in range(e_local)] for _ in range(world_size)]
+    for ti in range(x.shape[0]):
+        for kk in range(top_idxs.shape[1]):
+            ex = int(top_idxs[ti, kk])
+            dst = ex // e_local
+            buckets[dst][ex - dst * e_local].append(x[ti])
+    counts = np.zeros((world_size, e_local), np.int32)
+    offs, sizes = np.zeros(world_size, np.int32), np.zeros(world_size, np.int32)
+    chunks, running = [], 0
+    for dst in range(world_size):
+        offs[dst] = running
+        for el in range(e_local):
+            n = len(buckets[dst][el])
+            counts[dst, el] = n
+            if n:
+                chunks.append(np.stack(buckets[dst][el]))
+            sizes[dst] += n
+        running += int(sizes[dst])
+    payload = np.concatenate(chunks) if running else np.empty((0, x.shape[1]), x.dtype)
+    return payload, counts, offs, sizes
+
+
 def route_and_pack_padding_free(x, w, topk, world_size, num_experts_total, bias=None):
     """The reference's host routine end to end (utils.py:176-246).
 
@@ -330,15 +358,20 @@ def pair_capacity(dst_sizes_all: np.ndarray) -> int:
 # --------------------------------------------------------------------------------------
 # a8: fixed [W, M, H] send layout  (reference README.md:5-7)
 # --------------------------------------------------------------------------------------
-def pack_fixed_m(payload: np.ndarray, dst_offsets: np.ndarray, dst_sizes: np.ndarray, M: int) -> np.ndarray:
-    """send[dst, m, :] = payload[dst_offsets[dst] + m] for m < dst_sizes[dst], else zeros."""
+def pack_fixed_m(payload: np.ndarray, dst_offsets: np.ndarray, dst_sizes: np.ndarray, M: int,
+                 drop: bool = False) -> np.ndarray:
+    """send[dst, m, :] = payload[dst_offsets[dst] + m] for m < dst_sizes[dst], else zeros.
+
+    A destination with more than M rows is an error, unless ``drop``: then its rows at and past M are
+    dropped (the capacity-overflow behaviour of the kernels, which also raise a status word; the reference
+    skips the whole exchange instead, benchmark.py:137-142)."""
     W = len(dst_sizes)
     H = payload.shape[1]
-    if int(np.max(dst_sizes, initial=0)) > M:
+    if int(np.max(dst_sizes, initial=0)) > M and not drop:
         raise ValueError(f"pair capacity M={M} < max dst size {int(np.max(dst_sizes))}")
     out = np.zeros((W, M, H), dtype=payload.dtype)
     for d in range(W):
-        n = int(dst_sizes[d])
+        n = min(int(dst_sizes[d]), M)
         o = int(dst_offsets[d])
         out[d, :n] = payload[o:o + n]
     return out
@@ -389,6 +422,7 @@ def recv_to_token_buf(recv: np.ndarray, recv_counts: np.ndarray, capacity: int) 
         for e in range(e_local):
             c = int(recv_counts[s, e])
             o = int(offs[s, e])
+            c = max(min(c, M - o), 0)  # rows at or past M never reached the slot (dropped by the sender's pack): zeros
             tb[e, s, :c] = recv[s, o:o + c]
     return tb, np.ascontiguousarray(recv_counts.T).astype(np.int32)
 
@@ -422,7 +456,10 @@ def unpack_expert_major(recv: np.ndarray, recv_counts: np.ndarray) -> np.ndarray
         for s in range(W):
             c = int(recv_counts[s, e])
             o = int(offs[s, e])
-            parts.append(recv[s, o:o + c])
+            have = max(min(c, M - o), 0)  # counted rows at or past M were dropped by the sender's pack: zero rows
+            parts.append(recv[s, o:o + have])
+            if have < c:
+                parts.append(np.zeros((c - have, H), dtype=recv.dtype))
     return np.concatenate(parts, axis=0) if parts else np.zeros((0, H), dtype=recv.dtype)
 
 
@@ -568,7 +605,8 @@ def return_pack(y: np.ndarray, recv_counts: np.ndarray, M: int) -> np.ndarray:
         for s in range(W):
             c = int(recv_counts[s, e])
             o = int(offs[s, e])
-            ret[s, o:o + c] = y[r:r + c]
+            have = max(min(c, M - o), 0)  # rows at or past M have no slot on the way back
+            ret[s, o:o + have] = y[r:r + have]
             r += c
     return ret
 
@@ -579,14 +617,18 @@ def combine(ret: np.ndarray, idx: np.ndarray, pos: np.ndarray, gate: np.ndarray,
 
     ret [W,M,H] is the returned buffer in the same slots the send buffer used.  fp32
     accumulate in ascending kk, one fp32 multiply and one fp32 add per term (no fused
-    multiply-add), then one rounding to ``dtype``.
+    multiply-add), then one rounding to ``dtype``.  A slot whose row lies outside [0, M) (dropped by a pack
+    that ran over the pair capacity) or whose dst lies outside [0, W) has no returned row and is skipped.
     """
     T, k = idx.shape
     W, M, H = ret.shape
     out = np.zeros((T, H), dtype=np.float32)
     for kk in range(k):
         d = (idx[:, kk] // e_local).astype(np.int64)
-        m = pos[:, kk].astype(np.int64) - dst_offsets.astype(np.int64)[d]
-        rows = ret[d, m].astype(np.float32)
-        out = (out + (gate[:, kk:kk + 1].astype(np.float32) * rows).astype(np.float32)).astype(np.float32)
+        d_ok = (d >= 0) & (d < W)
+        m = pos[:, kk].astype(np.int64) - dst_offsets.astype(np.int64)[np.where(d_ok, d, 0)]
+        have = d_ok & (m >= 0) & (m < M)
+        rows = ret[np.where(have, d, 0), np.where(have, m, 0)].astype(np.float32)
+        term = (out + (gate[:, kk:kk + 1].astype(np.float32) * rows).astype(np.float32)).astype(np.float32)
+        out = np.where(have[:, None], term, out)
     return round_to(out, dtype)

@@ -123,6 +123,31 @@ def test_expert_layer_signature():
     np.testing.assert_allclose(to_np(out), want, rtol=1e-4, atol=1e-4)
 
 
+def test_expert_layer_bf16_reuses_retiled_weights_until_they_change():
+    """bf16 weights are re-tiled once per tensor version: a second call gives the same bits, an in-place update of
+    the weights is seen by the next call, and the result is the oracle's."""
+    from iris_testing_amd.layers import expert as expert_mod
+    rng = np.random.default_rng(2)
+    cnt = np.array([300, 0, 45, 130], dtype=np.int32)
+    S = int(cnt.sum())
+    x = O.bf16_round(rng.standard_normal((S + 2, 256)).astype(np.float32))
+    w = O.bf16_round((rng.standard_normal((4, 256, 192)) / 16).astype(np.float32))
+    xt, wt = torch.from_numpy(x).bfloat16().to(DEV), torch.from_numpy(w).bfloat16().to(DEV)
+    ct = torch.from_numpy(cnt).to(DEV)
+    out1 = expert(xt, wt, ct, 4)
+    n_cached = len(expert_mod._PACKED)
+    out2 = expert(xt, wt, ct, 4)
+    assert len(expert_mod._PACKED) == n_cached and torch.equal(out1, out2)
+    want = O.grouped_gemm(x[:S], w, cnt, "bf16")
+    got = to_np(out1)
+    rms = float(np.sqrt((want.astype(np.float64) ** 2).mean()))
+    assert (np.abs(got[:S] - want) <= 2.0 ** -7 * np.abs(want) + 2.0 ** -7 * rms).all()
+    assert (got[S:] == 0).all()
+    wt.mul_(2.0)  # exact in bf16: the product doubles exactly
+    out3 = expert(xt, wt, ct, 4)
+    assert torch.equal(out3, out1 * 2), "an in-place weight update must reach the kernel"
+
+
 def test_benchmark_driver_point_and_overflow_report(capsys):
     """The environment-variable driver (the reference's benchmark.py knobs): one point with a CAPACITY smaller
     than the largest per-expert count prints the skip notice, still times, and its correctness report (fixed-M

@@ -164,6 +164,90 @@ def test_zero_tokens_and_overflow_flag():
     assert torch.equal(guard[:cfg.world * M], kept), "token-major pack drops the same rows as the slot-major one"
 
 
+def test_overflowed_pack_drops_rows_consistently_down_the_path():
+    """M below the largest pair size: the pack raises the status word and drops the rows at and past M; every
+    later stage must treat exactly those rows as absent (zero rows on the receive side, no slot on the way back,
+    no contribution to the combine) and stay inside its buffers.  Bit-exact against the oracle's drop semantics;
+    the copy-free destination side (row map with -1 entries, gathering / scattering GEMM) against the copies."""
+    cfg = _cfg("zipf_k4", 512)
+    W, E, E_l, k, H = cfg.world, cfg.experts, cfg.e_local, cfg.topk, cfg.hidden
+    w = gen_router(cfg)
+    b = gen_router_bias(cfg)
+    xs = [gen_shard_tokens(cfg, s) for s in range(W)]
+    xn = [to_np(x) for x in xs]
+    shards, M_full, CAP = oracle_world(cfg, xn, to_np(w), to_np(b))
+    M = M_full - 37
+    assert all(int(sh["sizes"][0]) > M for sh in shards)  # every source overflows its slot on rank 0
+    # source side of shard 0: both packs drop the same rows and raise the flag
+    s0 = shards[0]
+    x0 = xs[0].to(DEV)
+    idx0, pos0 = torch.from_numpy(s0["idx"]).to(DEV), torch.from_numpy(s0["pos"]).to(DEV)
+    sizes0, offs0 = torch.from_numpy(s0["sizes"]).to(DEV), torch.from_numpy(s0["offs"]).to(DEV)
+    o_send0 = O.pack_fixed_m(O.send_payload(xn[0], s0["row_token"]), s0["offs"], s0["sizes"], M, drop=True)
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    send = ops.pack_tokens(x0, idx0, pos0, sizes0, offs0, E_l, M, status=status)
+    assert int(status.item()) == 1
+    assert_bits_equal(send, o_send0, "token-major pack with dropped rows")
+    send2 = ops.pack_fixed_m(x0, torch.from_numpy(s0["row_token"]).to(DEV), sizes0, offs0, M)
+    assert_bits_equal(send2, o_send0, "slot-major pack with dropped rows")
+    # destination side of rank 0
+    o_recv = np.stack([O.pack_fixed_m(O.send_payload(x, sh["row_token"]), sh["offs"], sh["sizes"], M, drop=True)[0]
+                       for x, sh in zip(xn, shards)])
+    o_rc = np.stack([sh["counts"][0] for sh in shards]).astype(np.int32)
+    recv = torch.from_numpy(o_recv).to(cfg.torch_dtype).to(DEV)
+    rc = torch.from_numpy(o_rc).to(DEV)
+    S = int(o_rc.sum())
+    o_rows = O.unpack_expert_major(o_recv, o_rc)
+    n_dropped = int((np.abs(o_rows).sum(1) == 0).sum())
+    assert n_dropped > 0
+    rows, cnt = ops.unpack_expert_major(recv, rc, S)
+    assert_bits_equal(rows, o_rows, "expert-major rows (dropped rows read as zeros)")
+    status.zero_()
+    tb, pca = ops.unpack_token_buf(recv, rc, CAP, status=status)
+    assert int(status.item()) == 1
+    assert_bits_equal(tb, O.recv_to_token_buf(o_recv, o_rc, CAP)[0], "token_buf")
+    y = (rows * 2).contiguous()
+    guard = torch.full((W * M + 8, H), 3.0, dtype=rows.dtype, device=DEV)
+    ret = ops.return_pack(y, rc, M, out=guard[:W * M].view(W, M, H))
+    assert_bits_equal(ret, O.return_pack(o_rows * 2, o_rc, M), "return buffer")
+    assert (guard[W * M:] == 3.0).all()
+    # the copy-free destination side: dropped rows carry -1 in the row map, read row 0 and store nothing
+    row_map, cnt2 = ops.recv_row_map(rc, M, S)
+    assert torch.equal(cnt, cnt2)
+    rm = to_np(row_map)
+    assert int((rm < 0).sum()) == n_dropped and rm.max() < W * M
+    keep = rm >= 0
+    assert_bits_equal(recv.view(W * M, H)[torch.from_numpy(rm[keep]).long().to(DEV)], o_rows[keep], "rows picked by the row map")
+    rng = np.random.default_rng(5)
+    N = 256
+    wt = torch.from_numpy(O.bf16_round((rng.standard_normal((E_l, H, N)) * H ** -0.5).astype(np.float32))).to(torch.bfloat16).to(DEV)
+    packed = ops.prepack_weights(wt)
+    plain = torch.zeros((S, N), dtype=torch.bfloat16, device=DEV)
+    ops.grouped_gemm_mapped(rows, None, packed, cnt, S, N, "none", plain)
+    want = torch.full((W * M + 8, N), 3.0, dtype=torch.bfloat16, device=DEV)
+    want[:W * M] = ops.return_pack(plain, rc, M).view(W * M, N)
+    got = torch.full((W * M + 8, N), 3.0, dtype=torch.bfloat16, device=DEV)
+    ops.grouped_gemm_mapped(recv.view(W * M, H), row_map, packed, cnt, S, N, "none", got, c_row_map=row_map)
+    ops.zero_padding_rows(got[:W * M].view(W, M, N), rc)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16)), "gathering / scattering GEMM with dropped rows"
+    # combine on shard 0: returned = 2 * what was sent; dropped slots contribute nothing; flag raised
+    returned = torch.from_numpy(o_send0 * 2).to(cfg.torch_dtype).to(DEV)
+    gate0 = torch.from_numpy(s0["gate"]).to(DEV)
+    status.zero_()
+    out = ops.combine(returned, idx0, pos0, gate0, offs0, E_l, status=status)
+    assert int(status.item()) == 1
+    assert_bits_equal(out, O.combine(o_send0 * 2, s0["idx"], s0["pos"], s0["gate"], s0["offs"], E_l, cfg.dtype), "combine")
+    # an expert id outside the layout is skipped as well (no read outside the buffer)
+    bad_idx = idx0.clone()
+    bad_idx[3, 1] = E + 5 * E_l
+    status.zero_()
+    out = ops.combine(returned, bad_idx, pos0, gate0, offs0, E_l, status=status)
+    assert int(status.item()) == 1
+    o_bad = s0["idx"].copy()
+    o_bad[3, 1] = E + 5 * E_l
+    assert_bits_equal(out, O.combine(o_send0 * 2, o_bad, s0["pos"], s0["gate"], s0["offs"], E_l, cfg.dtype), "combine, bad id")
+
+
 UNPACK_CASES = [("plumbing", None), ("small", None), ("mixtral", 1024), ("finegrained", 512), ("zipf_k4", 1024)]
 
 

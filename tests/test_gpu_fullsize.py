@@ -18,7 +18,7 @@ from iris_testing_amd.pipeline import DispatchPipeline  # noqa: E402
 DEV = "cuda"
 
 
-@pytest.mark.parametrize("name", ["mixtral", "finegrained", "zipf_k4"])
+@pytest.mark.parametrize("name", ["mixtral", "finegrained", "zipf_k1", "zipf_k4", "zipf_k8"])
 def test_full_size_pipeline(name):
     cfg = CONFIGS[name]
     print(f"case {cfg}", flush=True)
@@ -87,7 +87,7 @@ def test_full_size_pipeline(name):
     assert_bits_equal(out1[:256], o_out, "combine (first 256 tokens)")
 
 
-@pytest.mark.parametrize("name", ["mixtral", "finegrained", "small", "zipf_k2"])
+@pytest.mark.parametrize("name", ["mixtral", "finegrained", "small", "zipf_k1", "zipf_k2", "zipf_k8"])
 def test_fused_destination_equals_copies(name):
     """The destination side without the two row copies (row map, gathering first GEMM, scattering second
     GEMM, zeroed padding rows) runs the same arithmetic on the same rows as unpack + MLP + return pack, so

@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/moe_gfx950.h but not exported"
     assert sorted(L.exported_symbols()) == declared, "ctypes table and header disagree"
-    assert lib.moe_abi_version() == 1
+    assert lib.moe_abi_version() == 2
     assert lib.moe_last_error() == b""
 
 

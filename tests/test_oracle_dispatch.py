@@ -53,6 +53,8 @@ def test_counts_offsets_payload_against_bucket_loop(T, E, k, W, seed):
     assert np.array_equal(o_counts, counts) and o_counts.dtype == np.int32
     assert np.array_equal(o_sizes, sizes) and np.array_equal(o_offs, offs)
     assert np.array_equal(O.send_payload(x, row_token), payload)
+    lp, lc, lo, ls = O.bucket_loop_pack(x, idx, W, E)  # the per-slot loop the benchmark times for the record
+    assert np.array_equal(lp, payload) and np.array_equal(lc, counts) and np.array_equal(lo, offs) and np.array_equal(ls, sizes)
     # brute-force count cube and invariants
     cube = np.zeros(E, np.int64)
     np.add.at(cube, idx.reshape(-1), 1)
@@ -203,3 +205,73 @@ def test_oracle_reproduces_the_frozen_dispatch_vectors():
     # a few facts that must hold for the vectors to mean anything
     assert int(frozen["M"]) == max(int(frozen[f"counts{s}"].sum(1).max()) for s in range(3))
     assert int(frozen["recv_counts"].sum()) == frozen["rows"].shape[0] and (frozen["pca"] == frozen["recv_counts"].T).all()
+
+
+def test_capacity_overflow_drops_the_same_rows_everywhere():
+    """With M below the largest pair size the pack drops the rows at and past M of a slot; the receive side then
+    sees zero rows where they were counted, the way back has no slot for them, and the combine skips them.
+    Pinned per element against the definition (a routed slot survives iff its row inside the slot is < M)."""
+    rng = np.random.default_rng(11)
+    T, H, E, k, W = 40, 4, 6, 2, 3
+    E_l = E // W
+    xs = [coded_rows(T, H) + 1000.0 * s for s in range(W)]
+    idxs = [np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32) for _ in range(W)]
+    parts = []
+    for x, idx in zip(xs, idxs):
+        counts = O.send_counts(idx, W, E)
+        sizes, offs = O.dst_sizes_offsets(counts)
+        pos, row_token = O.payload_positions(idx, E)
+        parts.append(dict(counts=counts, sizes=sizes, offs=offs, pos=pos, row_token=row_token))
+    M_full = O.pair_capacity(np.stack([p["sizes"] for p in parts]))
+    M = M_full - 6
+    assert any((p["sizes"] > M).any() for p in parts)
+    with pytest.raises(ValueError):
+        O.pack_fixed_m(O.send_payload(xs[0], parts[0]["row_token"]), parts[0]["offs"], parts[0]["sizes"], M)
+    sends = [O.pack_fixed_m(O.send_payload(x, p["row_token"]), p["offs"], p["sizes"], M, drop=True) for x, p in zip(xs, parts)]
+    # the pack, per element
+    for x, idx, p, send in zip(xs, idxs, parts, sends):
+        seen = np.zeros((W, M), bool)
+        for t in range(T):
+            for kk in range(k):
+                d = idx[t, kk] // E_l
+                m = p["pos"][t, kk] - p["offs"][d]
+                if m < M:
+                    assert np.array_equal(send[d, m], x[t])
+                    seen[d, m] = True
+        assert (send[~seen] == 0).all()
+    # the receive side of rank 0
+    recv = np.stack([s[0] for s in sends])
+    rc = np.stack([p["counts"][0] for p in parts]).astype(np.int32)
+    rows = O.unpack_expert_major(recv, rc)
+    assert rows.shape[0] == rc.sum()
+    eo = O.build_expert_offsets(rc)
+    r = 0
+    n_dropped = 0
+    for e in range(E_l):
+        for s in range(W):
+            for j in range(rc[s, e]):
+                m = eo[s, e] + j
+                if m < M:
+                    assert np.array_equal(rows[r], recv[s, m])
+                else:
+                    assert (rows[r] == 0).all()
+                    n_dropped += 1
+                r += 1
+    assert n_dropped > 0
+    CAP = int(rc.max())
+    tb, _ = O.recv_to_token_buf(recv, rc, CAP)
+    assert np.array_equal(O.shuffle(tb, rc.T), rows)
+    # the way back: the surviving rows return to their slots, the dropped ones have none
+    back = O.return_pack(rows * 2, rc, M)
+    assert np.array_equal(back, recv * 2)
+    # combine on shard 0: dropped slots contribute nothing
+    p0, gate = parts[0], rng.random((T, k)).astype(np.float32)
+    out = O.combine(sends[0], idxs[0], p0["pos"], gate, p0["offs"], E_l, "f32")
+    for t in range(T):
+        acc = np.zeros(H, np.float32)
+        for kk in range(k):
+            d = idxs[0][t, kk] // E_l
+            m = p0["pos"][t, kk] - p0["offs"][d]
+            if m < M:
+                acc = (acc + gate[t, kk] * xs[0][t]).astype(np.float32)
+        assert np.array_equal(out[t], acc)

@@ -69,3 +69,89 @@ def test_fp8_mlp_is_the_dequantised_mlp():
     ref = O.expert_mlp(x, cnt, wg, wd, "swiglu", "f32", w_up=wu)
     rms = np.sqrt((ref ** 2).mean())
     assert np.abs(out - ref).max() < 0.25 * rms  # fp8 noise, far below signal
+
+
+def _fp8_explicit(x, cnt, gq, gs, uq, us, dq, ds, swap_scales=False, per_expert_scale=False, swap_gate_up=False):
+    """The fp8 SwiGLU expert spelled out with torch's own e4m3 / bf16 casts and float64 arithmetic:
+    quantise rows (amax/448), decode every code with torch.float8_e4m3fn, multiply in float64, scale by
+    s_tok[m] * s_ch[n], SwiGLU, round to bf16, re-quantise, multiply, scale, round.  The keyword arguments
+    plant the plausible mistakes.  Returns (hidden [S,F], out [S,H]) as float32 arrays."""
+    import torch
+    dec = lambda q: torch.from_numpy(np.ascontiguousarray(q)).view(torch.float8_e4m3fn).double()  # noqa: E731
+
+    def quant_rows(a):  # a: torch float32 [R,C] -> codes (as float64 values), scales float32
+        amax = a.abs().amax(dim=1)
+        safe = torch.where(amax == 0, torch.ones_like(amax), amax)
+        scale = torch.where(amax == 0, torch.ones_like(amax), safe / 448.0)
+        inv = torch.where(amax == 0, torch.ones_like(amax), 448.0 / safe)
+        q = (a * inv[:, None]).to(torch.float8_e4m3fn)
+        return q.double(), scale
+
+    xt = torch.from_numpy(x)
+    xq, xs = quant_rows(xt)
+    gs_, us_ = (us, gs) if swap_scales else (gs, us)
+    if per_expert_scale:
+        gs_ = np.repeat(gs.mean(axis=1, keepdims=True), gs.shape[1], axis=1)
+        us_ = np.repeat(us.mean(axis=1, keepdims=True), us.shape[1], axis=1)
+    S, F = x.shape[0], gq.shape[2]
+    h = torch.zeros((S, F), dtype=torch.float64)
+    r = 0
+    for e, c in enumerate(cnt):
+        c = int(c)
+        if c:
+            sx = xs[r:r + c, None].double()
+            g = (xq[r:r + c] @ dec(gq[e])) * sx * torch.from_numpy(gs_[e]).double()[None, :]
+            u = (xq[r:r + c] @ dec(uq[e])) * sx * torch.from_numpy(us_[e]).double()[None, :]
+            if swap_gate_up:
+                g, u = u, g
+            h[r:r + c] = g / (1.0 + torch.exp(-g)) * u
+        r += c
+    hb = h.float().bfloat16().float()
+    hq, hs = quant_rows(hb)
+    y = torch.zeros((S, dq.shape[2]), dtype=torch.float64)
+    r = 0
+    for e, c in enumerate(cnt):
+        c = int(c)
+        if c:
+            y[r:r + c] = (hq[r:r + c] @ dec(dq[e])) * hs[r:r + c, None].double() * torch.from_numpy(ds[e]).double()[None, :]
+        r += c
+    return hb.numpy(), y.float().bfloat16().float().numpy()
+
+
+def _within_a_bf16_step(got, ref):
+    """|got - ref| <= 2^-7 |ref| + 2^-10 rms(ref): one bf16 rounding step (fp32 against float64 summation can flip
+    a rounding) and a floor for outputs that cancel to almost nothing."""
+    rms = float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))
+    return np.abs(got.astype(np.float64) - ref) <= 2.0 ** -7 * np.abs(ref) + 2.0 ** -10 * rms
+
+
+def test_fp8_expert_halves_against_an_explicit_dequantised_evaluation():
+    rng = np.random.default_rng(21)
+    E_l, H, Fd = 3, 128, 96
+    cnt = np.array([37, 0, 28], np.int32)
+    S = int(cnt.sum())
+    x = O.bf16_round((rng.standard_normal((S, H)) * rng.uniform(0.3, 3.0, (S, 1))).astype(np.float32))
+    # channel magnitudes spread over a factor of eight, differently for gate and up, so that a wrong scale shows
+    wg = (rng.standard_normal((E_l, H, Fd)) * rng.uniform(0.25, 2.0, (E_l, 1, Fd)) / np.sqrt(H)).astype(np.float32)
+    wu = (rng.standard_normal((E_l, H, Fd)) * rng.uniform(0.25, 2.0, (E_l, 1, Fd)) / np.sqrt(H)).astype(np.float32)
+    wd = (rng.standard_normal((E_l, Fd, H)) * rng.uniform(0.25, 2.0, (E_l, 1, H)) / np.sqrt(Fd)).astype(np.float32)
+    (gq, gs), (uq, us), (dq, ds) = (O.quantize_cols_fp8(w) for w in (wg, wu, wd))
+    h_ref, _ = _fp8_explicit(x, cnt, gq, gs, uq, us, dq, ds)
+    h = O.expert_up_fp8(x, cnt, gq, gs, uq, us)
+    assert _within_a_bf16_step(h, h_ref).all(), "expert_up_fp8 differs from the explicit evaluation"
+    # the second half on the same hidden activation (the explicit evaluation re-quantises what it is given)
+    _, y_ref = _fp8_explicit(x, cnt, gq, gs, uq, us, dq, ds)
+    y = O.expert_down_fp8(h_ref, cnt, dq, ds)
+    assert _within_a_bf16_step(y, y_ref).all(), "expert_down_fp8 differs from the explicit evaluation"
+    # planted mistakes must fail the same bound, by a wide margin
+    for kw in (dict(swap_scales=True), dict(per_expert_scale=True), dict(swap_gate_up=True)):
+        h_bad, y_bad = _fp8_explicit(x, cnt, gq, gs, uq, us, dq, ds, **kw)
+        frac = 1.0 - _within_a_bf16_step(h, h_bad).mean()
+        assert frac > 0.5, f"{kw}: only {frac:.2f} of the hidden activations notice"
+    # the row quantisation on its own, codes and scales, against torch's cast
+    import torch
+    q, s = O.quantize_rows_fp8(x)
+    xt = torch.from_numpy(x)
+    amax = xt.abs().amax(dim=1)
+    assert np.array_equal(s, (amax / 448.0).numpy())
+    assert np.array_equal(q, (xt * (448.0 / amax)[:, None]).to(torch.float8_e4m3fn).view(torch.uint8).numpy())
