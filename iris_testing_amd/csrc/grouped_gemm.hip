@@ -188,6 +188,15 @@ __device__ __forceinline__ void gg_dma16(const uint8_t* sbase, uint32_t voff, ui
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0" : : "s"(sbase), "v"(voff), "s"(lds_addr) : "memory");
 }
 
+// The lane id read afresh (two instructions) where it is needed.  What the epilogue and the tile set-up derive from it
+// is then computed there, once per tile, instead of being hoisted out of the tile loop as a dozen lane-constant
+// invariants that occupy -- or spill -- registers across the whole K loop.
+__device__ __forceinline__ int gg_lane_now() {
+    int l;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+    return l;
+}
+
 // a wave-uniform value forced into scalar registers
 __device__ __forceinline__ const uint8_t* gg_uniform(const uint8_t* p) {
     const uint64_t v = (uint64_t)p;
@@ -248,6 +257,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     __shared__ int g_row_start[GG_MAXG + 1];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wave_s = __builtin_amdgcn_readfirstlane(wave);  // the same, known to be wave-uniform (a scalar register)
     const int wm = wave >> 1, wn = wave & 1;
     const int Nt = p.Npad / BN;
 
@@ -300,9 +310,12 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     const uint8_t* Ab_ = (p.a_map ? p.A : p.A + (size_t)(t).row0 * p.K * ES) + (size_t)(t).ks0 * ROWB;      \
     const uint8_t* Bb_ = p.B + (size_t)(t).g * p.Npad * p.K * ES + (size_t)(t).nt * BN * ROWB + (size_t)(t).ks0 * b_slab; \
     uint32_t aoff_[RA];                                                                                     \
+    const int ln_ = gg_lane_now();  /* lrow and lchunk again, derived per tile */                              \
+    const int lrow_ = wave_s * WROWS + (ln_ >> 2);                                                            \
+    const uint32_t lcb_ = (uint32_t)(((ln_ & 3) ^ ((ln_ >> 4) & 3)) * 16);                                     \
     _Pragma("unroll") for (int r = 0; r < RA; ++r) {                                                         \
-        const int lr_ = max(min(r * LR + lrow, (t).rv - 1), 0);  /* tile row this lane fetches, clamped */     \
-        aoff_[r] = (uint32_t)(p.a_map ? max(p.a_map[(t).row0 + lr_], 0) : lr_) * ldk + lchunk * 16;           \
+        const int lr_ = max(min(r * LR + lrow_, (t).rv - 1), 0);  /* tile row this lane fetches, clamped */    \
+        aoff_[r] = (uint32_t)(p.a_map ? max(p.a_map[(t).row0 + lr_], 0) : lr_) * ldk + lcb_;                  \
     }
     // load d (0 .. LPS-1) of one stage: A rounds first, then B rounds
 #define GG_LD(d, ap_, bp_, aoff_, slot)                                                                       \
@@ -466,10 +479,11 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         if constexpr (SPLIT) {  // (every tile of this instantiation is a part; the epilogue below is the other one's)
             float* wsT = p.part_ws + (size_t)unit * (BM * BN);
             constexpr int NQp = FP8 ? 4 : 1;
-            const int clp = FP8 ? (lane >> 5) * 4 : (lane >> 4) * 4;
+            const int lane_p = gg_lane_now(), rbase_p = (wave_s >> 1) * (BM / NWM);
+            const int clp = FP8 ? (lane_p >> 5) * 4 : (lane_p >> 4) * 4;
 #pragma unroll
             for (int i = 0; i < TM; ++i) {
-                const int r = wm * (BM / NWM) + i * MT + (lane & (MT - 1));
+                const int r = rbase_p + i * MT + (lane_p & (MT - 1));
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
 #pragma unroll
@@ -502,13 +516,15 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         bf16_t* C = (bf16_t*)p.C;
         constexpr int NQ = FP8 ? 4 : 1;              // runs of four columns per lane and tile
         constexpr int UPJ = 32 / MT;                 // tiles between a gate tile and its up tile
-        const int clane = FP8 ? (lane >> 5) * 4 : (lane >> 4) * 4;  // first column of the lane's run inside 8 (fp8) / 16 (bf16) columns
+        // (the lane-derived constants of the epilogue are derived here, once per tile, from a fresh read of the lane id)
+        const int lane_e = gg_lane_now(), rbase_e = (wave_s >> 1) * (BM / NWM), cbase_e = (wave_s & 1) * (BN / 2);
+        const int clane = FP8 ? (lane_e >> 5) * 4 : (lane_e >> 4) * 4;  // first column of the lane's run inside 8 (fp8) / 16 (bf16) columns
         bool ok[TM];
         bf16_t* crow[TM];
         float rs[TM];
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            const int r = wm * (BM / NWM) + i * MT + (lane & (MT - 1));
+            const int r = rbase_e + i * MT + (lane_e & (MT - 1));
             ok[i] = r < rv;
             const size_t grow = (size_t)(row0 + (ok[i] ? r : 0));
             rs[i] = 1.f;
@@ -528,7 +544,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             if constexpr (EPI == EPI_SWIGLU) {
                 if ((j / UPJ) % 2 == 1) continue;  // an up tile: consumed together with its gate tile
             }
-            const int pcol = nt * BN + wn * (BN / 2) + j * MT;  // first packed column of the tile
+            const int pcol = nt * BN + cbase_e + j * MT;  // first packed column of the tile
             const int colj = (EPI == EPI_SWIGLU ? (pcol / 64) * 32 + pcol % 32 : pcol) + clane;
             if (FP8 && i == 0) {
 #pragma unroll

@@ -126,7 +126,8 @@ def test_expert_layer_signature():
 def test_expert_layer_bf16_reuses_retiled_weights_until_they_change():
     """bf16 weights are re-tiled once per tensor version: a second call gives the same bits, an in-place update of
     the weights is seen by the next call, and the result is the oracle's."""
-    from iris_testing_amd.layers import expert as expert_mod
+    import importlib
+    expert_mod = importlib.import_module("iris_testing_amd.layers.expert")  # (the package re-exports the function under this name)
     rng = np.random.default_rng(2)
     cnt = np.array([300, 0, 45, 130], dtype=np.int32)
     S = int(cnt.sum())
