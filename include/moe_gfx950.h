@@ -70,6 +70,18 @@ int moe_count_and_offsets(const int32_t* topk_idx, int T, int k, int E, int W, i
                           int32_t* expert_offs, int32_t* dst_sizes, int32_t* dst_offsets, int32_t* caps,
                           int32_t* pos, int32_t* row_token, void* ws, size_t ws_bytes, moe_stream_t stream);
 
+/* moe_count_and_offsets for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): no counterpart in the reference.  Same arguments and results
+ * without the workspace: the scratch is a fixed MOE_COUNT_SCRATCH_BYTES array inside the library's device image,
+ * one copy per GPU, held until the process ends.  Sizes whose moe_count_workspace_bytes(T,k,E) exceed it are
+ * rejected with MOE_ERR_WORKSPACE.  All calls on one GPU share that array: calls that overlap on one GPU (two
+ * streams, two threads) race; calls on one stream are ordered and safe.  Nothing is allocated or freed. */
+#define MOE_COUNT_SCRATCH_BYTES (4u << 20)
+size_t moe_count_static_scratch_bytes(void);
+int moe_count_and_offsets_static(const int32_t* topk_idx, int T, int k, int E, int W, int32_t* send_counts,
+                                 int32_t* expert_offs, int32_t* dst_sizes, int32_t* dst_offsets, int32_t* caps,
+                                 int32_t* pos, int32_t* row_token, moe_stream_t stream);
+
 /* ---- a4/a5 on their own: build_expert_offsets (reference utils.py:20-31) and _build_dst_offsets
  * (benchmark.py:44-49) for a given counts [W,E_l].  dst_sizes / dst_offsets may be NULL. */
 int moe_build_expert_offsets(const int32_t* counts, int W, int E_l, int32_t* expert_offs, int32_t* dst_sizes,

@@ -35,6 +35,8 @@ _SIGNATURES = {
     "moe_route_topk": (c_int, [P, P, P, c_int, c_int, c_int, c_int, c_int, P, P, P, P]),
     "moe_count_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "moe_count_and_offsets": (c_int, [P, c_int, c_int, c_int, c_int, P, P, P, P, P, P, P, P, c_size_t, P]),
+    "moe_count_static_scratch_bytes": (c_size_t, []),
+    "moe_count_and_offsets_static": (c_int, [P, c_int, c_int, c_int, c_int, P, P, P, P, P, P, P, P]),
     "moe_build_expert_offsets": (c_int, [P, c_int, c_int, P, P, P, P]),
     "moe_max_floor1": (c_int, [P, c_int, P, P]),
     "moe_pack_payload": (c_int, [P, c_int, c_int, c_int, P, c_int, P, P]),

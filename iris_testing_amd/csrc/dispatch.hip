@@ -12,6 +12,7 @@
 // earlier lanes of this block),  with LDS histograms, a wave prefix scan and per-expert lane masks.
 // All integer work: results are bit-exact by construction.
 #include "common.h"
+#include <atomic>
 
 namespace {
 
@@ -638,6 +639,52 @@ extern "C" int moe_count_and_offsets(const int32_t* topk_idx, int T, int k, int 
     offsets_kernel<<<1, WAVE, 0, s>>>(counts, E, W, expert_start, send_counts, expert_offs, dst_sizes, dst_offsets, caps);
     if (T > 0) rank_kernel<<<ceil_div(NB, 4), 256, 0, s>>>(topk_idx, base, expert_start, pos, row_token, T, k, E, NB);
     return moe_check_launch("count_and_offsets");
+}
+
+// ---- the same entry point for callers that may not allocate: the workspace is a fixed array in the library's own
+// device image instead of a caller buffer.  Each GPU holds its own copy of the array at its own address; the address
+// is looked up once per device, with that device current, and kept.
+static __device__ __align__(256) unsigned char scratch[MOE_COUNT_SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::atomic<void*> g_scratch_ptr[MAX_DEVICES];
+
+int count_scratch(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return moe_fail(MOE_ERR_LAUNCH, "count_and_offsets_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= MAX_DEVICES) return moe_fail(MOE_ERR_UNSUPPORTED, "count_and_offsets_static: device %d", dev);
+    void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            return moe_fail(MOE_ERR_LAUNCH, "count_and_offsets_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // (racing first calls look up the same address)
+    }
+    *out = ptr;
+    return MOE_OK;
+}
+}  // namespace
+
+extern "C" size_t moe_count_static_scratch_bytes(void) { return MOE_COUNT_SCRATCH_BYTES; }
+
+extern "C" int moe_count_and_offsets_static(const int32_t* topk_idx, int T, int k, int E, int W, int32_t* send_counts,
+                                            int32_t* expert_offs, int32_t* dst_sizes, int32_t* dst_offsets, int32_t* caps,
+                                            int32_t* pos, int32_t* row_token, moe_stream_t stream) {
+    MOE_REQUIRE(T >= 0 && E > 0 && k >= 1, MOE_ERR_INVALID, "count_and_offsets_static: bad shape T=%d E=%d k=%d", T, E, k);
+    const size_t need = moe_count_workspace_bytes(T, k, E);
+    MOE_REQUIRE(need <= (size_t)MOE_COUNT_SCRATCH_BYTES, MOE_ERR_WORKSPACE,
+                "count_and_offsets_static: T=%d tokens with E=%d experts need %zu bytes of scratch, the built-in array holds %zu "
+                "(use moe_count_and_offsets with a workspace of your own)", T, E, need, (size_t)MOE_COUNT_SCRATCH_BYTES);
+    void* ws = nullptr;
+    const int rc = count_scratch(&ws);
+    if (rc) return rc;
+    // every cell of the workspace that the kernels read is written earlier in the same call (histogram cells by the
+    // block that owns them, prefixes by the scan): nothing has to start at zero, stale contents of an earlier call
+    // are never read
+    return moe_count_and_offsets(topk_idx, T, k, E, W, send_counts, expert_offs, dst_sizes, dst_offsets, caps, pos, row_token, ws,
+                                 (size_t)MOE_COUNT_SCRATCH_BYTES, stream);
 }
 
 extern "C" int moe_build_expert_offsets(const int32_t* counts, int W, int E_l, int32_t* expert_offs, int32_t* dst_sizes,

@@ -43,6 +43,18 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.moe_count_workspace_bytes(1000, 2, 8) == 4 * (2 * 8 * 16 + 2 * 8 + 1)
 
 
+def test_static_scratch_count_rejects_oversized_inputs_without_a_gpu():
+    """The allocation-free counting entry point checks its size limit before it touches the GPU."""
+    from iris_testing_amd import _lib as L
+    lib = L.lib()
+    cap = lib.moe_count_static_scratch_bytes()
+    assert cap == 4 << 20
+    assert lib.moe_count_workspace_bytes(1 << 17, 2, 512) > cap
+    rc = lib.moe_count_and_offsets_static(None, 1 << 17, 2, 512, 8, None, None, None, None, None, None, None, None)
+    assert rc == -3 and b"scratch" in lib.moe_last_error()
+    assert lib.moe_count_and_offsets_static(None, 64, 0, 8, 4, None, None, None, None, None, None, None, None) == -1
+
+
 def test_host_layer_rejects_cpu_tensors_like_the_reference():
     from iris_testing_amd import utils
     from iris_testing_amd.baseline import reorder_flat_to_token_buf
