@@ -49,13 +49,18 @@ const char* moe_last_error(void);
 
 /* ---- a1: router softmax + top-k ------------------------------------------------------------
  * Replaces `F.softmax(einsum('th,he->te', tokens, router)); topk(...)` (reference utils.py:200-202).
- * logits[t,e] = bias[e] + fp32 fmaf chain over ascending h; selection on the logits, descending,
- * ties to the lower expert id; topk_gate = softmax probability of each selected expert (not
- * renormalised).  x [T,H], router [H,E] in `dtype`; bias fp32 [E] or NULL.
- * logits_ws: fp32 [T,E] scratch (also an output: the raw logits). */
+ * Pinned fp32 arithmetic: h is cut into MOE_ROUTE_SEGMENTS contiguous segments of L = ceil(H/8) rounded up
+ * to a multiple of 8 elements; s_p = fmaf chain over the h of segment p in ascending order from +0 (an
+ * empty segment gives +0); logits[t,e] = ((..(s_0 + s_1) + ..) + s_7) + bias[e], fp32 additions in that
+ * order.  Selection on the logits, descending, ties to the lower expert id; topk_gate = softmax
+ * probability of each selected expert (not renormalised).  x [T,H], router [H,E] in `dtype`; bias fp32
+ * [E] or NULL.  logits: fp32 [T,E] output (the raw logits).  ws: moe_route_workspace_bytes(T,E) bytes of
+ * scratch (the segments' partial sums). */
+#define MOE_ROUTE_SEGMENTS 8
+size_t moe_route_workspace_bytes(int T, int E);
 int moe_route_topk(const void* x, const void* router, const float* bias, int dtype, int T, int H, int E,
-                   int k, float* logits_ws, int32_t* topk_idx /*[T,k]*/, float* topk_gate /*[T,k]*/,
-                   moe_stream_t stream);
+                   int k, float* logits /*[T,E]*/, int32_t* topk_idx /*[T,k]*/, float* topk_gate /*[T,k]*/,
+                   void* ws, size_t ws_bytes, moe_stream_t stream);
 
 /* ---- a2/a4/a5/a6/a7 + payload order of a3 ----------------------------------------------------
  * Replaces the bucket loop and count/offset bookkeeping of route_and_pack_padding_free

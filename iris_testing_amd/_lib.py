@@ -32,7 +32,8 @@ P = c_void_p
 _SIGNATURES = {
     "moe_abi_version": (c_int, []),
     "moe_last_error": (c_char_p, []),
-    "moe_route_topk": (c_int, [P, P, P, c_int, c_int, c_int, c_int, c_int, P, P, P, P]),
+    "moe_route_workspace_bytes": (c_size_t, [c_int, c_int]),
+    "moe_route_topk": (c_int, [P, P, P, c_int, c_int, c_int, c_int, c_int, P, P, P, P, c_size_t, P]),
     "moe_count_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "moe_count_and_offsets": (c_int, [P, c_int, c_int, c_int, c_int, P, P, P, P, P, P, P, P, c_size_t, P]),
     "moe_count_static_scratch_bytes": (c_size_t, []),

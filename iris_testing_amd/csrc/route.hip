@@ -4,18 +4,26 @@
 // Replaces the device work of `F.softmax(torch.einsum('th,he->te', tokens, router), dim=-1)`
 // followed by `torch.topk(..., topk)` in the reference (utils.py:200-202).
 //
-// Reduction order (what makes the indices reproducible bit-for-bit on a CPU):
-//   logit[t,e] = bias[e] + chain,  chain = fmaf(x[t,h], w[h,e], chain) for h = 0..H-1, chain0 = +0.0f
-// Every (t,e) chain is one accumulator element walked over H in ascending order, so no cross-lane or
-// cross-block partial sums exist.  The chains run on the matrix cores, but only through K = 1 fp32 MFMAs,
-// which perform exactly one fused multiply-add per output element and instruction; MFMAs with K > 1 (and all
-// bf16 ones) sum several products in an order that is not specified and are not used.
+// Reduction order (what makes the indices reproducible bit-for-bit on a CPU): h is cut into MOE_ROUTE_SEGMENTS = 8
+// contiguous segments of L = ceil(H / 8) rounded up to a multiple of 8 elements (the last ones shorter or empty);
+//   s_p        = chain over the h of segment p,  chain = fmaf(x[t,h], w[h,e], chain) in ascending h, chain0 = +0.0f
+//   logit[t,e] = ((((((s_0 + s_1) + s_2) + s_3) + s_4) + s_5) + s_6) + s_7, then + bias[e]   (fp32 additions, in this order)
+// Eight independent chains per (t,e) instead of one: a chain is a sequence of dependent instructions, and its length,
+// not the memory system, bounded the kernel while it ran over all of H.  Every chain is one accumulator element of one
+// block walked over its segment in ascending order; the eight partial sums meet in the top-k kernel.  The chains run on
+// the matrix cores, but only through K = 1 fp32 MFMAs, which perform exactly one fused multiply-add per output element
+// and instruction; MFMAs with K > 1 (and all bf16 ones) sum several products in an order that is not specified and are
+// not used.
 #include "common.h"
 #include <type_traits>
 
 namespace {
 
 constexpr int RT_TB = 64;  // tokens per block: one per lane
+constexpr int RT_P = MOE_ROUTE_SEGMENTS;
+
+// length of a segment of the reduction (part of the specification of the logits: the CPU checker evaluates the same)
+__host__ __device__ inline int route_segment_len(int H) { return ((H + RT_P - 1) / RT_P + 7) & ~7; }
 
 template <typename XT>
 struct VecLoad;
@@ -51,41 +59,58 @@ struct VecLoad<float> {
 //   B operand: lane l holds w[h][e0 + l % SHAPE]         (the SHAPE experts, repeated across the lanes)
 //   D, SHAPE = 16: register v holds token t0 + 16 * (v / 4) + 4 * (l / 16) + v % 4, expert e0 + l % 16
 //   D, SHAPE = 4:  register v holds token t0 + 4 * (l / 4) + v,                     expert e0 + l % 4
-// Block = NWV waves on the same 64 tokens, wave i on experts [e0 + i * SHAPE, + SHAPE).  Both operands are converted
-// to fp32 on their way into LDS (the lane reads four consecutive h of its own token row, and of its expert in the
-// transposed router slab, with one 128-bit read each).
+// Block = NWV waves on the same TB x 64 tokens; wave i takes G groups of SHAPE experts, [e0 + (i G + g) SHAPE, + SHAPE),
+// and runs the TB x G chains of one h side by side (independent accumulators: their MFMAs follow each other without
+// waiting, and each operand register read from LDS serves G or TB instructions).  Both operands are converted to fp32
+// on their way into LDS (the lane reads four consecutive h of its own token row, and of its expert in the transposed
+// router slab, with one 128-bit read each).
 typedef float rt_f4 __attribute__((ext_vector_type(4)));
 typedef float rt_f16 __attribute__((ext_vector_type(16)));
 typedef unsigned int rt_u4 __attribute__((ext_vector_type(4)));
 
-template <typename XT, int SHAPE, int NWV>
-__global__ __launch_bounds__(NWV * WAVE) void route_logits_mfma_kernel(const XT* __restrict__ x, const XT* __restrict__ w,
-                                                                        const float* __restrict__ bias,
-                                                                        float* __restrict__ logits, int T, int H, int E) {
+template <typename XT, int SHAPE, int TB, int G, int NWV, int CPR /* 16-byte chunks of a token row per slab */>
+__global__ __launch_bounds__(NWV * WAVE, (NWV == 4 && TB == 2 ? 2 : 1)) void route_logits_mfma_kernel(const XT* __restrict__ x, const XT* __restrict__ w,
+                                                                        float* __restrict__ part /*[RT_P][T][E]*/, int T,
+                                                                        int Hrow, int E) {
     static_assert(SHAPE == 4 || SHAPE == 16, "experts per MFMA");
     constexpr int NTH = NWV * WAVE;
-    constexpr int EB = NWV * SHAPE;            // experts per block
+    constexpr int NTOK = TB * RT_TB;           // tokens per block
+    constexpr int EB = NWV * G * SHAPE;        // experts per block
     constexpr int VN = VecLoad<XT>::N;         // elements per 16 bytes
-    constexpr int KC = 16 * VN;                // h per slab: 256 bytes of every token row
+    constexpr int KC = CPR * VN;               // h per slab: CPR x 16 bytes of every token row
+    constexpr int NCH = CPR;                   // chunks (VN consecutive h) per slab
     constexpr int XS = KC + 4;                 // padded fp32 row (conflict-free 128-bit row reads)
-    constexpr int XPT = RT_TB * 16 / NTH;      // 16-byte x chunks per thread and slab
+    constexpr int XPT = NTOK * CPR / NTH;      // 16-byte x chunks per thread and slab
     constexpr int WQ = KC * EB / (4 * NTH);    // groups of four h of one expert per thread and slab
-    // slabs in flight per block: one block holds D x 16 KB of token rows in registers, which is what hides the
-    // memory latency when there is only one block of 64 tokens per compute unit
-    constexpr int D = NWV == 1 ? 2 : 4;
+    // slabs in flight per block (in registers, until their turn in LDS)
+    constexpr int D = 2;
     constexpr int NACC = SHAPE == 16 ? 16 : 4;
     typedef typename std::conditional<SHAPE == 16, rt_f16, rt_f4>::type acc_t;
-    static_assert((KC * EB) % (4 * NTH) == 0, "router slab split");
-    __shared__ __align__(16) float xs[RT_TB][XS];
+    static_assert((KC * EB) % (4 * NTH) == 0 && (NTOK * CPR) % NTH == 0 && (CPR == 8 || CPR == 16), "router slab split");
+    __shared__ __align__(16) float xs[NTOK][XS];
     __shared__ __align__(16) float wsT[EB][KC + 4];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int t0 = blockIdx.x * RT_TB, eb0 = blockIdx.y * EB;
-    const float* wrow = &wsT[wave * SHAPE + lane % SHAPE][0];
-    const float* xrow = &xs[lane][0];
-    acc_t acc;
+    // (the segment is the fastest-running block index: the blocks that are resident together then read whole token
+    // rows between them, not the same eighth of every row, which would load the memory channels unevenly)
+    const int t0 = blockIdx.y * NTOK, eb0 = blockIdx.z * EB;
+    // this block's segment of the reduction: h in [h0, h0 + H) of rows that are Hrow long (H = 0: an empty segment)
+    const int seg = blockIdx.x, seg_len = route_segment_len(Hrow);
+    const int h0 = min(seg * seg_len, Hrow);
+    const int H = min(seg_len, Hrow - h0);
+    const float* wrow[G];
+    const float* xrow[TB];
 #pragma unroll
-    for (int v = 0; v < NACC; ++v) acc[v] = 0.f;
+    for (int g = 0; g < G; ++g) wrow[g] = &wsT[(wave * G + g) * SHAPE + lane % SHAPE][0];
+#pragma unroll
+    for (int b = 0; b < TB; ++b) xrow[b] = &xs[b * RT_TB + lane][0];
+    acc_t acc[TB][G];
+#pragma unroll
+    for (int b = 0; b < TB; ++b)
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int v = 0; v < NACC; ++v) acc[b][g][v] = 0.f;
 
     // Slab s covers h in [ks, ks + KC), ks = min(s * KC, H - KC) (0 when H < KC): the last slab of a row whose
     // length is no multiple of KC overlaps its predecessor and is consumed from offset s * KC - ks on; slabs past
@@ -96,15 +121,18 @@ __global__ __launch_bounds__(NWV * WAVE) void route_logits_mfma_kernel(const XT*
 #pragma unroll
     for (int i = 0; i < XPT; ++i) {
         const int c = tid + i * NTH;
-        xoff[i] = min(c / 16, T - 1 - t0) * H + min((c % 16) * VN, H - VN);
+        xoff[i] = min(c / CPR, T - 1 - t0) * Hrow + max(min((c % CPR) * VN, H - VN), 0);
     }
 #pragma unroll
     for (int i = 0; i < WQ; ++i) {
         const int c = tid + i * NTH;  // expert c % EB, h 4 * (c / EB) .. + 3 of the slab
 #pragma unroll
-        for (int q = 0; q < 4; ++q) woff[i][q] = min(4 * (c / EB) + q, H - 1) * E + min(eb0 + c % EB, E - 1);
+        for (int q = 0; q < 4; ++q) woff[i][q] = max(min(4 * (c / EB) + q, H - 1), 0) * E + min(eb0 + c % EB, E - 1);
     }
-    const XT* xblk = x + (size_t)t0 * H;
+    // (an empty segment starts at h0 = Hrow: its clamped, never consumed fetches are moved back inside the rows)
+    const int hb = H > 0 ? h0 : 0;
+    const XT* xblk = x + (size_t)t0 * Hrow + hb;
+    w += (size_t)hb * E;
 
     // slabs wait in registers until their turn in LDS
     rt_u4 xr[D][XPT];  // (vector types, not HIP's uint4 struct: the arrays must stay in registers)
@@ -130,10 +158,10 @@ __global__ __launch_bounds__(NWV * WAVE) void route_logits_mfma_kernel(const XT*
                                    __uint_as_float(r_.y << 16), __uint_as_float(r_.y & 0xffff0000u)};                \
                 const rt_f4 hi_ = {__uint_as_float(r_.z << 16), __uint_as_float(r_.z & 0xffff0000u),                 \
                                    __uint_as_float(r_.w << 16), __uint_as_float(r_.w & 0xffff0000u)};                \
-                *reinterpret_cast<rt_f4*>(&xs[c / 16][(c % 16) * VN]) = lo_;                                         \
-                *reinterpret_cast<rt_f4*>(&xs[c / 16][(c % 16) * VN + 4]) = hi_;                                     \
+                *reinterpret_cast<rt_f4*>(&xs[c / CPR][(c % CPR) * VN]) = lo_;                                       \
+                *reinterpret_cast<rt_f4*>(&xs[c / CPR][(c % CPR) * VN + 4]) = hi_;                                   \
             } else {                                                                                                 \
-                *reinterpret_cast<rt_u4*>(&xs[c / 16][(c % 16) * VN]) = xr[d][i];                                    \
+                *reinterpret_cast<rt_u4*>(&xs[c / CPR][(c % CPR) * VN]) = xr[d][i];                                  \
             }                                                                                                        \
         }                                                                                                            \
         _Pragma("unroll") for (int i = 0; i < WQ; ++i) {                                                              \
@@ -144,23 +172,28 @@ __global__ __launch_bounds__(NWV * WAVE) void route_logits_mfma_kernel(const XT*
         }                                                                                                            \
     } while (0)
 
-    // One chunk = VN consecutive h of the lane's token row: VN chained MFMAs.  Within one wave a vector
-    // instruction does not overlap the chain (measured: one VALU between two dependent MFMAs adds 12 to 14 cycles,
-    // a second one 8 more), so the chain's wave does no arithmetic of its own: the operands of the next chunk come
-    // out of LDS ready made (token values converted at the stash), read as one group ahead of the chunk's MFMAs.
+    // One chunk = VN consecutive h: per h, the TB x G independent MFMAs of the wave's chains.  The operands of the next
+    // chunk come out of LDS ready made (token values converted at the stash), read as one group ahead of the chunk's
+    // MFMAs; the wave itself does no arithmetic between its MFMAs.
 #define RT_MFMA(XV, WV, u)                                                                                           \
     do {                                                                                                             \
-        if constexpr (SHAPE == 16)                                                                                   \
-            acc = __builtin_amdgcn_mfma_f32_16x16x1f32(XV[(u) / 4][(u) % 4], WV[(u) / 4][(u) % 4], acc, 0, 0, 0);    \
-        else acc = __builtin_amdgcn_mfma_f32_4x4x1f32(XV[(u) / 4][(u) % 4], WV[(u) / 4][(u) % 4], acc, 0, 0, 0);     \
+        _Pragma("unroll") for (int b_ = 0; b_ < TB; ++b_)                                                             \
+            _Pragma("unroll") for (int g_ = 0; g_ < G; ++g_) {                                                        \
+                if constexpr (SHAPE == 16)                                                                           \
+                    acc[b_][g_] = __builtin_amdgcn_mfma_f32_16x16x1f32(XV[b_][(u) / 4][(u) % 4], WV[g_][(u) / 4][(u) % 4], acc[b_][g_], 0, 0, 0); \
+                else                                                                                                 \
+                    acc[b_][g_] = __builtin_amdgcn_mfma_f32_4x4x1f32(XV[b_][(u) / 4][(u) % 4], WV[g_][(u) / 4][(u) % 4], acc[b_][g_], 0, 0, 0); \
+            }                                                                                                        \
         __builtin_amdgcn_sched_barrier(0);                                                                           \
     } while (0)
     // chunk c: MFMAs on XV / WV, behind the LDS reads of chunk c+1 (at slab offset nxt) into XN / WN
 #define RT_CHUNK(XV, WV, XN, WN, nxt)                                                                                \
     do {                                                                                                             \
         _Pragma("unroll") for (int q_ = 0; q_ < VN / 4; ++q_) {                                                       \
-            XN[q_] = *reinterpret_cast<const rt_f4*>(xrow + (nxt) + 4 * q_);                                         \
-            WN[q_] = *reinterpret_cast<const rt_f4*>(wrow + (nxt) + 4 * q_);                                         \
+            _Pragma("unroll") for (int b_ = 0; b_ < TB; ++b_)                                                         \
+                XN[b_][q_] = *reinterpret_cast<const rt_f4*>(xrow[b_] + (nxt) + 4 * q_);                             \
+            _Pragma("unroll") for (int g_ = 0; g_ < G; ++g_)                                                          \
+                WN[g_][q_] = *reinterpret_cast<const rt_f4*>(wrow[g_] + (nxt) + 4 * q_);                             \
         }                                                                                                            \
         __builtin_amdgcn_sched_barrier(0);                                                                           \
         RT_MFMA(XV, WV, 0); RT_MFMA(XV, WV, 1); RT_MFMA(XV, WV, 2); RT_MFMA(XV, WV, 3);                              \
@@ -186,18 +219,21 @@ __global__ __launch_bounds__(NWV * WAVE) void route_logits_mfma_kernel(const XT*
             const int sh = k0 - min(k0, ks_max);        // where h = k0 sits in the slab
             const int kend = sh + max(min(KC, H - k0), 0);
             if (sh < kend) {
-                rt_f4 xa[2], xb[2], wa[2], wb[2];
+                rt_f4 xa[TB][2], xb[TB][2], wa[G][2], wb[G][2];
 #pragma unroll
                 for (int q = 0; q < VN / 4; ++q) {
-                    xa[q] = *reinterpret_cast<const rt_f4*>(xrow + sh + 4 * q);
-                    wa[q] = *reinterpret_cast<const rt_f4*>(wrow + sh + 4 * q);
+#pragma unroll
+                    for (int b = 0; b < TB; ++b) xa[b][q] = *reinterpret_cast<const rt_f4*>(xrow[b] + sh + 4 * q);
+#pragma unroll
+                    for (int g = 0; g < G; ++g) wa[g][q] = *reinterpret_cast<const rt_f4*>(wrow[g] + sh + 4 * q);
                 }
                 if (sh == 0 && kend == KC) {
-                    // a whole slab: sixteen chunks of straight-line code (the read past the last chunk repeats it)
+                    // a whole slab: NCH chunks of straight-line code (the read past the last chunk repeats it)
 #define RT_PAIR(c) /* chunks c (even) and c + 1 */                                         \
     RT_CHUNK(xa, wa, xb, wb, ((c) + 1) * VN);                                              \
-    RT_CHUNK(xb, wb, xa, wa, ((c) + 2 < 16 ? (c) + 2 : 15) * VN)
-                    RT_PAIR(0); RT_PAIR(2); RT_PAIR(4); RT_PAIR(6); RT_PAIR(8); RT_PAIR(10); RT_PAIR(12); RT_PAIR(14);
+    RT_CHUNK(xb, wb, xa, wa, ((c) + 2 < NCH ? (c) + 2 : NCH - 1) * VN)
+                    RT_PAIR(0); RT_PAIR(2); RT_PAIR(4); RT_PAIR(6);
+                    if constexpr (NCH == 16) { RT_PAIR(8); RT_PAIR(10); RT_PAIR(12); RT_PAIR(14); }
 #undef RT_PAIR
                 } else {
                     for (int kk = sh; kk < kend; kk += 2 * VN) {
@@ -214,14 +250,18 @@ __global__ __launch_bounds__(NWV * WAVE) void route_logits_mfma_kernel(const XT*
 #undef RT_MFMA
 #undef RT_STASH
 #undef RT_FETCH
-    const int e = eb0 + wave * SHAPE + lane % SHAPE;
-    if (e < E) {
-        const float bv = bias ? bias[e] : 0.f;
+    float* out = part + (size_t)seg * T * E;
 #pragma unroll
-        for (int v = 0; v < NACC; ++v) {
-            const int t = t0 + (SHAPE == 16 ? 16 * (v / 4) + 4 * (lane / 16) + v % 4 : 4 * (lane / 4) + v);
-            if (t < T) logits[(size_t)t * E + e] = bias ? __fadd_rn(acc[v], bv) : acc[v];
-        }
+    for (int g = 0; g < G; ++g) {
+        const int e = eb0 + (wave * G + g) * SHAPE + lane % SHAPE;
+        if (e >= E) continue;
+#pragma unroll
+        for (int b = 0; b < TB; ++b)
+#pragma unroll
+            for (int v = 0; v < NACC; ++v) {
+                const int t = t0 + b * RT_TB + (SHAPE == 16 ? 16 * (v / 4) + 4 * (lane / 16) + v % 4 : 4 * (lane / 4) + v);
+                if (t < T) out[(size_t)t * E + e] = acc[b][g][v];
+            }
     }
 }
 
@@ -230,8 +270,10 @@ __global__ __launch_bounds__(NWV * WAVE) void route_logits_mfma_kernel(const XT*
 constexpr int TK_MAXV = 8;  // values per lane -> E <= 8*G
 
 template <int G>
-__global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict__ logits, int32_t* __restrict__ idx,
-                                                         float* __restrict__ gate, int T, int E, int k) {
+__global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict__ part /*[RT_P][T][E]*/,
+                                                         const float* __restrict__ bias, float* __restrict__ logits,
+                                                         int32_t* __restrict__ idx, float* __restrict__ gate, int T, int E,
+                                                         int k) {
     constexpr int TPW = WAVE / G;  // tokens per wave
     const int lane = lane_id();
     const int gl = lane % G;
@@ -246,7 +288,20 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict_
 #pragma unroll
         for (int i = 0; i < TK_MAXV; ++i) {
             const int e = gl + i * G;
-            v[i] = (live && e < E) ? logits[(size_t)t * E + e] : NEG_INF;
+            v[i] = NEG_INF;
+            if (live && e < E) {
+                // the segments' partial sums in segment order, then the bias: this fixes the logit's bits
+                const float* pp = part + (size_t)t * E + e;
+                float s[RT_P];
+#pragma unroll
+                for (int p = 0; p < RT_P; ++p) s[p] = pp[(size_t)p * T * E];
+                float sum = s[0];
+#pragma unroll
+                for (int p = 1; p < RT_P; ++p) sum = __fadd_rn(sum, s[p]);
+                if (bias) sum = __fadd_rn(sum, bias[e]);
+                v[i] = sum;
+                logits[(size_t)t * E + e] = sum;
+            }
         }
         unsigned taken = 0;
         float row_max = 0.f;
@@ -297,26 +352,41 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict_
     }
 }
 
-template <typename XT, int SHAPE>
-void launch_logits_mfma(const XT* x, const XT* w, const float* bias, float* logits, int T, int H, int E, hipStream_t s) {
-    const int gx = ceil_div(T, RT_TB), groups = ceil_div(E, SHAPE);
-    if (groups == 1) route_logits_mfma_kernel<XT, SHAPE, 1><<<dim3(gx, 1), WAVE, 0, s>>>(x, w, bias, logits, T, H, E);
-    else if (groups == 2) route_logits_mfma_kernel<XT, SHAPE, 2><<<dim3(gx, 1), 2 * WAVE, 0, s>>>(x, w, bias, logits, T, H, E);
-    else route_logits_mfma_kernel<XT, SHAPE, 4><<<dim3(gx, ceil_div(groups, 4)), 4 * WAVE, 0, s>>>(x, w, bias, logits, T, H, E);
-}
-
+// Block shapes.  Many tokens: 128 tokens per block and slabs of 64 h, so that every wave runs two chains per group of
+// experts side by side and T / 128 x 8 segments of blocks are resident together (four blocks of this size fit a
+// compute unit's LDS); two waves (one group of four experts each) up to 8 experts, four up to 16; beyond that 16
+// experts per instruction and four or eight waves (64 or 128 experts per block).  Few tokens: 64 tokens per block
+// and one chain per wave, for four times as many waves.
 template <typename XT>
-int launch_logits(const XT* x, const XT* w, const float* bias, float* logits, int T, int H, int E, hipStream_t s) {
-    // 16 experts per instruction when that alone gives every SIMD of the chip a wave, else 4 (four times the waves)
-    if (E > 8 && ceil_div(T, RT_TB) * ceil_div(E, 16) >= 1024) launch_logits_mfma<XT, 16>(x, w, bias, logits, T, H, E, s);
-    else launch_logits_mfma<XT, 4>(x, w, bias, logits, T, H, E, s);
+int launch_logits(const XT* x, const XT* w, float* part, int T, int H, int E, hipStream_t s) {
+    constexpr int CPR = 64 / VecLoad<XT>::N;  // slabs of 64 h
+#define RT_LAUNCH(SHAPEv, TBv, Gv, NWVv, CPRv, gz) \
+    route_logits_mfma_kernel<XT, SHAPEv, TBv, Gv, NWVv, CPRv><<<dim3(RT_P, ceil_div(T, TBv * RT_TB), gz), NWVv * WAVE, 0, s>>>(x, w, part, T, H, E)
+    if (T <= 2048) {
+        if (E <= 4) RT_LAUNCH(4, 1, 1, 1, 16, 1);
+        else if (E <= 8) RT_LAUNCH(4, 1, 1, 2, 16, 1);
+        else if (E <= 64) RT_LAUNCH(4, 1, 1, 4, 16, ceil_div(E, 16));
+        else RT_LAUNCH(16, 1, 1, 4, 16, ceil_div(E, 64));
+    } else {
+        if (E <= 4) RT_LAUNCH(4, 2, 1, 1, CPR, 1);
+        else if (E <= 8) RT_LAUNCH(4, 2, 1, 2, CPR, 1);
+        else if (E <= 16) RT_LAUNCH(4, 2, 1, 4, CPR, 1);
+        else if (E <= 64) RT_LAUNCH(16, 2, 1, 4, CPR, 1);
+        else RT_LAUNCH(16, 2, 1, 8, CPR, ceil_div(E, 128));
+    }
+#undef RT_LAUNCH
     return moe_check_launch("route_logits");
 }
 
 }  // namespace
 
+extern "C" size_t moe_route_workspace_bytes(int T, int E) {
+    return sizeof(float) * (size_t)RT_P * (size_t)(T > 0 ? T : 0) * (size_t)(E > 0 ? E : 0);
+}
+
 extern "C" int moe_route_topk(const void* x, const void* router, const float* bias, int dtype, int T, int H, int E,
-                              int k, float* logits_ws, int32_t* topk_idx, float* topk_gate, moe_stream_t stream) {
+                              int k, float* logits, int32_t* topk_idx, float* topk_gate, void* ws, size_t ws_bytes,
+                              moe_stream_t stream) {
     hipStream_t s = (hipStream_t)stream;
     MOE_REQUIRE(T >= 0 && H > 0 && E > 0, MOE_ERR_INVALID, "route_topk: bad shape T=%d H=%d E=%d", T, H, E);
     MOE_REQUIRE(k >= 1 && k <= E, MOE_ERR_INVALID, "route_topk: topk=%d must be in [1, E=%d]", k, E);
@@ -325,10 +395,12 @@ extern "C" int moe_route_topk(const void* x, const void* router, const float* bi
     MOE_REQUIRE(dtype == MOE_F32 || dtype == MOE_BF16, MOE_ERR_INVALID, "route_topk: dtype %d", dtype);
     MOE_REQUIRE((H * dtype_size(dtype)) % 16 == 0, MOE_ERR_INVALID, "route_topk: rows must be 16-byte multiples (H=%d)", H);
     if (T == 0) return MOE_OK;
-    MOE_REQUIRE(x && router && logits_ws && topk_idx && topk_gate, MOE_ERR_INVALID, "route_topk: null pointer");
-    int rc = dtype == MOE_F32
-                 ? launch_logits<float>((const float*)x, (const float*)router, bias, logits_ws, T, H, E, s)
-                 : launch_logits<bf16_t>((const bf16_t*)x, (const bf16_t*)router, bias, logits_ws, T, H, E, s);
+    MOE_REQUIRE(x && router && logits && topk_idx && topk_gate && ws, MOE_ERR_INVALID, "route_topk: null pointer");
+    MOE_REQUIRE(ws_bytes >= moe_route_workspace_bytes(T, E), MOE_ERR_WORKSPACE, "route_topk: workspace %zu < %zu", ws_bytes,
+                moe_route_workspace_bytes(T, E));
+    float* part = (float*)ws;
+    int rc = dtype == MOE_F32 ? launch_logits<float>((const float*)x, (const float*)router, part, T, H, E, s)
+                              : launch_logits<bf16_t>((const bf16_t*)x, (const bf16_t*)router, part, T, H, E, s);
     if (rc) return rc;
     // lanes per token: the fewest that hold all experts at TK_MAXV per lane (more tokens per wave, fewer shuffles)
     int G = 8;
@@ -338,10 +410,10 @@ extern "C" int moe_route_topk(const void* x, const void* router, const float* bi
     const int waves = ceil_div(T, tpw);
     const int blocks = min(ceil_div(waves, 4), 4096);
     switch (G) {
-        case 8: topk_gate_kernel<8><<<blocks, 256, 0, s>>>(logits_ws, topk_idx, topk_gate, T, E, k); break;
-        case 16: topk_gate_kernel<16><<<blocks, 256, 0, s>>>(logits_ws, topk_idx, topk_gate, T, E, k); break;
-        case 32: topk_gate_kernel<32><<<blocks, 256, 0, s>>>(logits_ws, topk_idx, topk_gate, T, E, k); break;
-        default: topk_gate_kernel<64><<<blocks, 256, 0, s>>>(logits_ws, topk_idx, topk_gate, T, E, k); break;
+        case 8: topk_gate_kernel<8><<<blocks, 256, 0, s>>>(part, bias, logits, topk_idx, topk_gate, T, E, k); break;
+        case 16: topk_gate_kernel<16><<<blocks, 256, 0, s>>>(part, bias, logits, topk_idx, topk_gate, T, E, k); break;
+        case 32: topk_gate_kernel<32><<<blocks, 256, 0, s>>>(part, bias, logits, topk_idx, topk_gate, T, E, k); break;
+        default: topk_gate_kernel<64><<<blocks, 256, 0, s>>>(part, bias, logits, topk_idx, topk_gate, T, E, k); break;
     }
     return moe_check_launch("topk_gate");
 }

@@ -45,8 +45,10 @@ def route_topk(x: torch.Tensor, router: torch.Tensor, topk: int, bias: Optional[
     logits = torch.empty((T, E), dtype=torch.float32, device=dev)
     idx = torch.empty((T, topk), dtype=torch.int32, device=dev)
     gate = torch.empty((T, topk), dtype=torch.float32, device=dev)
+    nbytes = L.lib().moe_route_workspace_bytes(T, E)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=dev)
     L.check(L.lib().moe_route_topk(L.ptr(x), L.ptr(router), L.ptr(bias), L.dtype_code(x.dtype), T, H, E, topk,
-                                   L.ptr(logits), L.ptr(idx), L.ptr(gate), L.stream_ptr()))
+                                   L.ptr(logits), L.ptr(idx), L.ptr(gate), L.ptr(ws), nbytes, L.stream_ptr()))
     return idx, gate, logits
 
 

@@ -45,6 +45,8 @@ class DispatchPipeline:
         self.code = L.dtype_code(dt)
         # source side
         self.logits = torch.empty((T, E), dtype=torch.float32, device=dev)
+        self.route_ws_bytes = lib.moe_route_workspace_bytes(T, E)
+        self.route_ws = torch.empty(max(self.route_ws_bytes, 16), dtype=torch.uint8, device=dev)
         self.idx, self.gate = i32(T, k), torch.empty((T, k), dtype=torch.float32, device=dev)
         self.send_counts, self.expert_offs = i32(W, E_l), i32(W, E_l)
         self.dst_sizes, self.dst_offsets, self.caps = i32(W), i32(W), i32(2)
@@ -79,7 +81,8 @@ class DispatchPipeline:
     def route(self, s):
         c, w = self.cfg, self.world
         L.check(L.lib().moe_route_topk(self._p(w.x0), self._p(w.router), self._p(w.bias), self.code, c.tokens, c.hidden,
-                                       c.experts, c.topk, self._p(self.logits), self._p(self.idx), self._p(self.gate), s))
+                                       c.experts, c.topk, self._p(self.logits), self._p(self.idx), self._p(self.gate),
+                                       self._p(self.route_ws), self.route_ws_bytes, s))
 
     def count(self, s):
         c = self.cfg

@@ -175,11 +175,13 @@ def quantize_cols_fp8(w: np.ndarray) -> Tuple[np.ndarray, np.ndarray]:
 # a1: router  (reference utils.py:200-202)
 # --------------------------------------------------------------------------------------
 def router_logits(x: np.ndarray, w: np.ndarray, bias: Optional[np.ndarray] = None) -> np.ndarray:
-    """logits[t,e] = bias[e] + sum_h x[t,h] w[h,e]: one fp32 fmaf chain per (t,e), ascending h.
+    """logits[t,e] = bias[e] + sum_h x[t,h] w[h,e] in pinned fp32 arithmetic: h in eight contiguous
+    segments of ceil(H/8) rounded up to a multiple of 8, one fmaf chain per segment in ascending h from
+    +0, the eight chains added in segment order, the bias last (see oracle/router_ref.c).
 
-    Restates ``torch.einsum('th,he->te', tokens, router)`` (utils.py:201) with the
-    reduction order pinned (see oracle/router_ref.c).  ``bias`` (per-expert, added to
-    the logits) is the load-skew term of the fine-grained / Zipf workloads.
+    Restates ``torch.einsum('th,he->te', tokens, router)`` (utils.py:201), whose own order is
+    unspecified.  ``bias`` (per-expert, added to the logits) is the load-skew term of the fine-grained /
+    Zipf workloads.
     """
     x = np.ascontiguousarray(x, dtype=np.float32)
     w = np.ascontiguousarray(w, dtype=np.float32)

@@ -7,14 +7,21 @@
  * Restates the matmul inside the reference's router
  *     routed_values = F.softmax(torch.einsum('th,he->te', tokens, router), dim=-1)
  * (reference utils.py:201) with a *specified* fp32 reduction order, so that the
- * top-k indices derived from it can be compared bit-for-bit with the HIP kernel:
+ * top-k indices derived from it can be compared bit-for-bit with the HIP kernel.
+ * h is cut into ROUTE_SEGMENTS = 8 contiguous segments of
+ *     L = ceil(H / 8) rounded up to a multiple of 8
+ * elements (the last ones shorter, or empty when H is small);
  *
- *     logit[t,e] = bias[e] + chain_h( fmaf(x[t,h], w[h,e], acc) ),  h = 0 .. H-1,
+ *     s_p        = chain_h( fmaf(x[t,h], w[h,e], acc) ),  h = p*L .. min((p+1)*L, H) - 1,  acc0 = +0.0f
+ *     logit[t,e] = (((((((s_0 + s_1) + s_2) + s_3) + s_4) + s_5) + s_6) + s_7) + bias[e]
  *
- * i.e. one fused-multiply-add chain per (t,e) in ascending h, starting from
- * +0.0f, every operand widened exactly to fp32 first, and the bias added last
- * with one fp32 addition.  torch's own einsum is free to use any order; this
- * one is fixed so that CPU and GPU agree on every bit.
+ * i.e. eight fused-multiply-add chains per (t,e), each in ascending h and starting
+ * from +0.0f (an empty segment stays +0.0f), every operand widened exactly to fp32
+ * first; the chains are added in segment order with one fp32 addition each, the
+ * bias last.  torch's own einsum is free to use any order; this one is fixed so
+ * that CPU and GPU agree on every bit.  (Eight chains and not one because a chain
+ * is a sequence of dependent instructions: over all of H its length, not memory,
+ * bounds a GPU; the segment count is part of the specification, not a tuning knob.)
  *
  * Build: see oracle/Makefile (gcc -O2 -ffp-contract=off; the fmaf below is
  * either the hardware FMA or libm's correctly-rounded software fmaf, both give
@@ -26,6 +33,9 @@
 #include <string.h>
 
 #define CLONES __attribute__((target_clones("avx2,fma", "default")))
+#define ROUTE_SEGMENTS 8
+
+static inline int segment_len(int H) { return ((H + ROUTE_SEGMENTS - 1) / ROUTE_SEGMENTS + 7) & ~7; }
 
 static inline float bf16_to_f32(uint16_t v) {
     uint32_t u = ((uint32_t)v) << 16;
@@ -40,23 +50,31 @@ int oracle_router_logits_f32(const float* x, const float* w, const float* bias,
                              int T, int H, int E, float* out) {
     if (T < 0 || H < 0 || E <= 0) return -1;
     float* acc = (float*)malloc(sizeof(float) * (size_t)E);
-    if (!acc) return -2;
+    float* sum = (float*)malloc(sizeof(float) * (size_t)E);
+    if (!acc || !sum) { free(acc); free(sum); return -2; }
+    const int L = segment_len(H);
     for (int t = 0; t < T; ++t) {
-        for (int e = 0; e < E; ++e) acc[e] = 0.0f;
         const float* xr = x + (size_t)t * H;
-        for (int h = 0; h < H; ++h) {
-            const float xv = xr[h];
-            const float* wr = w + (size_t)h * E;
-            for (int e = 0; e < E; ++e) acc[e] = __builtin_fmaf(xv, wr[e], acc[e]);
+        for (int p = 0; p < ROUTE_SEGMENTS; ++p) {
+            const int h0 = p * L < H ? p * L : H, h1 = h0 + L < H ? h0 + L : H;
+            for (int e = 0; e < E; ++e) acc[e] = 0.0f;
+            for (int h = h0; h < h1; ++h) {
+                const float xv = xr[h];
+                const float* wr = w + (size_t)h * E;
+                for (int e = 0; e < E; ++e) acc[e] = __builtin_fmaf(xv, wr[e], acc[e]);
+            }
+            if (p == 0) { for (int e = 0; e < E; ++e) sum[e] = acc[e]; }
+            else { for (int e = 0; e < E; ++e) sum[e] = sum[e] + acc[e]; }
         }
         float* o = out + (size_t)t * E;
         if (bias) {
-            for (int e = 0; e < E; ++e) o[e] = acc[e] + bias[e];
+            for (int e = 0; e < E; ++e) o[e] = sum[e] + bias[e];
         } else {
-            for (int e = 0; e < E; ++e) o[e] = acc[e];
+            for (int e = 0; e < E; ++e) o[e] = sum[e];
         }
     }
     free(acc);
+    free(sum);
     return 0;
 }
 
@@ -67,25 +85,33 @@ int oracle_router_logits_bf16(const uint16_t* x, const uint16_t* w, const float*
     if (T < 0 || H < 0 || E <= 0) return -1;
     float* wf = (float*)malloc(sizeof(float) * (size_t)H * (size_t)E);
     float* acc = (float*)malloc(sizeof(float) * (size_t)E);
-    if (!wf || !acc) { free(wf); free(acc); return -2; }
+    float* sum = (float*)malloc(sizeof(float) * (size_t)E);
+    if (!wf || !acc || !sum) { free(wf); free(acc); free(sum); return -2; }
     for (size_t i = 0; i < (size_t)H * (size_t)E; ++i) wf[i] = bf16_to_f32(w[i]);
+    const int L = segment_len(H);
     for (int t = 0; t < T; ++t) {
-        for (int e = 0; e < E; ++e) acc[e] = 0.0f;
         const uint16_t* xr = x + (size_t)t * H;
-        for (int h = 0; h < H; ++h) {
-            const float xv = bf16_to_f32(xr[h]);
-            const float* wr = wf + (size_t)h * E;
-            for (int e = 0; e < E; ++e) acc[e] = __builtin_fmaf(xv, wr[e], acc[e]);
+        for (int p = 0; p < ROUTE_SEGMENTS; ++p) {
+            const int h0 = p * L < H ? p * L : H, h1 = h0 + L < H ? h0 + L : H;
+            for (int e = 0; e < E; ++e) acc[e] = 0.0f;
+            for (int h = h0; h < h1; ++h) {
+                const float xv = bf16_to_f32(xr[h]);
+                const float* wr = wf + (size_t)h * E;
+                for (int e = 0; e < E; ++e) acc[e] = __builtin_fmaf(xv, wr[e], acc[e]);
+            }
+            if (p == 0) { for (int e = 0; e < E; ++e) sum[e] = acc[e]; }
+            else { for (int e = 0; e < E; ++e) sum[e] = sum[e] + acc[e]; }
         }
         float* o = out + (size_t)t * E;
         if (bias) {
-            for (int e = 0; e < E; ++e) o[e] = acc[e] + bias[e];
+            for (int e = 0; e < E; ++e) o[e] = sum[e] + bias[e];
         } else {
-            for (int e = 0; e < E; ++e) o[e] = acc[e];
+            for (int e = 0; e < E; ++e) o[e] = sum[e];
         }
     }
     free(wf);
     free(acc);
+    free(sum);
     return 0;
 }
 

@@ -34,9 +34,9 @@ def test_argument_errors_are_reported_without_a_gpu():
     lib = L.lib()
     rc = lib.moe_count_and_offsets(None, 4, 2, 9, 4, None, None, None, None, None, None, None, None, 0, None)
     assert rc == -1 and b"divisible" in lib.moe_last_error()
-    rc = lib.moe_route_topk(None, None, None, 0, 4, 64, 8, 9, None, None, None, None)
+    rc = lib.moe_route_topk(None, None, None, 0, 4, 64, 8, 9, None, None, None, None, 0, None)
     assert rc == -1 and b"topk" in lib.moe_last_error()
-    rc = lib.moe_route_topk(None, None, None, 1, 4, 60, 8, 2, None, None, None, None)
+    rc = lib.moe_route_topk(None, None, None, 1, 4, 60, 8, 2, None, None, None, None, 0, None)
     assert rc == -1 and b"16-byte" in lib.moe_last_error()
     with pytest.raises(L.MoeLibraryError):
         L.check(lib.moe_pack(None, 7, 1, 64, None, None, None, 4, 4, None, None, None, None))

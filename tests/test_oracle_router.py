@@ -23,22 +23,59 @@ def test_logits_match_float64_dot():
     assert (np.abs(lg - ref) <= bound).all()
 
 
-def test_logits_fixed_order_is_an_fma_chain():
-    # brute force in Python with exact rational arithmetic emulating fmaf: float32(x*w + acc) with the
-    # product and sum exact in float64 for small integers -> catches a swapped/dropped term or a
-    # non-fused multiply
-    rng = np.random.default_rng(3)
-    x = rng.integers(-8, 9, size=(5, 37)).astype(np.float32) / 4
-    w = rng.integers(-8, 9, size=(37, 6)).astype(np.float32) / 8
+def _segmented_chain(x, w, t, e, fma):
+    """The specified order spelled out in Python: eight contiguous segments of ceil(H/8) rounded up to a
+    multiple of 8, a chain per segment from +0, the chains added in segment order."""
+    H = x.shape[1]
+    L = (-(-H // 8) + 7) // 8 * 8
+    total = None
+    for p in range(8):
+        acc = np.float32(0)
+        for h in range(min(p * L, H), min((p + 1) * L, H)):
+            acc = fma(x[t, h], w[h, e], acc)
+        total = acc if total is None else np.float32(total + acc)
+    return total
+
+
+@pytest.mark.parametrize("H", [37, 8, 64, 100, 130])
+def test_logits_fixed_order_is_eight_fma_chains(H):
+    # brute force in Python emulating fmaf: float32(x*w + acc) with the product and the sum exact in
+    # float64 (operands are small integers over 4 and 8, sums stay far below 2^53) -> catches a swapped or
+    # dropped term, a non-fused multiply, a wrong segment boundary or a wrong order of the final additions
+    rng = np.random.default_rng(3 + H)
+    x = rng.integers(-8, 9, size=(5, H)).astype(np.float32) / 4
+    w = rng.integers(-8, 9, size=(H, 6)).astype(np.float32) / 8
     lg = O.router_logits(x, w)
-    want = np.zeros((5, 6), np.float32)
-    for t in range(5):
-        for e in range(6):
-            acc = np.float32(0)
-            for h in range(37):
-                acc = np.float32(np.float64(x[t, h]) * np.float64(w[h, e]) + np.float64(acc))
-            want[t, e] = acc
+    fma = lambda a, b, c: np.float32(np.float64(a) * np.float64(b) + np.float64(c))  # noqa: E731
+    want = np.array([[_segmented_chain(x, w, t, e, fma) for e in range(6)] for t in range(5)], np.float32)
     assert np.array_equal(lg.view(np.uint32), want.view(np.uint32))
+
+
+def test_segment_sums_are_added_in_segment_order_with_fp32_rounding():
+    # H = 64 -> eight segments of 8.  Segment sums 2^24, 1, 1, -2^24, 0...: in fp32, in segment order,
+    # ((2^24 + 1) + 1) - 2^24 = 0 (each +1 is rounded away); any other association, or a wider accumulator,
+    # gives 1 or 2.  A single chain over all of H would give 0 + ... as well only by accident: it is
+    # excluded by the next case, where the order inside a segment matters instead.
+    x = np.zeros((1, 64), np.float32)
+    w = np.ones((64, 1), np.float32)
+    x[0, 0], x[0, 8], x[0, 16], x[0, 24] = 2.0 ** 24, 1.0, 1.0, -2.0 ** 24
+    assert O.router_logits(x, w)[0, 0] == 0.0
+    # the same four values inside ONE segment in the order 2^24, -2^24, 1, 1 give 2: chains run in ascending h
+    x = np.zeros((1, 64), np.float32)
+    x[0, 0], x[0, 1], x[0, 2], x[0, 3] = 2.0 ** 24, -2.0 ** 24, 1.0, 1.0
+    assert O.router_logits(x, w)[0, 0] == 2.0
+    # segments 1 and 2 hold 1 and 1, segment 0 holds 2^24 and segment 3 -2^24, bias 0.5 last: (0 + 0.5)
+    x = np.zeros((1, 64), np.float32)
+    x[0, 7], x[0, 15], x[0, 23], x[0, 31] = 2.0 ** 24, 1.0, 1.0, -2.0 ** 24
+    assert O.router_logits(x, w, np.array([0.5], np.float32))[0, 0] == 0.5
+    # boundaries: with H = 100 the segments are 16 long (ceil(100/8) = 13 -> 16): h = 15 and h = 16 lie in
+    # different segments, h = 96..99 form the seventh, the eighth is empty
+    x = np.zeros((1, 100), np.float32)
+    w = np.ones((100, 1), np.float32)
+    x[0, 15], x[0, 16], x[0, 17] = 2.0 ** 24, 1.0, -2.0 ** 24   # (2^24) + (1 - 2^24 -> -2^24 + 1 = exact) ...
+    # segment 0 sum = 2^24; segment 1 chain: fma(1,1,0) = 1, then fma(-2^24,1,1) = -2^24 + 1 = -16777215 (exact)
+    # total = 2^24 + (-16777215) = 1; a single chain would give (2^24 + 1 -> 2^24) - 2^24 = 0
+    assert O.router_logits(x, w)[0, 0] == 1.0
 
 
 def test_fma_is_fused():
