@@ -248,6 +248,36 @@ int moe_grouped_mlp_fp8_mapped(const void* a_base_bf16, int a_rows, const int32_
                                const float* sd, uint8_t* xq_ws, float* xs_ws, void* h_ws, uint8_t* hq_ws, float* hs_ws,
                                void* out, int out_rows, const int32_t* c_row_map, moe_stream_t stream);
 
+/* ---- gradients (every backward of the reference is an empty stub: layers/expert.py:62-64,
+ * layers/token_shuffle.py:58-60, layers/all_to_all.py:121-123) -----------------------------------------------------
+ * For out[rows of g] = x[rows of g] @ w[g]:
+ *   d x[rows of g] = d out[rows of g] @ w[g]^T : moe_grouped_gemm_mapped on weights re-tiled by
+ *                    moe_prepack_weights_transposed (moe_prepack_bytes(dtype, E_l, N, K) bytes; with w_up the pair
+ *                    (w, w_up) is transposed together in the fused gate/up column order, N = columns of ONE matrix,
+ *                    twice the bytes); fp32: moe_transpose_weights_f32 then moe_grouped_gemm.
+ *   d w[g]         = x[rows of g]^T @ d out[rows of g] : moe_grouped_gemm_dw, one launch for all groups, the ragged row
+ *                    count being the reduction dimension (both operands are first rewritten row-index-fastest, every
+ *                    group padded to a multiple of 64 rows with zeros, into ws of moe_dw_workspace_bytes bytes);
+ *                    groups without rows get zeros.  split_F > 0 (bf16): dy is [S_rows, 2 split_F] in the fused
+ *                    gate/up column order and dw comes out as [E_l, K, 2 split_F] = [d w_gate | d w_up] side by side.
+ * moe_mlp_act_backward: gradient through the activation of the expert MLP; a1 = pre-activations ([rows,F]; SwiGLU:
+ *   [rows,2F] in the fused gate/up column order, as moe_grouped_gemm_mapped produces them with MOE_ACT_NONE), dh [rows,F],
+ *   d_a1 in the layout of a1.
+ * moe_combine_backward: d ret[slot(t,kk)] = gate[t,kk] * d out[t] (padding slots zeroed, like the pack) and
+ *   d gate[t,kk] = <d out[t], ret[slot(t,kk)]>.  The gradient of the fixed-M pack is moe_combine with unit gates; that of
+ *   the expert-major unpack is moe_return_pack, and the other way round; moe_shuffle_backward is declared above. */
+int moe_prepack_weights_transposed(const void* w, const void* w_up, int dtype, int E_l, int K, int N, void* packed,
+                                   moe_stream_t stream);
+size_t moe_dw_workspace_bytes(int S_rows, int E_l, int K, int N);
+int moe_grouped_gemm_dw(const void* x, const void* dy, const int32_t* expert_cnt, int dtype, int S_rows, int K, int N,
+                        int E_l, int split_F, void* dw, void* ws, size_t ws_bytes, moe_stream_t stream);
+int moe_transpose_weights_f32(const float* w, int E_l, int K, int N, float* out, moe_stream_t stream);
+int moe_mlp_act_backward(const void* a1, const void* dh, int dtype, int rows, int F, int act, void* d_a1,
+                         moe_stream_t stream);
+int moe_combine_backward(const void* d_out, const void* ret, int dtype, int W, int M, int H, const int32_t* topk_idx,
+                         const int32_t* pos, const float* gate, const int32_t* dst_sizes, const int32_t* dst_offsets, int T,
+                         int k, int E_l, void* d_ret, float* d_gate, moe_stream_t stream);
+
 /* ---- a13: return path and combine (not in the reference; defined by the task statement) -------
  * ret[s, expert_offs_s[e]+j, :] = y[off[e,s]+j, :], zero padding: the [W,M,H] buffer this rank
  * sends back, slot s in the order source s sent its rows. */

@@ -61,6 +61,12 @@ _SIGNATURES = {
     "moe_recv_row_map": (c_int, [P, c_int, c_int, c_int, c_int, P, P, P, P]),
     "moe_grouped_gemm_mapped": (c_int, [P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P, c_int, P, P, c_size_t, P]),
     "moe_gemm_part_workspace_bytes": (c_size_t, []),
+    "moe_prepack_weights_transposed": (c_int, [P, P, c_int, c_int, c_int, c_int, P, P]),
+    "moe_dw_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "moe_grouped_gemm_dw": (c_int, [P, P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, P, c_size_t, P]),
+    "moe_transpose_weights_f32": (c_int, [P, c_int, c_int, c_int, P, P]),
+    "moe_mlp_act_backward": (c_int, [P, P, c_int, c_int, c_int, c_int, P, P]),
+    "moe_combine_backward": (c_int, [P, P, c_int, c_int, c_int, c_int, P, P, P, P, P, c_int, c_int, c_int, P, P, P]),
     "moe_gemm_split_plan": (c_int, [c_int, c_int, c_int, c_int, P]),
     "moe_zero_padding_rows": (c_int, [P, c_int, c_int, c_int, c_int, P, c_int, P]),
     "moe_grouped_mlp_fp8_mapped": (c_int, [P, c_int, P, P, c_int, c_int, c_int, c_int, P, P, P, P, P, P, P, P, P, P, P, c_int, P, P]),

@@ -502,31 +502,95 @@ __global__ __launch_bounds__(WPB * WAVE) void combine_kernel(const uint4* __rest
                 if (!have[j] && status && lane == 0) *status = 1;
             }
         }
-#pragma unroll 2
-        for (int c = lane; c < row_vec; c += WAVE) {
-            uint4 v[KMAX];
+        // U columns per lane and pass, so that sixteen 16-byte row reads are in flight per lane whatever k is
+        constexpr int U = KT ? (KT >= 16 ? 1 : 16 / KT) : 1;
+        for (int c0 = lane; c0 < row_vec; c0 += U * WAVE) {
+            uint4 v[U][KMAX];
 #pragma unroll
-            for (int j = 0; j < KMAX; ++j)
-                if (j < k && have[j]) {
-                    // every returned row is read once: no cache retention wanted
-                    const u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(ret + rows[j] + c));
-                    v[j] = make_uint4(raw.x, raw.y, raw.z, raw.w);
+            for (int u = 0; u < U; ++u) {
+                const int c = c0 + u * WAVE;
+#pragma unroll
+                for (int j = 0; j < KMAX; ++j)
+                    if (j < k && have[j] && c < row_vec) {
+                        // every returned row is read once: no cache retention wanted
+                        const u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(ret + rows[j] + c));
+                        v[u][j] = make_uint4(raw.x, raw.y, raw.z, raw.w);
+                    }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int c = c0 + u * WAVE;
+                if (c >= row_vec) break;
+                float acc[N];
+#pragma unroll
+                for (int i = 0; i < N; ++i) acc[i] = 0.f;
+#pragma unroll
+                for (int j = 0; j < KMAX; ++j) {
+                    if (j < k && have[j]) {
+                        float f[N];
+                        Vec16<XT>::unpack(v[u][j], f);
+#pragma unroll
+                        for (int i = 0; i < N; ++i) acc[i] = __fadd_rn(acc[i], __fmul_rn(g[j], f[i]));
+                    }
                 }
-            float acc[N];
+                const uint4 o = Vec16<XT>::pack(acc);
+                const u32x4 ov = {o.x, o.y, o.z, o.w};
+                __builtin_nontemporal_store(ov, reinterpret_cast<u32x4*>(out + (size_t)t * row_vec + c));
+            }
+        }
+    }
+}
+
+// ---- gradient of the combine: out[t] = sum_kk gate[t,kk] * ret[slot(t,kk)] ------------------------------------------
+//   d ret[slot(t,kk)] = gate[t,kk] * d out[t]        (every slot belongs to one (t,kk): a scatter, like the pack)
+//   d gate[t,kk]      = < d out[t], ret[slot(t,kk)] > (fp32 sum over the row: per-lane partial sums in column order, then
+//                                                     a butterfly over the lanes -- reproducible from call to call)
+// Rows [0, T) of the launch are tokens (one wave each); rows [T, T + W*M) are the slots of d ret, which only get zeros when
+// they are padding (no (t,kk) maps there) -- as in pack_tokens_kernel.  Dropped slots (outside [W,M]) get no gradient.
+template <typename XT, int WPB>
+__global__ __launch_bounds__(WPB * WAVE) void combine_backward_kernel(const uint4* __restrict__ dout, const uint4* __restrict__ ret,
+                                                                       const int32_t* __restrict__ idx, const int32_t* __restrict__ pos,
+                                                                       const float* __restrict__ gate,
+                                                                       const int32_t* __restrict__ dst_sizes,
+                                                                       const int32_t* __restrict__ dst_offsets, int T, int k, int E_l,
+                                                                       int W, int M, int row_vec, uint4* __restrict__ dret,
+                                                                       float* __restrict__ dgate) {
+    constexpr int N = Vec16<XT>::N;
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const int n_rows = T + W * M;
+    for (int r = blockIdx.x * WPB + wave; r < n_rows; r += gridDim.x * WPB) {
+        if (r >= T) {
+            const int d = (r - T) / M, m = (r - T) % M;
+            if (m < dst_sizes[d]) continue;
+            uint4* o = dret + (size_t)(r - T) * row_vec;
+            for (int c = lane; c < row_vec; c += WAVE) o[c] = make_uint4(0, 0, 0, 0);
+            continue;
+        }
+        const uint4* drow = dout + (size_t)r * row_vec;
+        for (int j = 0; j < k; ++j) {
+            const int d = idx[(size_t)r * k + j] / E_l;
+            const bool d_ok = (unsigned)d < (unsigned)W;
+            const int m = pos[(size_t)r * k + j] - dst_offsets[d_ok ? d : 0];
+            const bool have = d_ok && (unsigned)m < (unsigned)M;
+            const float g = gate[(size_t)r * k + j];
+            float dot = 0.f;
+            if (have) {
+                const size_t slot = ((size_t)d * M + m) * row_vec;
+                for (int c = lane; c < row_vec; c += WAVE) {
+                    float dv[N], rv[N], ov[N];
+                    Vec16<XT>::unpack(drow[c], dv);
+                    Vec16<XT>::unpack(ret[slot + c], rv);
 #pragma unroll
-            for (int i = 0; i < N; ++i) acc[i] = 0.f;
-#pragma unroll
-            for (int j = 0; j < KMAX; ++j) {
-                if (j < k && have[j]) {
-                    float f[N];
-                    Vec16<XT>::unpack(v[j], f);
-#pragma unroll
-                    for (int i = 0; i < N; ++i) acc[i] = __fadd_rn(acc[i], __fmul_rn(g[j], f[i]));
+                    for (int i = 0; i < N; ++i) {
+                        dot = __fadd_rn(dot, __fmul_rn(dv[i], rv[i]));
+                        ov[i] = __fmul_rn(g, dv[i]);
+                    }
+                    dret[slot + c] = Vec16<XT>::pack(ov);
                 }
             }
-            const uint4 o = Vec16<XT>::pack(acc);
-            const u32x4 ov = {o.x, o.y, o.z, o.w};
-            __builtin_nontemporal_store(ov, reinterpret_cast<u32x4*>(out + (size_t)t * row_vec + c));
+#pragma unroll
+            for (int off = WAVE / 2; off >= 1; off >>= 1) dot = __fadd_rn(dot, __shfl_xor(dot, off, WAVE));
+            if (lane == 0) dgate[(size_t)r * k + j] = dot;
         }
     }
 }
@@ -874,6 +938,29 @@ extern "C" int moe_return_pack(const void* y, int dtype, int S_rows, int H, cons
     MOE_REQUIRE((long long)W * M < (1ll << 31), MOE_ERR_UNSUPPORTED, "return_pack: W*M too large");
     return recv_driven("return_pack", SRC_RETURN, y, ret, dtype, H, recv_counts, W, E_l, M, 1, W * M, nullptr, nullptr, map_ws,
                        nullptr, (hipStream_t)stream);
+}
+
+extern "C" int moe_combine_backward(const void* d_out, const void* ret, int dtype, int W, int M, int H, const int32_t* topk_idx,
+                                    const int32_t* pos, const float* gate, const int32_t* dst_sizes, const int32_t* dst_offsets,
+                                    int T, int k, int E_l, void* d_ret, float* d_gate, moe_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    int rc = check_rows("combine_backward", dtype, H);
+    if (rc) return rc;
+    MOE_REQUIRE(W > 0 && M >= 1 && T >= 0 && E_l > 0, MOE_ERR_INVALID, "combine_backward: bad shape");
+    MOE_REQUIRE(k >= 1 && k <= MOE_MAX_TOPK, MOE_ERR_UNSUPPORTED, "combine_backward: topk=%d outside [1,%d]", k, MOE_MAX_TOPK);
+    MOE_REQUIRE((long long)W * M + T < (1ll << 31), MOE_ERR_UNSUPPORTED, "combine_backward: W*M + T too large");
+    MOE_REQUIRE(d_ret && dst_sizes && dst_offsets, MOE_ERR_INVALID, "combine_backward: null pointer");
+    MOE_REQUIRE(T == 0 || (d_out && ret && topk_idx && pos && gate && d_gate), MOE_ERR_INVALID, "combine_backward: null pointer");
+    const int n_rows = T + W * M;
+    const int blocks = min(ceil_div(n_rows, 4), 65535 * 8);
+    const int row_vec = H * dtype_size(dtype) / 16;
+    if (dtype == MOE_F32)
+        combine_backward_kernel<float, 4><<<blocks, 4 * WAVE, 0, s>>>((const uint4*)d_out, (const uint4*)ret, topk_idx, pos, gate, dst_sizes,
+                                                                      dst_offsets, T, k, E_l, W, M, row_vec, (uint4*)d_ret, d_gate);
+    else
+        combine_backward_kernel<bf16_t, 4><<<blocks, 4 * WAVE, 0, s>>>((const uint4*)d_out, (const uint4*)ret, topk_idx, pos, gate, dst_sizes,
+                                                                       dst_offsets, T, k, E_l, W, M, row_vec, (uint4*)d_ret, d_gate);
+    return moe_check_launch("combine_backward");
 }
 
 extern "C" int moe_combine(const void* ret, int dtype, int W, int M, int H, const int32_t* topk_idx, const int32_t* pos,

@@ -55,6 +55,13 @@ struct GemmParams {
     // kernel adds the parts of a tile in part order and applies the epilogue.  NULL: no split.
     float* part_ws;
     int max_units;
+    // Weight-gradient mode (template flag DW): C[g] (dw_rows x N, at C + g * c_group_stride elements) = A_g^T-like product
+    // whose reduction runs over the rows of group g.  A is then the TRANSPOSED activation matrix [dw_rows, K] with
+    // K = the padded row total (every group's rows padded to a multiple of 64, zero filled), B the output gradients
+    // re-tiled like weights over the same padded rows; group g owns K stages [kstart_g, kstart_g + 2 ceil(cnt_g / 64)).
+    int dw_rows;
+    int dw_src_rows;  // rows of the untransposed operands: the counts are clamped to it, as the operand kernels clamp them
+    size_t c_group_stride;
 };
 
 constexpr int GG_MAX_PARTS = 16;   // parts per tile at most
@@ -131,10 +138,13 @@ struct GgTile {
 };
 
 // lin -> tile: group-major, 16-row bands, 16-column super-columns (see the XCD-aware walk above)
-template <int BM>
-__device__ __forceinline__ GgTile gg_decode(const int* g_tile_start, const int* g_row_start, int E_l, int Nt, int S_rows, int lin) {
+// DW (weight-gradient mode): every non-empty group has the same ceil(dw_rows / BM) x Nt tiles, rows [0, dw_rows) of its own
+// output matrix; g_row_start then holds the groups' first K stages (set by the caller from it).
+template <int BM, bool DW = false>
+__device__ __forceinline__ GgTile gg_decode(const int* g_tile_start, const int* g_row_start, int E_l, int Nt, int S_rows, int lin,
+                                            int dw_rows = 0) {
     const int g = seg_of(g_tile_start, E_l + 1, lin);
-    const int cnt_g = g_row_start[g + 1] - g_row_start[g];
+    const int cnt_g = DW ? dw_rows : g_row_start[g + 1] - g_row_start[g];
     const int Mt = (cnt_g + BM - 1) / BM;
     const int idx = lin - g_tile_start[g];
     const int band = idx / (SUP * Nt), rem = idx % (SUP * Nt);
@@ -145,17 +155,17 @@ __device__ __forceinline__ GgTile gg_decode(const int* g_tile_start, const int* 
     GgTile t;
     t.g = g;
     t.nt = sc * SUP + rem2 % wc;
-    t.row0 = g_row_start[g] + mt * BM;
-    t.rv = min(min(BM, cnt_g - mt * BM), S_rows - t.row0);
+    t.row0 = (DW ? 0 : g_row_start[g]) + mt * BM;
+    t.rv = DW ? min(BM, cnt_g - mt * BM) : min(min(BM, cnt_g - mt * BM), S_rows - t.row0);
     return t;
 }
 
 // next non-empty tile of this workgroup at or after round `base` (base is advanced past it)
 // SPLIT = false walks the whole tiles [0, full); SPLIT = true walks the parts of the tiles [full, total): unit q
 // is part q % P of tile full + q / P.
-template <int BM, bool SPLIT>
+template <int BM, bool SPLIT, bool DW = false>
 __device__ __forceinline__ GgTile gg_next_tile(const int* g_tile_start, const int* g_row_start, int E_l, int Nt, int S_rows,
-                                               const GgPlan& pl, int nk, int my, int stride, int& base) {
+                                               const GgPlan& pl, int nk, int my, int stride, int& base, int dw_rows = 0) {
     GgTile t;
     t.g = t.nt = t.row0 = 0;
     t.rv = 0;
@@ -165,8 +175,12 @@ __device__ __forceinline__ GgTile gg_next_tile(const int* g_tile_start, const in
         const int lin = base + my;
         base += stride;
         if (lin < n) {
-            t = gg_decode<BM>(g_tile_start, g_row_start, E_l, Nt, S_rows, SPLIT ? pl.full + lin / pl.P : lin);
+            t = gg_decode<BM, DW>(g_tile_start, g_row_start, E_l, Nt, S_rows, SPLIT ? pl.full + lin / pl.P : lin, dw_rows);
             t.ks0 = 0; t.nks = nk; t.unit = -1;
+            if constexpr (DW) {
+                t.ks0 = g_row_start[t.g];
+                t.nks = g_row_start[t.g + 1] - t.ks0;
+            }
             if constexpr (SPLIT) {
                 t.ks0 = (lin % pl.P) * pl.nkp;
                 t.nks = min(pl.nkp, nk - t.ks0);
@@ -221,8 +235,10 @@ __device__ __forceinline__ void gg_wait() {
 // blocks of MFMA work to land.
 // SPLIT = false: the launch that takes whole tiles.  SPLIT = true: the launch that takes the tiles of an
 // under-filled last round in parts of the K range and leaves fp32 partial sums in the workspace (GemmParams).
-template <int BM, int NWM, int EPI, bool FP8, bool SPLIT>
+template <int BM, int NWM, int EPI, bool FP8, bool SPLIT, bool DW = false>
 __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const GemmParams p) {
+    static_assert(!DW || (!SPLIT && !FP8 && EPI == EPI_NONE), "the weight-gradient mode is a plain bf16 GEMM");
+    constexpr bool VARK = SPLIT || DW;  // the K range differs from tile to tile
     constexpr int BN = GG_BN;
     constexpr int ES = FP8 ? 1 : 2;
     constexpr int NW = NWM * 2;                        // waves per workgroup
@@ -263,19 +279,28 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 
     if (tid == 0) {
         int ts = 0, rs = 0;
+        [[maybe_unused]] int dw_seen = 0;
         for (int g = 0; g < p.E_l; ++g) {
             g_tile_start[g] = ts;
             g_row_start[g] = rs;
-            const int c = max(p.cnt[g], 0);
-            ts += ((c + BM - 1) / BM) * Nt;
-            rs += c;
+            int c = max(p.cnt[g], 0);
+            if constexpr (DW) {
+                // tiles of the group's own dw_rows x N output; its K stages: the rows padded to 64 (two stages of 32)
+                c = min(c, max(p.dw_src_rows - dw_seen, 0));
+                dw_seen += c;
+                ts += c > 0 ? ((p.dw_rows + BM - 1) / BM) * Nt : 0;
+                rs += ((c + 63) / 64) * 2;
+            } else {
+                ts += ((c + BM - 1) / BM) * Nt;
+                rs += c;
+            }
         }
         g_tile_start[p.E_l] = ts;
         g_row_start[p.E_l] = rs;
     }
     __syncthreads();
     const int nk = (p.K * ES) / ROWB;  // ring stages per tile; even (K * ES is a multiple of 2 * ROWB)
-    const GgPlan plan = gg_plan(g_tile_start[p.E_l], (int)gridDim.x, nk, p.part_ws != nullptr, p.max_units);
+    const GgPlan plan = gg_plan(g_tile_start[p.E_l], (int)gridDim.x, nk, !DW && p.part_ws != nullptr, p.max_units);
     if (SPLIT && plan.P == 1) return;  // nothing was left over for this launch
 
     // XCD-aware position inside a round of gridDim.x tiles: workgroups b, b+8, b+16, ... share an L2.
@@ -308,7 +333,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 
 #define GG_TILE_PTRS(t, Ab_, Bb_, aoff_)                                                                   \
     const uint8_t* Ab_ = (p.a_map ? p.A : p.A + (size_t)(t).row0 * p.K * ES) + (size_t)(t).ks0 * ROWB;      \
-    const uint8_t* Bb_ = p.B + (size_t)(t).g * p.Npad * p.K * ES + (size_t)(t).nt * BN * ROWB + (size_t)(t).ks0 * b_slab; \
+    const uint8_t* Bb_ = p.B + (DW ? (size_t)0 : (size_t)(t).g * p.Npad * p.K * ES) + (size_t)(t).nt * BN * ROWB + (size_t)(t).ks0 * b_slab; \
     uint32_t aoff_[RA];                                                                                     \
     const int ln_ = gg_lane_now();  /* lrow and lchunk again, derived per tile */                              \
     const int lrow_ = wave_s * WROWS + (ln_ >> 2);                                                            \
@@ -352,7 +377,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     } while (0)
 
     int base = 0;
-    GgTile cur = gg_next_tile<BM, SPLIT>(g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, plan, nk, my, gridDim.x, base);
+    GgTile cur = gg_next_tile<BM, SPLIT, DW>(g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, plan, nk, my, gridDim.x, base, p.dw_rows);
     uint32_t a_off[RA];
     const uint8_t *Ab = p.A, *Bb = p.B;
     if (cur.rv > 0) {
@@ -361,12 +386,12 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         Bb = Bb0;
 #pragma unroll
         for (int r = 0; r < RA; ++r) a_off[r] = a_off0[r];
-        GG_PROLOGUE(Ab, Bb, a_off, (SPLIT ? cur.nks : nk));
+        GG_PROLOGUE(Ab, Bb, a_off, (VARK ? cur.nks : nk));
     }
     while (cur.rv > 0) {
         const int g = __builtin_amdgcn_readfirstlane(cur.g), nt = __builtin_amdgcn_readfirstlane(cur.nt);
         const int row0 = __builtin_amdgcn_readfirstlane(cur.row0), rv = __builtin_amdgcn_readfirstlane(cur.rv);
-        const int nks = SPLIT ? __builtin_amdgcn_readfirstlane(cur.nks) : nk;
+        const int nks = VARK ? __builtin_amdgcn_readfirstlane(cur.nks) : nk;
         const int unit = SPLIT ? __builtin_amdgcn_readfirstlane(cur.unit) : -1;
 
         typedef typename std::conditional<FP8, floatx16, floatx4>::type acc_t;
@@ -467,11 +492,11 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 
         // ---- next tile: decode it and request its first stages now (every slot is free once all waves
         // have passed the barrier: the last fragments of this tile are already in registers)
-        const GgTile nxt = gg_next_tile<BM, SPLIT>(g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, plan, nk, my, gridDim.x, base);
+        const GgTile nxt = gg_next_tile<BM, SPLIT, DW>(g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, plan, nk, my, gridDim.x, base, p.dw_rows);
         GG_TILE_PTRS(nxt, Ab_n, Bb_n, a_off_n);
         if (nxt.rv > 0) {
             __syncthreads();
-            GG_PROLOGUE(Ab_n, Bb_n, a_off_n, (SPLIT ? nxt.nks : nk));
+            GG_PROLOGUE(Ab_n, Bb_n, a_off_n, (VARK ? nxt.nks : nk));
         }
 
         // ---- a part of a tile: its fp32 partial sums go to the workspace as they are (tile row major, 256
@@ -531,7 +556,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             if constexpr (FP8) rs[i] = p.row_scale[grow];
             const int crow_i = p.c_map ? p.c_map[grow] : 0;
             ok[i] = ok[i] && crow_i >= 0;  // a negative map entry: the row has no place in the output
-            crow[i] = C + (p.c_map ? (size_t)max(crow_i, 0) : grow) * p.ldc;
+            crow[i] = C + (p.c_map ? (size_t)max(crow_i, 0) : grow) * p.ldc + (DW ? (size_t)g * p.c_group_stride : (size_t)0);
         }
         float4 sc0[NQ], sc1[NQ];  // fp8: channel scales of the lane's columns (gate / only; up)
 #pragma unroll
@@ -916,6 +941,203 @@ __global__ __launch_bounds__(256) void quantize_rows_fp8_kernel(const bf16_t* __
     }
 }
 
+// ---- backward pass helpers -----------------------------------------------------------------------------------------
+// Re-tiling of w [E_l,K,N] as the weights of the TRANSPOSED product (d tokens = d out @ w^T: reduction over N, K output
+// columns): out[e][n / SK][k][n % SK] = w[e][k][n], rows k in [K, Kpad) zero.  No transposition is involved: the 64-byte
+// runs of n are contiguous on both sides.  With w_up the slabs alternate (32 n of w, 32 n of w_up, ...), which is the
+// column order of the fused gate/up product, so the same call serves d tokens = [d gate | d up] @ [w_gate | w_up]^T.
+template <typename T>
+__global__ __launch_bounds__(256) void prepack_t_kernel(const T* __restrict__ w, const T* __restrict__ w_up, T* __restrict__ out,
+                                                         int K, int N, int Kpad) {
+    constexpr int SK = ROWB / (int)sizeof(T);
+    constexpr int VPS = ROWB / 16;  // 16-byte vectors per 64-byte run
+    const int e = blockIdx.y;
+    const int nsl = N / SK, passes = w_up ? 2 : 1;
+    const size_t total = (size_t)nsl * passes * Kpad * VPS;
+    const uint4 z = make_uint4(0, 0, 0, 0);
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const int v = (int)(i % VPS);
+        const int k = (int)((i / VPS) % Kpad);
+        const int slab = (int)(i / ((size_t)VPS * Kpad));  // output slab: (n / SK) * passes + pass
+        const int ns = slab / passes, pass = slab % passes;
+        const T* src = (pass ? w_up : w) + (size_t)e * K * N;
+        uint4 val = z;
+        if (k < K) val = *reinterpret_cast<const uint4*>(src + (size_t)k * N + (size_t)ns * SK + v * (16 / (int)sizeof(T)));
+        *reinterpret_cast<uint4*>(out + (((size_t)e * nsl * passes + slab) * Kpad + k) * SK + v * (16 / (int)sizeof(T))) = val;
+    }
+}
+
+// Operands of the weight-gradient product d w[g] = x_g^T @ dy_g, whose reduction runs over the rows of group g: both
+// matrices are needed with the row index fastest.  Rows are renumbered s -> s' so that every group starts at a
+// multiple of 64 (two K stages of the GEMM) and its tail up to the next multiple of 64 is zero.  A block moves 64 rows
+// (one group's, never two) x 64 columns through LDS.
+//   SLAB = false: out = x^T, [cols, ld_out] row-major                       (the GEMM's activation operand)
+//   SLAB = true : out = the weight layout over the padded rows, [ld_out / SK][Npad][SK]  (the GEMM's weight operand)
+//                with split_F > 0 the input columns are in the fused gate/up order (32 gate, 32 up, ...) and leave in
+//                the order [all gate | all up], so that the product's columns are the two weight gradients side by side
+template <bool SLAB>
+__global__ __launch_bounds__(256) void dw_operand_kernel(const uint16_t* __restrict__ in, const int32_t* __restrict__ cnt, int E_l,
+                                                          int S_rows, int cols, uint16_t* __restrict__ out, int ld_out, int Npad,
+                                                          int split_F) {
+    __shared__ uint16_t tile[64][64 + 2];
+    __shared__ int s_src0, s_valid;
+    if (threadIdx.x == 0) {
+        // padded block blockIdx.y -> (first source row, valid rows); blocks past the padded total have nothing to do
+        int pb = 0, rs = 0, src0 = -1, valid = 0;
+        for (int g = 0; g < E_l; ++g) {
+            const int c = min(max(cnt[g], 0), max(S_rows - rs, 0));
+            const int nb = (c + 63) / 64;
+            if ((int)blockIdx.y < pb + nb) {
+                const int j = blockIdx.y - pb;
+                src0 = rs + j * 64;
+                valid = min(64, c - j * 64);
+                break;
+            }
+            pb += nb;
+            rs += c;
+        }
+        s_src0 = src0;
+        s_valid = valid;
+    }
+    __syncthreads();
+    const int src0 = s_src0, valid = s_valid;
+    if (src0 < 0) return;
+    const int c0 = blockIdx.x * 64;
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int r = i / 64, c = i % 64;
+        tile[r][c] = (r < valid && c0 + c < cols) ? in[(size_t)(src0 + r) * cols + c0 + c] : (uint16_t)0;
+    }
+    __syncthreads();
+    const int sp0 = blockIdx.y * 64;  // first padded row of the block
+    constexpr int SK = ROWB / 2;
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int c = i / 64, r = i % 64;  // consecutive threads walk the rows: contiguous in both output layouts
+        if (c0 + c >= (SLAB ? Npad : cols)) continue;
+        const uint16_t v = tile[r][c];  // (columns in [cols, Npad) were loaded as zeros)
+        const int sp = sp0 + r;
+        if constexpr (SLAB) {
+            int oc = c0 + c;
+            if (split_F > 0 && oc < 2 * split_F) oc = ((oc % 64) / 32) * split_F + (oc / 64) * 32 + oc % 32;
+            out[((size_t)(sp / SK) * Npad + oc) * SK + sp % SK] = v;
+        } else {
+            out[(size_t)(c0 + c) * ld_out + sp] = v;
+        }
+    }
+}
+
+// d w[g] <- 0 for the groups that received no row (the GEMM has no tile for them)
+__global__ __launch_bounds__(256) void dw_zero_empty_kernel(uint4* __restrict__ dw, const int32_t* __restrict__ cnt,
+                                                             size_t vec_per_group, int src_rows) {
+    // (a group whose rows all lie past the end of the operands counts as empty, as in the GEMM's own tables)
+    int before = 0;
+    for (int e = 0; e < (int)blockIdx.y; ++e) before += max(cnt[e], 0);
+    if (min(max(cnt[blockIdx.y], 0), max(src_rows - before, 0)) > 0) return;
+    uint4* d = dw + (size_t)blockIdx.y * vec_per_group;
+    const uint4 z = make_uint4(0, 0, 0, 0);
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < vec_per_group; i += (size_t)gridDim.x * blockDim.x) d[i] = z;
+}
+
+// Gradient through the activation of the expert MLP.  a1: the pre-activations as the first GEMM produces them without an
+// epilogue ([rows, F] for GELU / SiLU; [rows, 2F] in the fused gate/up column order -- 32 gate columns, their 32 up
+// columns, ... -- for SwiGLU); dh: gradient of the hidden activation [rows, F]; out: gradient of a1, same layout as a1.
+//   GELU (erf):  dx = dh * (Phi(x) + x phi(x));   SiLU: dx = dh * s (1 + x (1 - s)), s = sigmoid(x);
+//   SwiGLU h = silu(g) u:  dg = dh * u * silu'(g),  du = dh * silu(g).
+template <typename T>
+__device__ __forceinline__ void store_f32(T* p, float v);
+template <>
+__device__ __forceinline__ void store_f32<float>(float* p, float v) { *p = v; }
+template <>
+__device__ __forceinline__ void store_f32<bf16_t>(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+
+template <int EPI, typename T>
+__global__ __launch_bounds__(256) void act_backward_kernel(const T* __restrict__ a1, const T* __restrict__ dh,
+                                                            T* __restrict__ out, size_t rows, int F) {
+    const size_t total = rows * (size_t)F;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = i / F;
+        const int n = (int)(i % F);
+        const float d = load_f32<T>(dh + i);
+        if constexpr (EPI == EPI_SWIGLU) {
+            const size_t base = r * (size_t)(2 * F) + (size_t)(n / 32) * 64 + n % 32;
+            const float gv = load_f32<T>(a1 + base), uv = load_f32<T>(a1 + base + 32);
+            const float s = 1.0f / (1.0f + __expf(-gv));
+            store_f32<T>(out + base, d * uv * (s * (1.0f + gv * (1.0f - s))));
+            store_f32<T>(out + base + 32, d * (gv * s));
+        } else {
+            const float x = load_f32<T>(a1 + i);
+            float dv = d;
+            if constexpr (EPI == EPI_GELU)
+                dv = d * (0.5f * (1.0f + erff(x * 0.70710678118654752440f)) + x * 0.39894228040143267794f * __expf(-0.5f * x * x));
+            if constexpr (EPI == EPI_SILU) {
+                const float s = 1.0f / (1.0f + __expf(-x));
+                dv = d * (s * (1.0f + x * (1.0f - s)));
+            }
+            store_f32<T>(out + i, dv);
+        }
+    }
+}
+
+// fp32 path of the backward pass (plumbing-size workloads): d w[g] = x_g^T @ dy_g, 64 x 64 output tiles, the group's
+// rows in slabs of 32 through LDS; and the plain transposition w [E,K,N] -> [E,N,K] that d tokens = dy @ w^T needs.
+__global__ __launch_bounds__(256) void grouped_dw_f32_kernel(const float* __restrict__ x, const float* __restrict__ dy,
+                                                              const int32_t* __restrict__ cnt, int E_l, int K, int N, int S_rows,
+                                                              float* __restrict__ dw) {
+    constexpr int SC = 32;
+    __shared__ float xs[SC][64 + 1];
+    __shared__ float ys[SC][64 + 1];
+    const int g = blockIdx.z, k0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+    int row0 = 0;
+    for (int e = 0; e < g; ++e) row0 += max(cnt[e], 0);
+    const int c = min(max(cnt[g], 0), max(S_rows - row0, 0));
+    const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+    float acc[4][4] = {};
+    for (int s0 = 0; s0 < c; s0 += SC) {
+        for (int i = threadIdx.x; i < SC * 64; i += 256) {
+            const int r = i / 64, cc = i % 64;
+            const bool live = s0 + r < c;
+            xs[r][cc] = (live && k0 + cc < K) ? x[(size_t)(row0 + s0 + r) * K + k0 + cc] : 0.f;
+            ys[r][cc] = (live && n0 + cc < N) ? dy[(size_t)(row0 + s0 + r) * N + n0 + cc] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int r = 0; r < SC; ++r) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = xs[r][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = ys[r][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int k = k0 + ty * 4 + i, n = n0 + tx * 4 + j;
+            if (k < K && n < N) dw[((size_t)g * K + k) * N + n] = acc[i][j];
+        }
+}
+
+__global__ __launch_bounds__(256) void transpose_f32_kernel(const float* __restrict__ w, float* __restrict__ out, int K, int N) {
+    __shared__ float tile[32][33];
+    const float* src = w + (size_t)blockIdx.z * K * N;
+    float* dst = out + (size_t)blockIdx.z * K * N;
+    const int k0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+    for (int i = threadIdx.x; i < 1024; i += 256) {
+        const int k = i / 32, n = i % 32;
+        tile[k][n] = (k0 + k < K && n0 + n < N) ? src[(size_t)(k0 + k) * N + n0 + n] : 0.f;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 1024; i += 256) {
+        const int n = i / 32, k = i % 32;
+        if (k0 + k < K && n0 + n < N) dst[(size_t)(n0 + n) * K + k0 + k] = tile[k][n];
+    }
+}
+
 int num_cus() {
     static int cus = 0;
     if (cus == 0) {
@@ -1177,4 +1399,87 @@ extern "C" int moe_grouped_mlp_fp8(const void* tokens_bf16, const int32_t* exper
                                    void* out, moe_stream_t stream) {
     return moe_grouped_mlp_fp8_mapped(tokens_bf16, S_rows, nullptr, expert_cnt, S_rows, H, F, E_l, wgu_packed, sg, su, wd_packed,
                                       sd, xq_ws, xs_ws, h_ws, hq_ws, hs_ws, out, S_rows, nullptr, stream);
+}
+
+// ---- backward pass entry points --------------------------------------------------------------------------------------
+extern "C" int moe_prepack_weights_transposed(const void* w, const void* w_up, int dtype, int E_l, int K, int N, void* packed,
+                                              moe_stream_t stream) {
+    MOE_REQUIRE(dtype == MOE_BF16, MOE_ERR_INVALID, "prepack_weights_transposed: bf16 only (dtype %d)", dtype);
+    MOE_REQUIRE(E_l > 0 && K > 0 && N > 0 && w && packed, MOE_ERR_INVALID, "prepack_weights_transposed: bad arguments");
+    MOE_REQUIRE(N % 64 == 0 && K % 8 == 0, MOE_ERR_UNSUPPORTED,
+                "prepack_weights_transposed: needs N %% 64 == 0 and K %% 8 == 0 (K=%d N=%d)", K, N);
+    const int Kpad = round_up(K, GG_BN);
+    prepack_t_kernel<uint16_t><<<dim3(1024, E_l), 256, 0, (hipStream_t)stream>>>((const uint16_t*)w, (const uint16_t*)w_up,
+                                                                               (uint16_t*)packed, K, N, Kpad);
+    return moe_check_launch("prepack_weights_transposed");
+}
+
+extern "C" size_t moe_dw_workspace_bytes(int S_rows, int E_l, int K, int N) {
+    if (S_rows < 0 || E_l <= 0 || K <= 0 || N <= 0) return 0;
+    const size_t spad = (size_t)round_up(S_rows, 64) + (size_t)64 * E_l;
+    return spad * ((size_t)K + (size_t)round_up(N, GG_BN)) * 2;
+}
+
+extern "C" int moe_grouped_gemm_dw(const void* x, const void* dy, const int32_t* expert_cnt, int dtype, int S_rows, int K, int N,
+                                   int E_l, int split_F, void* dw, void* ws, size_t ws_bytes, moe_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    MOE_REQUIRE(S_rows >= 0 && K > 0 && N > 0 && E_l > 0 && E_l <= GG_MAXG, MOE_ERR_INVALID, "grouped_gemm_dw: bad shape");
+    MOE_REQUIRE(expert_cnt && dw && (S_rows == 0 || (x && dy)), MOE_ERR_INVALID, "grouped_gemm_dw: null pointer");
+    MOE_REQUIRE(split_F == 0 || (dtype == MOE_BF16 && split_F % 32 == 0 && N == 2 * split_F), MOE_ERR_INVALID,
+                "grouped_gemm_dw: split_F=%d needs bf16, split_F %% 32 == 0 and N == 2 split_F", split_F);
+    if (dtype == MOE_F32) {
+        grouped_dw_f32_kernel<<<dim3(ceil_div(N, 64), ceil_div(K, 64), E_l), 256, 0, s>>>((const float*)x, (const float*)dy, expert_cnt,
+                                                                                       E_l, K, N, S_rows, (float*)dw);
+        return moe_check_launch("grouped_gemm_dw_f32");
+    }
+    MOE_REQUIRE(dtype == MOE_BF16, MOE_ERR_INVALID, "grouped_gemm_dw: dtype %d", dtype);
+    MOE_REQUIRE(N % 8 == 0 && K % 8 == 0, MOE_ERR_UNSUPPORTED, "grouped_gemm_dw: bf16 needs K, N multiples of 8 (K=%d N=%d)", K, N);
+    MOE_REQUIRE(ws && ws_bytes >= moe_dw_workspace_bytes(S_rows, E_l, K, N), MOE_ERR_WORKSPACE, "grouped_gemm_dw: workspace %zu < %zu",
+                ws_bytes, moe_dw_workspace_bytes(S_rows, E_l, K, N));
+    const int spad = round_up(S_rows, 64) + 64 * E_l;  // upper bound of the padded row total, and the operands' pitch
+    MOE_REQUIRE((unsigned long long)K * (unsigned long long)spad * 2ull < (1ull << 32), MOE_ERR_UNSUPPORTED,
+                "grouped_gemm_dw: the transposed activations must stay under 4 GiB (%d x %d)", K, spad);
+    const int Npad = round_up(N, GG_BN);
+    uint16_t* xT = (uint16_t*)ws;                       // [K, spad]
+    uint16_t* dyP = xT + (size_t)K * spad;              // [spad / 32][Npad][32]
+    const int pblocks = spad / 64;
+    dw_zero_empty_kernel<<<dim3(256, E_l), 256, 0, s>>>((uint4*)dw, expert_cnt, (size_t)K * N * 2 / 16, S_rows);
+    if (S_rows > 0) {
+        dw_operand_kernel<false><<<dim3(ceil_div(K, 64), pblocks), 256, 0, s>>>((const uint16_t*)x, expert_cnt, E_l, S_rows, K, xT, spad, 0, 0);
+        dw_operand_kernel<true><<<dim3(Npad / 64, pblocks), 256, 0, s>>>((const uint16_t*)dy, expert_cnt, E_l, S_rows, N, dyP, spad, Npad, split_F);
+        GemmParams p{};
+        p.A = (const uint8_t*)xT; p.B = (const uint8_t*)dyP; p.C = dw; p.cnt = expert_cnt;
+        p.E_l = E_l; p.K = spad; p.N = N; p.Npad = Npad; p.ldc = N; p.S_rows = K;
+        p.dw_rows = K; p.dw_src_rows = S_rows; p.c_group_stride = (size_t)K * N;
+        grouped_gemm_kernel<256, GG_BIG_NWM, EPI_NONE, false, false, true><<<num_cus(), GG_BIG_NWM * 2 * WAVE, 0, s>>>(p);
+    }
+    return moe_check_launch("grouped_gemm_dw");
+}
+
+extern "C" int moe_transpose_weights_f32(const float* w, int E_l, int K, int N, float* out, moe_stream_t stream) {
+    MOE_REQUIRE(E_l > 0 && K > 0 && N > 0 && w && out, MOE_ERR_INVALID, "transpose_weights_f32: bad arguments");
+    transpose_f32_kernel<<<dim3(ceil_div(N, 32), ceil_div(K, 32), E_l), 256, 0, (hipStream_t)stream>>>(w, out, K, N);
+    return moe_check_launch("transpose_weights_f32");
+}
+
+extern "C" int moe_mlp_act_backward(const void* a1, const void* dh, int dtype, int rows, int F, int act, void* d_a1,
+                                    moe_stream_t stream) {
+    MOE_REQUIRE(rows >= 0 && F > 0, MOE_ERR_INVALID, "mlp_act_backward: bad shape");
+    MOE_REQUIRE(dtype == MOE_BF16 || (dtype == MOE_F32 && act != EPI_SWIGLU), MOE_ERR_UNSUPPORTED,
+                "mlp_act_backward: dtype %d with activation %d", dtype, act);
+    MOE_REQUIRE(act == EPI_GELU || act == EPI_SILU || act == EPI_SWIGLU, MOE_ERR_INVALID, "mlp_act_backward: activation %d", act);
+    MOE_REQUIRE(act != EPI_SWIGLU || F % 32 == 0, MOE_ERR_UNSUPPORTED, "mlp_act_backward: swiglu needs F %% 32 == 0");
+    if (rows == 0) return MOE_OK;
+    MOE_REQUIRE(a1 && dh && d_a1, MOE_ERR_INVALID, "mlp_act_backward: null pointer");
+    const int blocks = (int)std::min<size_t>(((size_t)rows * F + 255) / 256, (size_t)num_cus() * 32);
+    hipStream_t s = (hipStream_t)stream;
+#define GG_ACTB(EPIv, Tv) act_backward_kernel<EPIv, Tv><<<blocks, 256, 0, s>>>((const Tv*)a1, (const Tv*)dh, (Tv*)d_a1, (size_t)rows, F)
+    if (dtype == MOE_F32) {
+        if (act == EPI_GELU) GG_ACTB(EPI_GELU, float);
+        else GG_ACTB(EPI_SILU, float);
+    } else if (act == EPI_GELU) GG_ACTB(EPI_GELU, bf16_t);
+    else if (act == EPI_SILU) GG_ACTB(EPI_SILU, bf16_t);
+    else GG_ACTB(EPI_SWIGLU, bf16_t);
+#undef GG_ACTB
+    return moe_check_launch("mlp_act_backward");
 }

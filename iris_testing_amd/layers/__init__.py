@@ -4,4 +4,4 @@ layers/token_shuffle.py, layers/expert.py) plus the two the path needs that the 
 from .all_to_all import custom_a2a, SimulatedWorld, simulated_world  # noqa: F401
 from .token_shuffle import shuffle  # noqa: F401
 from .expert import expert, expert_mlp, ExpertWeights  # noqa: F401
-from .combine import combine  # noqa: F401
+from .combine import combine, pack_fixed_m  # noqa: F401

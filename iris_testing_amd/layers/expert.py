@@ -3,7 +3,7 @@ expert MLP the workloads define (Linear-act-Linear, SwiGLU, fp8) which the refer
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Optional
 
 import torch
@@ -13,23 +13,46 @@ from ..utils import _assert_cuda_int32
 
 
 # Re-tiled copies of weight tensors the operator has seen, keyed on the tensor's storage and version counter, so that
-# a weight that did not change between calls is re-tiled once, not on every forward (the re-tiling reads and writes the
+# a weight that did not change between calls is re-tiled once, not on every call (the re-tiling reads and writes the
 # whole tensor).  Entries die with their tensors (weak references); an in-place update bumps the version and re-tiles.
 _PACKED = {}
 _PART_WS = {}
 
 
-def _packed_weights(w: torch.Tensor) -> torch.Tensor:
+def _cached_pack(kind: str, w: torch.Tensor, w_up: Optional[torch.Tensor], build) -> torch.Tensor:
     import weakref
-    key = (w.data_ptr(), w._version, tuple(w.shape), w.dtype, w.device)
+    key = (kind, w.data_ptr(), w._version, None if w_up is None else (w_up.data_ptr(), w_up._version), tuple(w.shape), w.dtype,
+           w.device)
     hit = _PACKED.get(key)
     if hit is not None and hit[0]() is w:
         return hit[1]
-    for k in [k for k, v in _PACKED.items() if v[0]() is None or (v[0]() is w and k != key)]:
+    for k in [k for k, v in _PACKED.items() if v[0]() is None or (v[0]() is w and k[0] == kind)]:
         del _PACKED[k]
-    packed = ops.prepack_weights(w)
+    packed = build(w, w_up)
     _PACKED[key] = (weakref.ref(w), packed)
     return packed
+
+
+def _packed_weights(w: torch.Tensor, w_up: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Re-tiled w (with w_up: the fused gate/up pair) for the forward GEMM."""
+    return _cached_pack("N", w, w_up, ops.prepack_weights)
+
+
+def _packed_weights_t(w: torch.Tensor, w_up: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Re-tiled w^T (with w_up: of the pair, in the fused gate/up column order) for d tokens = d out @ w^T."""
+    return _cached_pack("T", w, w_up, ops.prepack_weights_transposed)
+
+
+def _grouped_gemm_t(do: torch.Tensor, weights: torch.Tensor, cnt: torch.Tensor) -> torch.Tensor:
+    """d tokens[rows of g] = do[rows of g] @ weights[g]^T; rows past sum(cnt) are zero."""
+    E_l, K, N = weights.shape
+    S = do.shape[0]
+    if do.dtype == torch.float32:
+        return ops.grouped_gemm(do, ops.transpose_weights_f32(weights.contiguous()), cnt)
+    out = torch.zeros((S, K), dtype=do.dtype, device=do.device)
+    if S:
+        ops.grouped_gemm_mapped(do, None, _packed_weights_t(weights), cnt, S, K, "none", out, part_ws=_part_ws(do.device))
+    return out
 
 
 def _part_ws(device) -> torch.Tensor:
@@ -42,7 +65,7 @@ def _part_ws(device) -> torch.Tensor:
 
 def _grouped_gemm(tokens: torch.Tensor, weights: torch.Tensor, cnt: torch.Tensor) -> torch.Tensor:
     """out[rows of g] = tokens[rows of g] @ weights[g]; rows past sum(cnt) are zero."""
-    if tokens.dtype != torch.bfloat16 or weights.shape[1] % 64 or weights.shape[2] % 8:
+    if tokens.dtype != torch.bfloat16 or weights.shape[1] % 64 or weights.shape[2] % 8:  # (what the MFMA kernel covers)
         return ops.grouped_gemm(tokens, weights, cnt)
     S, N = tokens.shape[0], weights.shape[2]
     out = torch.zeros((S, N), dtype=tokens.dtype, device=tokens.device)
@@ -67,32 +90,16 @@ class Expert(torch.autograd.Function):
     @staticmethod
     def backward(ctx, do):
         """Gradients of out[rows of g] = tokens[rows of g] @ weights[g] (not implemented in the reference,
-        layers/expert.py:62-64), both on the grouped GEMM kernel:
-          d tokens[rows of g] = do[rows of g] @ weights[g]^T        one grouped launch over the transposed weights
-          d weights[g]        = tokens[rows of g]^T @ do[rows of g]  one launch per expert: the reduction runs over
-                                                                      the expert's rows, zero padded to 64
-        Rows past the counted total get a zero gradient."""
+        layers/expert.py:62-64), both as grouped launches over all experts:
+          d tokens[rows of g] = do[rows of g] @ weights[g]^T        the grouped GEMM over the transposed, re-tiled weights
+          d weights[g]        = tokens[rows of g]^T @ do[rows of g]  the grouped GEMM in its weight-gradient mode: the
+                                                                      reduction runs over the expert's (ragged) rows
+        Rows past the counted total get a zero gradient, experts without rows a zero weight gradient."""
         tokens, weights, cnt = ctx.saved_tensors
         do = do.contiguous()
-        E_l, H, F = weights.shape
-        d_tokens = ops.grouped_gemm(do, weights.transpose(1, 2).contiguous(), cnt.contiguous())
-        counts = [max(int(c), 0) for c in cnt.cpu().tolist()]
-        total = min(sum(counts), tokens.shape[0])
-        if total < tokens.shape[0]:
-            d_tokens[total:].zero_()
-        d_weights = torch.zeros_like(weights)
-        h_rows = torch.full((1,), H, dtype=torch.int32, device=tokens.device)
-        row0 = 0
-        for g, c in enumerate(counts):
-            c = min(c, tokens.shape[0] - row0)
-            if c > 0:
-                pad = (c + 63) // 64 * 64
-                xt = torch.zeros((H, pad), dtype=tokens.dtype, device=tokens.device)
-                xt[:, :c] = tokens[row0:row0 + c].t()
-                dy = torch.zeros((1, pad, F), dtype=do.dtype, device=do.device)
-                dy[0, :c] = do[row0:row0 + c]
-                d_weights[g] = ops.grouped_gemm(xt, dy, h_rows)
-            row0 += c
+        cnt = cnt.contiguous()
+        d_tokens = _grouped_gemm_t(do, weights, cnt)
+        d_weights = ops.grouped_gemm_dw(tokens.contiguous(), do, cnt)
         return d_tokens, d_weights, None, None
 
 
@@ -115,16 +122,20 @@ class ExpertWeights:
     w2: torch.Tensor
     w_up: Optional[torch.Tensor] = None
     scales: Optional[tuple] = None  # fp8: (sg, su, sd)
+    # the tensors prepare() was given, in the reference layout: (w1, w2, w_up); the backward pass differentiates with
+    # respect to them and re-tiles their transposes on first use
+    raw: Optional[tuple] = field(default=None, repr=False)
 
     @classmethod
     def prepare(cls, act: str, w1: torch.Tensor, w2: torch.Tensor, w_up: Optional[torch.Tensor] = None):
         e_l, H, F = w1.shape
+        raw = (w1, w2, w_up)
         if w1.dtype == torch.float32:
             return cls(act, H, F, e_l, w1.dtype, w1.contiguous(), w2.contiguous(),
-                       None if w_up is None else w_up.contiguous())
+                       None if w_up is None else w_up.contiguous(), raw=raw)
         p1 = ops.prepack_weights(w1.contiguous(), None if w_up is None else w_up.contiguous())
         p2 = ops.prepack_weights(w2.contiguous())
-        return cls(act, H, F, e_l, w1.dtype, p1, p2)
+        return cls(act, H, F, e_l, w1.dtype, p1, p2, raw=raw)
 
     @classmethod
     def prepare_fp8(cls, wg_q, sg, wu_q, su, wd_q, sd):
@@ -135,6 +146,59 @@ class ExpertWeights:
         return cls("swiglu", H, F, e_l, torch.uint8, p1, p2, None, (sg.contiguous(), su.contiguous(), sd.contiguous()))
 
 
+class ExpertMLP(torch.autograd.Function):
+    """y = act(x W1) W2, or (silu(x Wg) * (x Wu)) Wd, on expert-major rows, with its gradients (the reference defines
+    neither the MLP nor a backward).  Inputs that autograd sees: tokens and the weight tensors ``prepare`` was given."""
+
+    @staticmethod
+    def forward(ctx, tokens, cnt, ew, w1, w2, w_up):
+        tokens = tokens.contiguous()
+        S = tokens.shape[0]
+        hidden = torch.empty((S, ew.ffn), dtype=tokens.dtype, device=tokens.device)
+        out = ops.grouped_mlp(tokens, cnt, ew.act, ew.w1, ew.w2, ew.w_up, F=ew.ffn, hidden_ws=hidden)
+        ctx.save_for_backward(tokens, hidden, cnt, w1, w2, w_up)
+        ctx.ew = ew
+        return out
+
+    @staticmethod
+    def backward(ctx, dy):
+        """With a1 the pre-activations (recomputed: the forward keeps only the hidden activation h):
+          d h  = dy @ W2^T          d W2 = h^T @ dy            (per expert, ragged rows as the reduction dimension)
+          d a1 = d h * act'(a1)     (SwiGLU: d g = d h * u * silu'(g), d u = d h * silu(g))
+          d x  = d a1 @ W1^T        d W1 = x^T @ d a1          (SwiGLU: both halves in one launch each)"""
+        tokens, hidden, cnt, w1, w2, w_up = ctx.saved_tensors
+        ew = ctx.ew
+        dy = dy.contiguous()
+        S, H, F = tokens.shape[0], ew.hidden, ew.ffn
+        swiglu = ew.act == "swiglu"
+        if tokens.dtype == torch.float32:
+            if swiglu:
+                raise NotImplementedError("expert_mlp backward: fp32 SwiGLU (the fp32 path serves the GELU / SiLU plumbing workload)")
+            dh = ops.grouped_gemm(dy, ops.transpose_weights_f32(w2.contiguous()), cnt)
+            dw2 = ops.grouped_gemm_dw(hidden, dy, cnt)
+            a1 = ops.grouped_gemm(tokens, w1.contiguous(), cnt)
+            da1 = ops.mlp_act_backward(a1, dh, ew.act)
+            dx = ops.grouped_gemm(da1, ops.transpose_weights_f32(w1.contiguous()), cnt)
+            dw1 = ops.grouped_gemm_dw(tokens, da1, cnt)
+            return dx, None, None, dw1, dw2, None
+        ws = _part_ws(tokens.device)
+        NP = 2 * F if swiglu else F
+        dh = torch.zeros((S, F), dtype=dy.dtype, device=dy.device)
+        dx = torch.zeros((S, H), dtype=dy.dtype, device=dy.device)
+        a1 = torch.zeros((S, NP), dtype=dy.dtype, device=dy.device)
+        if S:
+            ops.grouped_gemm_mapped(dy, None, _packed_weights_t(w2), cnt, S, F, "none", dh, part_ws=ws)
+            ops.grouped_gemm_mapped(tokens, None, ew.w1, cnt, S, NP, "none", a1, part_ws=ws)
+        dw2 = ops.grouped_gemm_dw(hidden, dy, cnt)
+        da1 = ops.mlp_act_backward(a1, dh, ew.act)
+        if S:
+            ops.grouped_gemm_mapped(da1, None, _packed_weights_t(w1, w_up), cnt, S, H, "none", dx, part_ws=ws)
+        dw1 = ops.grouped_gemm_dw(tokens, da1, cnt, split_F=F if swiglu else 0)
+        if swiglu:
+            return dx, None, None, dw1[..., :F], dw2, dw1[..., F:]
+        return dx, None, None, dw1, dw2, None
+
+
 def expert_mlp(tokens: torch.Tensor, weights: ExpertWeights, local_expert_cnt: torch.Tensor) -> torch.Tensor:
     """Full expert MLP on expert-major rows -> [S,H]."""
     assert tokens.is_cuda, "tokens must be CUDA"
@@ -142,5 +206,8 @@ def expert_mlp(tokens: torch.Tensor, weights: ExpertWeights, local_expert_cnt: t
     if weights.dtype == torch.uint8:
         sg, su, sd = weights.scales
         return ops.grouped_mlp_fp8(tokens.contiguous(), local_expert_cnt, weights.ffn, weights.w1, sg, su, weights.w2, sd)
+    raw = weights.raw
+    if torch.is_grad_enabled() and raw is not None and (tokens.requires_grad or any(t is not None and t.requires_grad for t in raw)):
+        return ExpertMLP.apply(tokens, local_expert_cnt.contiguous(), weights, raw[0], raw[1], raw[2])
     return ops.grouped_mlp(tokens.contiguous(), local_expert_cnt, weights.act, weights.w1, weights.w2, weights.w_up,
                            F=weights.ffn)

@@ -446,3 +446,80 @@ def build_expert_offsets(send_counts: torch.Tensor, with_dst: bool = False):
     L.check(L.lib().moe_build_expert_offsets(L.ptr(send_counts), W, E_l, L.ptr(offs), L.ptr(sizes), L.ptr(doffs),
                                              L.stream_ptr()))
     return (offs, sizes, doffs) if with_dst else offs
+
+
+# ---- gradients ----------------------------------------------------------------------------------
+def prepack_weights_transposed(w: torch.Tensor, w_up: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """[E_l,K,N] bf16 -> the kernels' layout of w^T (weights of d tokens = d out @ w^T); with ``w_up`` the pair is
+    transposed together in the fused gate/up column order."""
+    _req_cuda(w, "weights")
+    assert w.dtype == torch.bfloat16
+    E_l, K, N = w.shape
+    if w_up is not None:
+        _req_cuda(w_up, "w_up")
+        assert w_up.shape == w.shape and w_up.dtype == w.dtype
+    n_tot = N * (2 if w_up is not None else 1)
+    nbytes = L.lib().moe_prepack_bytes(L.MOE_BF16, E_l, n_tot, K)
+    out = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
+    L.check(L.lib().moe_prepack_weights_transposed(L.ptr(w), L.ptr(w_up), L.MOE_BF16, E_l, K, N, L.ptr(out), L.stream_ptr()))
+    return out
+
+
+def transpose_weights_f32(w: torch.Tensor) -> torch.Tensor:
+    """[E_l,K,N] fp32 -> [E_l,N,K]."""
+    _req_cuda(w, "weights")
+    assert w.dtype == torch.float32
+    E_l, K, N = w.shape
+    out = torch.empty((E_l, N, K), dtype=w.dtype, device=w.device)
+    L.check(L.lib().moe_transpose_weights_f32(L.ptr(w), E_l, K, N, L.ptr(out), L.stream_ptr()))
+    return out
+
+
+def grouped_gemm_dw(x: torch.Tensor, dy: torch.Tensor, expert_cnt: torch.Tensor, split_F: int = 0) -> torch.Tensor:
+    """d w[g] = x[rows of g]^T @ dy[rows of g] for all groups in one launch -> [E_l,K,N] (zeros for empty groups).
+    ``split_F`` > 0: dy is [S, 2 split_F] in the fused gate/up column order, the result [E_l,K,2 split_F] holds
+    [d w_gate | d w_up] side by side."""
+    _req_cuda(x, "x")
+    _req_cuda(dy, "dy")
+    _req_i32(expert_cnt, "expert_cnt")
+    assert x.dtype == dy.dtype and x.shape[0] == dy.shape[0]
+    S, K = x.shape
+    N = dy.shape[1]
+    E_l = expert_cnt.numel()
+    code = L.dtype_code(x.dtype)
+    dw = torch.empty((E_l, K, N), dtype=x.dtype, device=x.device)
+    nbytes = L.lib().moe_dw_workspace_bytes(S, E_l, K, N) if x.dtype == torch.bfloat16 else 0
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+    L.check(L.lib().moe_grouped_gemm_dw(L.ptr(x), L.ptr(dy), L.ptr(expert_cnt), code, S, K, N, E_l, split_F, L.ptr(dw), L.ptr(ws),
+                                        nbytes, L.stream_ptr()))
+    return dw
+
+
+def mlp_act_backward(a1: torch.Tensor, dh: torch.Tensor, act: str) -> torch.Tensor:
+    """Gradient of the pre-activations a1 ([S,F]; swiglu: [S,2F] in the fused gate/up column order) from d hidden [S,F]."""
+    _req_cuda(a1, "a1")
+    _req_cuda(dh, "dh")
+    assert a1.dtype == dh.dtype
+    S, F = dh.shape
+    out = torch.empty_like(a1)
+    L.check(L.lib().moe_mlp_act_backward(L.ptr(a1), L.ptr(dh), L.dtype_code(a1.dtype), S, F, L.ACT[act], L.ptr(out), L.stream_ptr()))
+    return out
+
+
+def combine_backward(d_out: torch.Tensor, ret: torch.Tensor, topk_idx: torch.Tensor, pos: torch.Tensor, gate: torch.Tensor,
+                     dst_sizes: torch.Tensor, dst_offsets: torch.Tensor, e_local: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(d ret [W,M,H], d gate [T,k]) of out = combine(ret, ...)."""
+    _req_cuda(d_out, "d_out")
+    _req_cuda(ret, "ret")
+    _req_i32(topk_idx, "topk_idx")
+    _req_i32(pos, "pos")
+    _req_i32(dst_sizes, "dst_sizes")
+    _req_i32(dst_offsets, "dst_offsets")
+    W, M, H = ret.shape
+    T, k = topk_idx.shape
+    d_ret = torch.empty_like(ret)
+    d_gate = torch.empty((T, k), dtype=torch.float32, device=ret.device)
+    L.check(L.lib().moe_combine_backward(L.ptr(d_out), L.ptr(ret), L.dtype_code(ret.dtype), W, M, H, L.ptr(topk_idx), L.ptr(pos),
+                                         L.ptr(gate), L.ptr(dst_sizes), L.ptr(dst_offsets), T, k, e_local, L.ptr(d_ret),
+                                         L.ptr(d_gate), L.stream_ptr()))
+    return d_ret, d_gate

@@ -1,0 +1,140 @@
+"""Gradients of the path's operators (every backward of the reference is an empty stub: layers/expert.py:62-64,
+layers/token_shuffle.py:58-60) against float64 autograd of the forward formulas on the CPU.  Parity unpinned by the
+reference, pinned by the mathematics; bf16 runs are bounded relative to the largest gradient entry."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import O, assert_bits_equal, to_np
+
+pytestmark = pytest.mark.gpu
+
+from iris_testing_amd import ops  # noqa: E402
+from iris_testing_amd.layers import ExpertWeights, combine, expert_mlp, pack_fixed_m  # noqa: E402
+
+DEV = "cuda"
+
+
+def _rel(got, want):
+    got, want = got.double().cpu(), want.double()
+    return float((got - want).abs().max()) / (float(want.abs().max()) + 1e-30)
+
+
+def _act64(a, act, u=None):
+    if act == "gelu":
+        return torch.nn.functional.gelu(a)
+    if act == "silu":
+        return torch.nn.functional.silu(a)
+    return torch.nn.functional.silu(a) * u
+
+
+@pytest.mark.parametrize("dtype,act,H,F,cnt", [(torch.bfloat16, "swiglu", 256, 384, (150, 0, 333, 64)),
+                                               (torch.bfloat16, "gelu", 128, 256, (70, 45)),
+                                               (torch.bfloat16, "silu", 192, 128, (1, 300, 0)),
+                                               (torch.bfloat16, "swiglu", 512, 1408, (700,)),
+                                               (torch.float32, "gelu", 256, 512, (100, 0, 157))])
+def test_expert_mlp_backward_matches_float64_autograd(dtype, act, H, F, cnt):
+    rng = np.random.default_rng(H + F + len(cnt))
+    cnt = np.array(cnt, dtype=np.int32)
+    E_l, S = len(cnt), int(cnt.sum()) + 3  # three rows past the counted total: no part in anything, zero gradient
+    mk = lambda *s, sc=1.0: torch.from_numpy((rng.standard_normal(s) * sc).astype(np.float32)).to(dtype)  # noqa: E731
+    x, w1, w2 = mk(S, H), mk(E_l, H, F, sc=H ** -0.5), mk(E_l, F, H, sc=F ** -0.5)
+    wu = mk(E_l, H, F, sc=H ** -0.5) if act == "swiglu" else None
+    g = mk(S, H)
+    leaves = [t.to(DEV).requires_grad_(True) for t in (x, w1, w2)] + ([wu.to(DEV).requires_grad_(True)] if wu is not None else [])
+    xd, w1d, w2d = leaves[:3]
+    wud = leaves[3] if wu is not None else None
+    ew = ExpertWeights.prepare(act, w1d, w2d, wud)
+    out = expert_mlp(xd, ew, torch.from_numpy(cnt).to(DEV))
+    assert out.requires_grad
+    out.backward(g.to(DEV))
+    # float64 autograd of the same formula
+    x64, w164, w264 = (t.double().requires_grad_(True) for t in (x, w1, w2))
+    wu64 = wu.double().requires_grad_(True) if wu is not None else None
+    parts, r = [], 0
+    for e, c in enumerate(cnt):
+        xe = x64[r:r + c]
+        h = _act64(xe @ w164[e], act, None if wu64 is None else xe @ wu64[e])
+        parts.append(h @ w264[e])
+        r += c
+    ref = torch.cat(parts + [torch.zeros((S - r, H), dtype=torch.float64)])
+    ref.backward(g.double())
+    tol = 1e-4 if dtype == torch.float32 else 2.0 ** -5
+    names = [("d tokens", xd.grad, x64.grad), ("d w1", w1d.grad, w164.grad), ("d w2", w2d.grad, w264.grad)]
+    if wu is not None:
+        names.append(("d w_up", wud.grad, wu64.grad))
+    for name, got, want in names:
+        assert got is not None and got.shape == want.shape, name
+        err = _rel(got, want)
+        print(f"{act} {dtype} {name}: max error / max |gradient| = {err:.2e}", flush=True)
+        assert err < tol, f"{name}: {err}"
+    total = int(cnt.sum())
+    assert bool((xd.grad[total:] == 0).all()), "rows past the counted total must get a zero gradient"
+    empty = torch.from_numpy(cnt == 0)
+    if bool(empty.any()):
+        for name, got, _ in names[1:]:
+            assert bool((got[empty.to(DEV)] == 0).all()), f"{name} of an expert without rows must be zero"
+
+
+@pytest.mark.parametrize("K,N,cnt,split", [(128, 192, (70, 0, 45, 64, 1), False), (256, 256, (300, 129), True),
+                                           (64, 264, (5,), False)])
+def test_grouped_weight_gradient_kernel(K, N, cnt, split):
+    """d w[g] = x_g^T dy_g with the ragged row count as the reduction dimension, one launch: against float64, with
+    empty groups, group sizes that are no multiple of the 64-row padding, stale workspace contents, and the fused
+    gate/up column order undone on the way out."""
+    rng = np.random.default_rng(K + N)
+    cnt = np.array(cnt, dtype=np.int32)
+    S = int(cnt.sum())
+    x = O.bf16_round(rng.standard_normal((S + 2, K)).astype(np.float32))
+    dy = O.bf16_round(rng.standard_normal((S + 2, N)).astype(np.float32))
+    xt, dyt = torch.from_numpy(x).bfloat16().to(DEV), torch.from_numpy(dy).bfloat16().to(DEV)
+    dw = to_np(ops.grouped_gemm_dw(xt, dyt, torch.from_numpy(cnt).to(DEV), split_F=N // 2 if split else 0))
+    r = 0
+    for e, c in enumerate(cnt):
+        want = x[r:r + c].astype(np.float64).T @ dy[r:r + c].astype(np.float64)
+        if split:  # input columns: 32 gate, 32 up, 32 gate, ...; output: all gate, then all up
+            F = N // 2
+            col = np.arange(N)
+            want = want[:, np.argsort(((col % 64) // 32) * F + (col // 64) * 32 + col % 32, kind="stable")]
+        scale = np.abs(want).max() + 1e-30
+        err = np.abs(dw[e] - want).max() / scale if c else np.abs(dw[e]).max()
+        assert err < 2.0 ** -7, f"group {e} ({c} rows): {err}"
+        r += c
+
+
+def test_combine_and_pack_gradients_match_float64_autograd():
+    rng = np.random.default_rng(4)
+    T, H, E, k, W = 90, 64, 12, 3, 4
+    E_l = E // W
+    idx = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+    counts = O.send_counts(idx, W, E)
+    sizes, offs = O.dst_sizes_offsets(counts)
+    pos, _ = O.payload_positions(idx, E)
+    M = O.pair_capacity(sizes) + 2
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(DEV)  # noqa: E731
+    idx_t, pos_t, sizes_t, offs_t = dev(idx), dev(pos), dev(sizes), dev(offs)
+    slot = torch.from_numpy((idx // E_l).astype(np.int64) * M + (pos - offs[idx // E_l]).astype(np.int64))  # [T,k] row of [W*M]
+    for dtype in (torch.float32, torch.bfloat16):
+        ret = torch.from_numpy(rng.standard_normal((W, M, H)).astype(np.float32)).to(dtype)
+        gate = torch.from_numpy(rng.random((T, k)).astype(np.float32))
+        g = torch.from_numpy(rng.standard_normal((T, H)).astype(np.float32)).to(dtype)
+        rd, gd = ret.to(DEV).requires_grad_(True), gate.to(DEV).requires_grad_(True)
+        out = combine(rd, idx_t, pos_t, gd, offs_t, E_l)
+        out.backward(g.to(DEV))
+        r64, g64 = ret.double().requires_grad_(True), gate.double().requires_grad_(True)
+        ref = (g64[:, :, None] * r64.view(W * M, H)[slot]).sum(1)
+        ref.backward(g.double())
+        tol = 1e-5 if dtype == torch.float32 else 2.0 ** -7
+        assert _rel(rd.grad, r64.grad) < tol and _rel(gd.grad, g64.grad) < tol
+        used = torch.zeros(W * M, dtype=torch.bool)
+        used[slot.reshape(-1)] = True
+        assert bool((rd.grad.view(W * M, H)[~used.to(DEV)] == 0).all()), "padding slots must get a zero gradient"
+        # the pack: d tokens[t] = sum of the gradients of its k slots
+        x = torch.from_numpy(rng.standard_normal((T, H)).astype(np.float32)).to(dtype)
+        gs = torch.from_numpy(rng.standard_normal((W, M, H)).astype(np.float32)).to(dtype)
+        xd = x.to(DEV).requires_grad_(True)
+        send = pack_fixed_m(xd, idx_t, pos_t, sizes_t, offs_t, E_l, M)
+        assert_bits_equal(send, O.pack_fixed_m(O.send_payload(to_np(x), O.payload_positions(idx, E)[1]), offs, sizes, M), "send")
+        send.backward(gs.to(DEV))
+        want = gs.double().view(W * M, H)[slot].sum(1)
+        assert _rel(xd.grad, want) < tol
