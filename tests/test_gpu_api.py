@@ -162,6 +162,56 @@ def test_benchmark_driver_point_and_overflow_report(capsys):
     assert res["source_ms"] > 0 and res["dest_ms"] > 0 and res["dest_direct_ms"] > 0
 
 
+def test_benchmark_driver_point_is_the_oracles_layout():
+    """The driver's CHECK compares two device routes with each other; here the buffers of the same point are held to
+    the CPU oracle: pca, the zero-padded token_buf and the receive buffer it was filled from, bit for bit."""
+    from iris_testing_amd import benchmark
+    from iris_testing_amd.configs import gen_router, gen_shard_tokens
+    res = benchmark.run_point({"WORLD_SIZE": 4, "BATCH": 1, "SEQ": 320, "HIDDEN": 256, "TOPK": 2, "E_LOCAL": 3,
+                               "CAPACITY": 8, "SEED": 7}, keep=True)
+    assert res["ok"] and res["baseline_agrees"]
+    cfg = res["world_obj"].cfg
+    xs = [to_np(gen_shard_tokens(cfg, s)) for s in range(cfg.world)]
+    router = to_np(gen_router(cfg))
+    shards = []
+    for x in xs:
+        idx = O.route(x, router, cfg.topk)[0]
+        counts = O.send_counts(idx, cfg.world, cfg.experts)
+        sizes, offs = O.dst_sizes_offsets(counts)
+        shards.append((counts, sizes, offs, O.payload_positions(idx, cfg.experts)[1]))
+    M = O.pair_capacity(np.stack([s[1] for s in shards]))
+    assert M == res["M"]
+    o_recv = np.stack([O.pack_fixed_m(O.send_payload(x, s[3]), s[2], s[1], M)[0] for x, s in zip(xs, shards)])
+    o_rc = np.stack([s[0][0] for s in shards]).astype(np.int32)
+    assert_bits_equal(res["recv"], o_recv, "receive buffer")
+    assert_bits_equal(res["recv_counts"], o_rc, "recv_counts")
+    o_tb, o_pca = O.recv_to_token_buf(o_recv, o_rc, res["cap"])
+    assert_bits_equal(res["pca"], o_pca, "pca")
+    assert_bits_equal(res["token_buf"], o_tb, "token_buf")
+
+
+def test_benchmark_sweep_prints_the_figure_tables(capsys, monkeypatch):
+    """One pass of SWEEP=topk at a small shape: one detailed row and one figure-style row per top-k value, the
+    library baseline moving the same bytes as the kernels at every point."""
+    from iris_testing_amd import benchmark
+    for k, v in {"WORLD_SIZE": "4", "BATCH": "1", "SEQ": "256", "HIDDEN": "256", "E_LOCAL": "4", "SEED": "3"}.items():
+        monkeypatch.setenv(k, v)
+    monkeypatch.setattr(benchmark, "WARMUP", 1)
+    monkeypatch.setattr(benchmark, "ITERS", 2)
+    rows = benchmark.run_sweep("topk")
+    out = capsys.readouterr().out.splitlines()
+    assert [v for v, _ in rows] == [1, 2, 4, 8] and all(r["baseline_agrees"] for _, r in rows)
+    head = [i for i, l in enumerate(out) if l.startswith("=== all2all_topk_change")]
+    assert len(head) == 1
+    fig = out[head[0] + 2: head[0] + 6]
+    assert [int(l.split()[0]) for l in fig] == [1, 2, 4, 8]
+    for l in fig:
+        cols = l.split()
+        assert len(cols) == 5 and float(cols[1]) > 0 and float(cols[2]) > 0 and cols[3].endswith("x") and cols[4] == "yes"
+    detail = [l for l in out[:head[0]] if l.split() and l.split()[0].isdigit()]
+    assert len(detail) == 4 and all(len(l.split()) == 9 for l in detail)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_shuffle_backward_puts_rows_back_and_zeroes_the_padding(dtype):
     """Gradient of the expert-major unpack (empty in the reference, token_shuffle.py:58-60): the shuffle is a row
