@@ -241,12 +241,14 @@ int moe_shuffle_backward(const void* grad_rows, int dtype, int E_l, int W, int C
                          void* grad_token_buf, int32_t* map_ws, moe_stream_t stream);
 /* moe_grouped_mlp_fp8 with the same row indirection: the row quantisation reads input row r from row
  * a_row_map[r] of a_base_bf16 (a_rows rows of H), the down GEMM writes result row r to row c_row_map[r]
- * of out (out_rows rows of H); either map may be NULL. */
+ * of out (out_rows rows of H); either map may be NULL.  part_ws (nullable): the K-split scratch of
+ * moe_grouped_gemm_mapped, used by both GEMMs in turn. */
 int moe_grouped_mlp_fp8_mapped(const void* a_base_bf16, int a_rows, const int32_t* a_row_map,
                                const int32_t* expert_cnt, int S_rows, int H, int F, int E_l,
                                const uint8_t* wgu_packed, const float* sg, const float* su, const uint8_t* wd_packed,
                                const float* sd, uint8_t* xq_ws, float* xs_ws, void* h_ws, uint8_t* hq_ws, float* hs_ws,
-                               void* out, int out_rows, const int32_t* c_row_map, moe_stream_t stream);
+                               void* out, int out_rows, const int32_t* c_row_map, void* part_ws, size_t part_ws_bytes,
+                               moe_stream_t stream);
 
 /* ---- gradients (every backward of the reference is an empty stub: layers/expert.py:62-64,
  * layers/token_shuffle.py:58-60, layers/all_to_all.py:121-123) -----------------------------------------------------

@@ -69,7 +69,8 @@ _SIGNATURES = {
     "moe_combine_backward": (c_int, [P, P, c_int, c_int, c_int, c_int, P, P, P, P, P, c_int, c_int, c_int, P, P, P]),
     "moe_gemm_split_plan": (c_int, [c_int, c_int, c_int, c_int, P]),
     "moe_zero_padding_rows": (c_int, [P, c_int, c_int, c_int, c_int, P, c_int, P]),
-    "moe_grouped_mlp_fp8_mapped": (c_int, [P, c_int, P, P, c_int, c_int, c_int, c_int, P, P, P, P, P, P, P, P, P, P, P, c_int, P, P]),
+    "moe_grouped_mlp_fp8_mapped": (c_int, [P, c_int, P, P, c_int, c_int, c_int, c_int, P, P, P, P, P, P, P, P, P, P, P, c_int, P, P,
+                                           c_size_t, P]),
     "moe_combine": (c_int, [P, c_int, c_int, c_int, c_int, P, P, P, P, c_int, c_int, c_int, P, P, P]),
 }
 

@@ -211,6 +211,11 @@ __device__ __forceinline__ int gg_lane_now() {
     return l;
 }
 
+// One dword per lane, HBM -> LDS: lane l's value lands at lds_addr + 4 l.
+__device__ __forceinline__ void gg_dma4(const uint8_t* sbase, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %1, %0" : : "s"(sbase), "v"(voff), "s"(lds_addr) : "memory");
+}
+
 // a wave-uniform value forced into scalar registers
 __device__ __forceinline__ const uint8_t* gg_uniform(const uint8_t* p) {
     const uint64_t v = (uint64_t)p;
@@ -271,6 +276,11 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     __shared__ __align__(1024) uint4 sB[NRING * BSLOT];
     __shared__ int g_tile_start[GG_MAXG + 1];
     __shared__ int g_row_start[GG_MAXG + 1];
+    // what the epilogue needs from global memory per tile row / tile column (fp8 scales, the output row map)
+    __shared__ __align__(16) float s_row_scale[BM];
+    __shared__ __align__(16) float s_col_scale[BN];
+    __shared__ int s_crow[BM];
+    static_assert(BM <= NWM * 2 * WAVE && BN <= NWM * 2 * WAVE, "one thread per tile row and per tile column");
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wave_s = __builtin_amdgcn_readfirstlane(wave);  // the same, known to be wave-uniform (a scalar register)
@@ -461,6 +471,31 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             // everything once per tile
             gg_wait<0, 15>();
             __syncthreads();
+            if constexpr (!SPLIT) {
+                // What the epilogue needs from global memory per tile row / column (fp8 scales, the output row map) is
+                // requested here, straight into LDS, one value per thread: every wave has left the previous tile's
+                // epilogue, the loads land during the first K stages (they are older than every load the K loop waits
+                // for), and no epilogue waits for a memory round trip.  No register holds anything across the K loop.
+                const int lane_t = gg_lane_now(), tid_t = wave_s * WAVE + lane_t;  // (a fresh lane id: nothing kept live for this)
+                const uint32_t t4 = (uint32_t)min(tid_t, rv - 1) * 4u;
+                if (wave_s * WAVE < BM) {
+                    if constexpr (FP8)
+                        gg_dma4(gg_uniform((const uint8_t*)(p.row_scale + row0)), t4,
+                                __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(s_row_scale + wave_s * WAVE)));
+                    if (p.c_map)
+                        gg_dma4(gg_uniform((const uint8_t*)(p.c_map + row0)), t4,
+                                __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(s_crow + wave_s * WAVE)));
+                }
+                if constexpr (FP8) {
+                    const int pc = nt * BN + tid_t;  // packed column of the launch; the lanes 32..63 of a wave hold up columns
+                    int col = EPI == EPI_SWIGLU ? (pc / 64) * 32 + pc % 32 : pc;
+                    col = col < p.N ? col : 0;  // (columns past N are never stored: any valid scale will do)
+                    const uint32_t lds_cs = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(s_col_scale + wave_s * WAVE));
+                    const uint32_t c4 = (uint32_t)col * 4u;
+                    if (EPI == EPI_SWIGLU && lane_t >= 32) gg_dma4(gg_uniform((const uint8_t*)(p.col_scale2 + (size_t)g * p.ncs)), c4, lds_cs);
+                    else gg_dma4(gg_uniform((const uint8_t*)(p.col_scale + (size_t)g * p.ncs)), c4, lds_cs);
+                }
+            }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -553,8 +588,8 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             ok[i] = r < rv;
             const size_t grow = (size_t)(row0 + (ok[i] ? r : 0));
             rs[i] = 1.f;
-            if constexpr (FP8) rs[i] = p.row_scale[grow];
-            const int crow_i = p.c_map ? p.c_map[grow] : 0;
+            if constexpr (FP8) rs[i] = s_row_scale[r];
+            const int crow_i = p.c_map ? s_crow[r] : 0;
             ok[i] = ok[i] && crow_i >= 0;  // a negative map entry: the row has no place in the output
             crow[i] = C + (p.c_map ? (size_t)max(crow_i, 0) : grow) * p.ldc + (DW ? (size_t)g * p.c_group_stride : (size_t)0);
         }
@@ -571,15 +606,15 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             }
             const int pcol = nt * BN + cbase_e + j * MT;  // first packed column of the tile
             const int colj = (EPI == EPI_SWIGLU ? (pcol / 64) * 32 + pcol % 32 : pcol) + clane;
-            if (FP8 && i == 0) {
+            if constexpr (FP8) {
+                // the column scales of the lane's columns, by packed column inside the tile (an LDS read: cheap enough
+                // to repeat for every row tile instead of holding eight vectors across them)
 #pragma unroll
                 for (int q = 0; q < NQ; ++q) {
-                    const int col = colj + 8 * q;
-                    sc0[q] = sc1[q] = make_float4(1.f, 1.f, 1.f, 1.f);
-                    if (col < p.N) {
-                        sc0[q] = *(const float4*)(p.col_scale + (size_t)g * p.ncs + col);
-                        if constexpr (EPI == EPI_SWIGLU) sc1[q] = *(const float4*)(p.col_scale2 + (size_t)g * p.ncs + col);
-                    }
+                    const int tc = cbase_e + j * MT + 8 * q + clane;
+                    sc0[q] = *(const float4*)(s_col_scale + tc);
+                    sc1[q] = make_float4(1.f, 1.f, 1.f, 1.f);
+                    if constexpr (EPI == EPI_SWIGLU) sc1[q] = *(const float4*)(s_col_scale + tc + 32);
                 }
             }
             {
@@ -1368,7 +1403,7 @@ extern "C" int moe_grouped_mlp_fp8_mapped(const void* a_base_bf16, int a_rows, c
                                           const uint8_t* wgu_packed, const float* sg, const float* su,
                                           const uint8_t* wd_packed, const float* sd, uint8_t* xq_ws, float* xs_ws, void* h_ws,
                                           uint8_t* hq_ws, float* hs_ws, void* out, int out_rows, const int32_t* c_row_map,
-                                          moe_stream_t stream) {
+                                          void* part_ws, size_t part_ws_bytes, moe_stream_t stream) {
     hipStream_t s = (hipStream_t)stream;
     MOE_REQUIRE(S_rows >= 0 && H > 0 && F > 0 && E_l > 0 && E_l <= GG_MAXG, MOE_ERR_INVALID, "grouped_mlp_fp8: bad shape");
     MOE_REQUIRE(H % 128 == 0 && F % 128 == 0, MOE_ERR_UNSUPPORTED, "grouped_mlp_fp8: needs H, F multiples of 128 (H=%d F=%d)", H, F);
@@ -1382,7 +1417,7 @@ extern "C" int moe_grouped_mlp_fp8_mapped(const void* a_base_bf16, int a_rows, c
     GemmParams p{};
     p.A = xq_ws; p.B = wgu_packed; p.C = h_ws; p.cnt = expert_cnt; p.row_scale = xs_ws; p.col_scale = sg; p.col_scale2 = su;
     p.E_l = E_l; p.K = H; p.N = F; p.Npad = round_up(2 * F, GG_BN); p.ldc = F; p.S_rows = S_rows; p.ncs = F;
-    rc = launch_gemm<true>(p, EPI_SWIGLU, s);
+    rc = launch_gemm<true>(p, EPI_SWIGLU, s, part_ws, part_ws_bytes);
     if (rc) return rc;
     rc = launch_quantize(h_ws, nullptr, S_rows, F, hq_ws, hs_ws, nullptr, s);
     if (rc) return rc;
@@ -1390,7 +1425,7 @@ extern "C" int moe_grouped_mlp_fp8_mapped(const void* a_base_bf16, int a_rows, c
     q.A = hq_ws; q.B = wd_packed; q.C = out; q.cnt = expert_cnt; q.row_scale = hs_ws; q.col_scale = sd;
     q.c_map = c_row_map;
     q.E_l = E_l; q.K = F; q.N = H; q.Npad = round_up(H, GG_BN); q.ldc = H; q.S_rows = S_rows; q.ncs = H;
-    return launch_gemm<true>(q, EPI_NONE, s);
+    return launch_gemm<true>(q, EPI_NONE, s, part_ws, part_ws_bytes);
 }
 
 extern "C" int moe_grouped_mlp_fp8(const void* tokens_bf16, const int32_t* expert_cnt, int S_rows, int H, int F, int E_l,
@@ -1398,7 +1433,7 @@ extern "C" int moe_grouped_mlp_fp8(const void* tokens_bf16, const int32_t* exper
                                    const float* sd, uint8_t* xq_ws, float* xs_ws, void* h_ws, uint8_t* hq_ws, float* hs_ws,
                                    void* out, moe_stream_t stream) {
     return moe_grouped_mlp_fp8_mapped(tokens_bf16, S_rows, nullptr, expert_cnt, S_rows, H, F, E_l, wgu_packed, sg, su, wd_packed,
-                                      sd, xq_ws, xs_ws, h_ws, hq_ws, hs_ws, out, S_rows, nullptr, stream);
+                                      sd, xq_ws, xs_ws, h_ws, hq_ws, hs_ws, out, S_rows, nullptr, nullptr, 0, stream);
 }
 
 // ---- backward pass entry points --------------------------------------------------------------------------------------

@@ -317,7 +317,8 @@ def quantize_rows_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
 
 
 def grouped_mlp_fp8(tokens: torch.Tensor, expert_cnt: torch.Tensor, F: int, wgu_packed, sg, su, wd_packed, sd,
-                    ws: Optional[dict] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    ws: Optional[dict] = None, out: Optional[torch.Tensor] = None,
+                    part_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
     _req_cuda(tokens, "tokens")
     assert tokens.dtype == torch.bfloat16
     S, H = tokens.shape
@@ -327,9 +328,16 @@ def grouped_mlp_fp8(tokens: torch.Tensor, expert_cnt: torch.Tensor, F: int, wgu_
         ws = fp8_workspace(S, H, F, dev)
     if out is None:
         out = torch.zeros((S, H), dtype=torch.bfloat16, device=dev)
-    L.check(L.lib().moe_grouped_mlp_fp8(L.ptr(tokens), L.ptr(expert_cnt), S, H, F, E_l, L.ptr(wgu_packed), L.ptr(sg),
-                                        L.ptr(su), L.ptr(wd_packed), L.ptr(sd), L.ptr(ws["xq"]), L.ptr(ws["xs"]),
-                                        L.ptr(ws["h"]), L.ptr(ws["hq"]), L.ptr(ws["hs"]), L.ptr(out), L.stream_ptr()))
+    if part_ws is None:
+        L.check(L.lib().moe_grouped_mlp_fp8(L.ptr(tokens), L.ptr(expert_cnt), S, H, F, E_l, L.ptr(wgu_packed), L.ptr(sg),
+                                            L.ptr(su), L.ptr(wd_packed), L.ptr(sd), L.ptr(ws["xq"]), L.ptr(ws["xs"]),
+                                            L.ptr(ws["h"]), L.ptr(ws["hq"]), L.ptr(ws["hs"]), L.ptr(out), L.stream_ptr()))
+    else:  # with the K-split scratch (gemm_part_workspace): an under-filled last round of tiles is cut along K
+        L.check(L.lib().moe_grouped_mlp_fp8_mapped(L.ptr(tokens), S, None, L.ptr(expert_cnt), S, H, F, E_l, L.ptr(wgu_packed),
+                                                   L.ptr(sg), L.ptr(su), L.ptr(wd_packed), L.ptr(sd), L.ptr(ws["xq"]),
+                                                   L.ptr(ws["xs"]), L.ptr(ws["h"]), L.ptr(ws["hq"]), L.ptr(ws["hs"]), L.ptr(out), S,
+                                                   None, L.ptr(part_ws), part_ws.numel() * part_ws.element_size(),
+                                                   L.stream_ptr()))
     return out
 
 

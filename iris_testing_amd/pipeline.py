@@ -64,8 +64,8 @@ class DispatchPipeline:
         self.ret = torch.empty((W, M, H), dtype=dt, device=dev)
         self.ret_map = i32(lib.moe_recv_map_ints(W, E_l, W * M))
         self.row_map = i32(max(S, 1))
-        # scratch for the K-split of an under-filled last round of GEMM tiles (bf16 experts)
-        self.part_ws_bytes = lib.moe_gemm_part_workspace_bytes() if weights.dtype == torch.bfloat16 else 0
+        # scratch for the K-split of an under-filled last round of GEMM tiles (bf16 and fp8 experts)
+        self.part_ws_bytes = lib.moe_gemm_part_workspace_bytes() if weights.dtype in (torch.bfloat16, torch.uint8) else 0
         self.part_ws = torch.empty(self.part_ws_bytes // 4, dtype=torch.float32, device=dev) if self.part_ws_bytes else None
         if weights.dtype == torch.uint8:
             self.xq = torch.empty((S, H), dtype=torch.uint8, device=dev)
@@ -112,20 +112,16 @@ class DispatchPipeline:
         lib = L.lib()
         if ew.dtype == torch.uint8:
             sg, su, sd = ew.scales
-            # the fp8 entry point runs quantise + gate/up + quantise + down in one call
-            if self.fused:
-                w = self.world
-                L.check(lib.moe_grouped_mlp_fp8_mapped(self._p(w.recv), c.world * w.M, self._p(self.row_map),
-                                                       self._p(self.expert_cnt), self.S, c.hidden, c.ffn, c.e_local,
-                                                       self._p(ew.w1), self._p(sg), self._p(su), self._p(ew.w2), self._p(sd),
-                                                       self._p(self.xq), self._p(self.xs), self._p(self.hidden), self._p(self.hq),
-                                                       self._p(self.hs), self._p(self.ret), c.world * w.M,
-                                                       self._p(self.row_map), s))
-                return
-            L.check(lib.moe_grouped_mlp_fp8(self._p(self.rows), self._p(self.expert_cnt), self.S, c.hidden, c.ffn, c.e_local,
-                                            self._p(ew.w1), self._p(sg), self._p(su), self._p(ew.w2), self._p(sd),
-                                            self._p(self.xq), self._p(self.xs), self._p(self.hidden), self._p(self.hq),
-                                            self._p(self.hs), self._p(self.y), s))
+            # the fp8 entry point runs quantise + gate/up + quantise + down in one call; fused: input rows gathered from
+            # the receive buffer, result rows scattered into the returned layout
+            w = self.world
+            src, n_src, a_map = (w.recv, c.world * w.M, self.row_map) if self.fused else (self.rows, self.S, None)
+            dst, n_dst, c_map = (self.ret, c.world * w.M, self.row_map) if self.fused else (self.y, self.S, None)
+            L.check(lib.moe_grouped_mlp_fp8_mapped(self._p(src), n_src, self._p(a_map), self._p(self.expert_cnt), self.S, c.hidden,
+                                                   c.ffn, c.e_local, self._p(ew.w1), self._p(sg), self._p(su), self._p(ew.w2),
+                                                   self._p(sd), self._p(self.xq), self._p(self.xs), self._p(self.hidden),
+                                                   self._p(self.hq), self._p(self.hs), self._p(dst), n_dst, self._p(c_map),
+                                                   self._p(self.part_ws), self.part_ws_bytes, s))
         elif ew.dtype == torch.float32:
             L.check(lib.moe_grouped_mlp(self._p(self.rows), self._p(self.expert_cnt), self.code, self.S, c.hidden, c.ffn,
                                         c.e_local, L.ACT[ew.act], self._p(ew.w1), self._p(ew.w_up), self._p(ew.w2),

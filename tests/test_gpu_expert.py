@@ -286,3 +286,42 @@ def test_expert_mlp_fp8(E_l, H, F, S):
     # against the unquantised fp32 MLP, to show what the quantisation itself costs (reported only)
     ref = O.expert_mlp(x, cnt, wg, wd, "swiglu", "f32", w_up=wu)
     print("fp8 vs unquantised fp32 MLP:", err_stats(out, ref.astype(np.float64)), flush=True)
+
+
+@pytest.mark.parametrize("E_l,H,F,rows", [(2, 2048, 1408, (300, 220)), (1, 512, 1024, (450,)), (3, 1024, 2048, (130, 0, 260))])
+def test_expert_mlp_fp8_k_split_of_the_last_round(E_l, H, F, rows):
+    """The fp8 GEMMs with the partial-sum workspace: few tiles on an otherwise idle chip are cut along K and summed by the
+    reduction kernel, which applies the same scales and epilogue.  Each GEMM is held to the oracle on its own inputs
+    (as in test_expert_mlp_fp8), the result is reproducible from call to call whatever the workspace held, and it is
+    within a rounding step of the unsplit kernels'."""
+    rng = np.random.default_rng(H + F + E_l)
+    cnt = np.array(rows, dtype=np.int32)
+    S_tot = int(cnt.sum())
+    x = _randn(rng, S_tot, H)
+    wg, wu = _randn(rng, E_l, H, F, scale=H ** -0.5), _randn(rng, E_l, H, F, scale=H ** -0.5)
+    wd = _randn(rng, E_l, F, H, scale=F ** -0.5)
+    (gq, gs), (uq, us), (dq, ds) = (O.quantize_cols_fp8(w) for w in (wg, wu, wd))
+    tq = lambda a: torch.from_numpy(a).to(DEV)  # noqa: E731
+    ew = ExpertWeights.prepare_fp8(tq(gq), tq(gs), tq(uq), tq(us), tq(dq), tq(ds))
+    sg, su, sd = ew.scales
+    cnt_t, x_t = torch.from_numpy(cnt).to(DEV), _t(x, "bf16")
+    plain_ws = ops.fp8_workspace(S_tot, H, F, DEV)
+    plain = ops.grouped_mlp_fp8(x_t, cnt_t, F, ew.w1, sg, su, ew.w2, sd, ws=plain_ws)
+    part = ops.gemm_part_workspace(DEV)
+    outs = []
+    for fill in (float("nan"), 3.0):
+        part.fill_(fill)
+        ws = ops.fp8_workspace(S_tot, H, F, DEV)
+        outs.append((ops.grouped_mlp_fp8(x_t, cnt_t, F, ew.w1, sg, su, ew.w2, sd, ws=ws, part_ws=part).clone(), ws))
+    torch.cuda.synchronize()
+    (split, ws1), (again, _) = outs
+    assert torch.equal(split.view(torch.int16), again.view(torch.int16)), "the fp8 K split is not reproducible"
+    assert bool(torch.isfinite(split.float()).all())
+    h_gpu = to_np(ws1["h"])
+    _check(h_gpu, O.expert_up_fp8(x, cnt, gq, gs, uq, us).astype(np.float64), BF16_RTOL, BF16_ATOL, "fp8 gate/up, K split")
+    _check(to_np(split), O.expert_down_fp8(h_gpu, cnt, dq, ds).astype(np.float64), BF16_RTOL, BF16_ATOL, "fp8 down, K split")
+    # against the unsplit kernels: the hidden activations within a rounding step (fp32 summation order)
+    a, b = ws1["h"].float(), plain_ws["h"].float()
+    assert bool(((a - b).abs() <= 2.0 ** -6 * torch.maximum(a.abs(), b.abs()) + 1e-6).all())
+    differs = int((ws1["h"].view(torch.int16) != plain_ws["h"].view(torch.int16)).sum().item())
+    print(f"fp8 K split: {differs} of {a.numel()} hidden activations differ in the last bits from the unsplit kernel", flush=True)
