@@ -90,6 +90,28 @@ __host__ __device__ inline GgPlan gg_plan(int total, int grid, int nk, bool spli
     return pl;
 }
 
+// Where a packed weight column sits inside its aligned group of 32 rows of the packed matrix.  The MFMA leaves a lane
+// with runs of FOUR consecutive rows of the weight operand (bf16 16x16: rows 4q .. 4q+3 of a tile for the lanes 16q ..
+// 16q+15; fp8 32x32: rows 8Q + 4h .. + 3 for the register quad Q and the lanes 32h .. 32h+31).  The rows of a group are
+// ordered so that two of a lane's runs are EIGHT consecutive output columns, which leave as one 16-byte store:
+//   bf16: column 8q + 4t + v of the group (t = 0, 1: the group's two MFMA tiles) at row 16t + 4q + v;
+//   fp8 : column 16P + 8h + 4t + v (P = 0, 1; quads 2P + t) at row 8 (2P + t) + 4h + v.
+// Runs of four columns that start at a multiple of four stay runs of four rows.
+template <bool FP8>
+__host__ __device__ inline int gg_col_to_row32(int c) {  // c in [0, 32)
+    if (FP8) return ((c >> 4) * 2 + ((c >> 2) & 1)) * 8 + ((c >> 3) & 1) * 4 + (c & 3);
+    return ((c >> 2) & 1) * 16 + (c >> 3) * 4 + (c & 3);
+}
+template <bool FP8>
+__host__ __device__ inline int gg_row_to_col32(int r) {  // the inverse
+    if (FP8) return (r >> 4) * 16 + ((r >> 2) & 1) * 8 + ((r >> 3) & 1) * 4 + (r & 3);
+    return ((r >> 2) & 3) * 8 + (r >> 4) * 4 + (r & 3);
+}
+template <bool FP8>
+__host__ __device__ inline int gg_packed_row(int col) { return (col & ~31) | gg_col_to_row32<FP8>(col & 31); }
+template <bool FP8>
+__host__ __device__ inline int gg_packed_col(int row) { return (row & ~31) | gg_row_to_col32<FP8>(row & 31); }
+
 // x * sigmoid(x) with the hardware reciprocal (1 ulp) instead of an IEEE division: the SwiGLU epilogue of a
 // 128 x 128 wave tile evaluates this 8192 times per lane-row, and the division was most of its cost
 // two fp32 -> packed bf16 (round to nearest even) in one hardware conversion
@@ -160,23 +182,51 @@ __device__ __forceinline__ GgTile gg_decode(const int* g_tile_start, const int* 
     return t;
 }
 
-// next non-empty tile of this workgroup at or after round `base` (base is advanced past it)
-// SPLIT = false walks the whole tiles [0, full); SPLIT = true walks the parts of the tiles [full, total): unit q
-// is part q % P of tile full + q / P.
-template <int BM, bool SPLIT, bool DW = false>
-__device__ __forceinline__ GgTile gg_next_tile(const int* g_tile_start, const int* g_row_start, int E_l, int Nt, int S_rows,
-                                               const GgPlan& pl, int nk, int my, int stride, int& base, int dw_rows = 0) {
+// The tiles of a workgroup, in the order it walks them: round r of the persistent grid gives it tile r * stride + my.
+// Decoding one costs a search and five integer divisions, so the workgroup decodes GG_TT of them at a time, one per
+// thread, into a table in LDS; the walk itself is then one 16-byte LDS read per tile.
+constexpr int GG_TT = 256;
+template <int BM, bool SPLIT, bool DW>
+__device__ __forceinline__ void gg_fill_table(int4* s_tiles, const int* g_tile_start, const int* g_row_start, int E_l, int Nt,
+                                              int S_rows, const GgPlan& pl, int my, int stride, int round0, int dw_rows) {
+    const int n = SPLIT ? pl.units - pl.full : pl.full;
+    for (int i = threadIdx.x; i < GG_TT; i += blockDim.x) {
+        const int lin = (round0 + i) * stride + my;
+        int4 e = make_int4(0, 0, 0, 0);  // (g, nt, row0, rv); rv <= 0: nothing there
+        if ((round0 + i) < (n + stride - 1) / stride && lin < n) {
+            const GgTile t = gg_decode<BM, DW>(g_tile_start, g_row_start, E_l, Nt, S_rows, SPLIT ? pl.full + lin / pl.P : lin, dw_rows);
+            e = make_int4(t.g, t.nt, t.row0, t.rv);
+        }
+        s_tiles[i] = e;
+    }
+}
+
+// Next non-empty tile of this workgroup at or after round `round` (advanced past it); rv = 0 when there is none.
+// round0 is the round the table starts at; the table is refilled (by the whole workgroup: every wave makes the same
+// calls) when the walk leaves it.
+template <int BM, bool SPLIT, bool DW>
+__device__ __forceinline__ GgTile gg_walk(int4* s_tiles, const int* g_tile_start, const int* g_row_start, int E_l, int Nt, int S_rows,
+                                          const GgPlan& pl, int nk, int my, int stride, int& round, int& round0, int dw_rows) {
     GgTile t;
     t.g = t.nt = t.row0 = 0;
     t.rv = 0;
     t.ks0 = 0; t.nks = nk; t.unit = -1;
     const int n = SPLIT ? pl.units - pl.full : pl.full;
-    while (base < n) {
-        const int lin = base + my;
-        base += stride;
-        if (lin < n) {
-            t = gg_decode<BM, DW>(g_tile_start, g_row_start, E_l, Nt, S_rows, SPLIT ? pl.full + lin / pl.P : lin, dw_rows);
-            t.ks0 = 0; t.nks = nk; t.unit = -1;
+    const int rounds = (n + stride - 1) / stride;
+    while (round < rounds) {
+        if (round >= round0 + GG_TT) {
+            __syncthreads();  // (every wave has read what it needed of the old table)
+            round0 = round;
+            gg_fill_table<BM, SPLIT, DW>(s_tiles, g_tile_start, g_row_start, E_l, Nt, S_rows, pl, my, stride, round0, dw_rows);
+            __syncthreads();
+        }
+        const int4 e = s_tiles[round - round0];
+        const int lin = round * stride + my;
+        ++round;
+        const int rv = __builtin_amdgcn_readfirstlane(e.w);
+        if (rv > 0) {
+            t.g = __builtin_amdgcn_readfirstlane(e.x); t.nt = __builtin_amdgcn_readfirstlane(e.y);
+            t.row0 = __builtin_amdgcn_readfirstlane(e.z); t.rv = rv;
             if constexpr (DW) {
                 t.ks0 = g_row_start[t.g];
                 t.nks = g_row_start[t.g + 1] - t.ks0;
@@ -186,7 +236,7 @@ __device__ __forceinline__ GgTile gg_next_tile(const int* g_tile_start, const in
                 t.nks = min(pl.nkp, nk - t.ks0);
                 t.unit = lin;
             }
-            if (t.rv > 0) break;
+            break;
         }
     }
     return t;
@@ -280,6 +330,8 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     __shared__ __align__(16) float s_row_scale[BM];
     __shared__ __align__(16) float s_col_scale[BN];
     __shared__ int s_crow[BM];
+    __shared__ int s_amap[BM];              // the NEXT tile's input rows (a_map), fetched while this one is multiplied
+    __shared__ __align__(16) int4 s_tiles[GG_TT];
     static_assert(BM <= NWM * 2 * WAVE && BN <= NWM * 2 * WAVE, "one thread per tile row and per tile column");
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -341,7 +393,9 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 #pragma unroll
     for (int r = 0; r < RB; ++r) b_off[r] = (uint32_t)(r * LR + lrow) * ROWB + lchunk * 16;
 
-#define GG_TILE_PTRS(t, Ab_, Bb_, aoff_)                                                                   \
+#define GG_MAPROW_GLOBAL(t, l) p.a_map[(t).row0 + (l)]   /* the first tile: straight from memory */
+#define GG_MAPROW_LDS(t, l) s_amap[(l)]                  /* later tiles: fetched into LDS one tile ahead */
+#define GG_TILE_PTRS(t, Ab_, Bb_, aoff_, MAPROW_)                                                          \
     const uint8_t* Ab_ = (p.a_map ? p.A : p.A + (size_t)(t).row0 * p.K * ES) + (size_t)(t).ks0 * ROWB;      \
     const uint8_t* Bb_ = p.B + (DW ? (size_t)0 : (size_t)(t).g * p.Npad * p.K * ES) + (size_t)(t).nt * BN * ROWB + (size_t)(t).ks0 * b_slab; \
     uint32_t aoff_[RA];                                                                                     \
@@ -350,7 +404,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     const uint32_t lcb_ = (uint32_t)(((ln_ & 3) ^ ((ln_ >> 4) & 3)) * 16);                                     \
     _Pragma("unroll") for (int r = 0; r < RA; ++r) {                                                         \
         const int lr_ = max(min(r * LR + lrow_, (t).rv - 1), 0);  /* tile row this lane fetches, clamped */    \
-        aoff_[r] = (uint32_t)(p.a_map ? max(p.a_map[(t).row0 + lr_], 0) : lr_) * ldk + lcb_;                  \
+        aoff_[r] = (uint32_t)(p.a_map ? max(MAPROW_(t, lr_), 0) : lr_) * ldk + lcb_;                       \
     }
     // load d (0 .. LPS-1) of one stage: A rounds first, then B rounds
 #define GG_LD(d, ap_, bp_, aoff_, slot)                                                                       \
@@ -386,12 +440,14 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 3, 3, 0, LPS, nks_);  \
     } while (0)
 
-    int base = 0;
-    GgTile cur = gg_next_tile<BM, SPLIT, DW>(g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, plan, nk, my, gridDim.x, base, p.dw_rows);
+    int round = 0, round0 = 0;
+    gg_fill_table<BM, SPLIT, DW>(s_tiles, g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, plan, my, (int)gridDim.x, 0, p.dw_rows);
+    __syncthreads();
+    GgTile cur = gg_walk<BM, SPLIT, DW>(s_tiles, g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, plan, nk, my, (int)gridDim.x, round, round0, p.dw_rows);
     uint32_t a_off[RA];
     const uint8_t *Ab = p.A, *Bb = p.B;
     if (cur.rv > 0) {
-        GG_TILE_PTRS(cur, Ab0, Bb0, a_off0);
+        GG_TILE_PTRS(cur, Ab0, Bb0, a_off0, GG_MAPROW_GLOBAL);
         Ab = Ab0;
         Bb = Bb0;
 #pragma unroll
@@ -471,6 +527,17 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             // everything once per tile
             gg_wait<0, 15>();
             __syncthreads();
+            if (p.a_map) {
+                // the input rows of the NEXT tile, one per thread, straight into LDS: the tile set-up at the end of this
+                // tile's K loop then reads them from there instead of waiting for memory with the matrix pipes idle
+                int round_pk = round;  // (a look ahead: the walk itself advances at the end of the K loop)
+                const GgTile pk = gg_walk<BM, SPLIT, DW>(s_tiles, g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, plan, nk, my, (int)gridDim.x, round_pk, round0, p.dw_rows);
+                if (pk.rv > 0 && wave_s * WAVE < BM) {
+                    const int tid_a = wave_s * WAVE + gg_lane_now();
+                    gg_dma4(gg_uniform((const uint8_t*)(p.a_map + pk.row0)), (uint32_t)min(tid_a, pk.rv - 1) * 4u,
+                            __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(s_amap + wave_s * WAVE)));
+                }
+            }
             if constexpr (!SPLIT) {
                 // What the epilogue needs from global memory per tile row / column (fp8 scales, the output row map) is
                 // requested here, straight into LDS, one value per thread: every wave has left the previous tile's
@@ -487,7 +554,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                                 __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(s_crow + wave_s * WAVE)));
                 }
                 if constexpr (FP8) {
-                    const int pc = nt * BN + tid_t;  // packed column of the launch; the lanes 32..63 of a wave hold up columns
+                    const int pc = gg_packed_col<true>(nt * BN + tid_t);  // packed column of the launch behind this row of the weight tile; the lanes 32..63 of a wave hold up columns
                     int col = EPI == EPI_SWIGLU ? (pc / 64) * 32 + pc % 32 : pc;
                     col = col < p.N ? col : 0;  // (columns past N are never stored: any valid scale will do)
                     const uint32_t lds_cs = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(s_col_scale + wave_s * WAVE));
@@ -527,8 +594,8 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 
         // ---- next tile: decode it and request its first stages now (every slot is free once all waves
         // have passed the barrier: the last fragments of this tile are already in registers)
-        const GgTile nxt = gg_next_tile<BM, SPLIT, DW>(g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, plan, nk, my, gridDim.x, base, p.dw_rows);
-        GG_TILE_PTRS(nxt, Ab_n, Bb_n, a_off_n);
+        const GgTile nxt = gg_walk<BM, SPLIT, DW>(s_tiles, g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, plan, nk, my, (int)gridDim.x, round, round0, p.dw_rows);
+        GG_TILE_PTRS(nxt, Ab_n, Bb_n, a_off_n, GG_MAPROW_LDS);
         if (nxt.rv > 0) {
             __syncthreads();
             GG_PROLOGUE(Ab_n, Bb_n, a_off_n, (VARK ? nxt.nks : nk));
@@ -566,19 +633,20 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 
         // ---- epilogue: acc -> (scales) -> activation -> bf16 -> C
         // acc(i,j) holds the TRANSPOSED MT x MT product (weights as the MFMA A operand, activations as B):
-        // a lane owns one token row of the tile and runs of four consecutive output columns -> 8-byte stores.
-        //   bf16 (16x16): row l % 16, columns 4 * (l / 16) + v, v = 0..3
-        //   fp8  (32x32): row l % 32, columns 8 * q + 4 * (l / 32) + v for the four register quads q
-        // SwiGLU: packed columns alternate gate / up in groups of 32, so the gate tile and its up tile lie
-        // 32 packed columns apart and land on output column (packed column of the gate) / 2 + ... .
-        // Column tiles are walked outermost: the fp8 per-channel scales of a column tile are fetched once and
-        // serve the wave's TM row tiles.
+        // a lane owns one token row of the tile and runs of four consecutive rows of the weight tile
+        //   bf16 (16x16): token row l % 16, weight rows 4 * (l / 16) + v, v = 0..3
+        //   fp8  (32x32): token row l % 32, weight rows 8 * q + 4 * (l / 32) + v for the four register quads q
+        // and the rows of a group of 32 packed columns are ordered (gg_col_to_row32) so that two of those runs are
+        // eight consecutive output columns -> 16-byte stores.
+        // SwiGLU: packed columns alternate gate / up in groups of 32, so a gate group and its up group lie
+        // 32 packed columns apart and land on output column (packed column of the gate group) / 2 + ... .
         bf16_t* C = (bf16_t*)p.C;
-        constexpr int NQ = FP8 ? 4 : 1;              // runs of four columns per lane and tile
-        constexpr int UPJ = 32 / MT;                 // tiles between a gate tile and its up tile
+        constexpr int GT = 32 / MT;                  // MFMA tiles per group of 32 packed columns
+        constexpr int NG = TN / GT;                  // groups per wave (its 128 packed columns)
+        constexpr int NU = FP8 ? 2 : 1;              // 16-byte stores per lane and group
         // (the lane-derived constants of the epilogue are derived here, once per tile, from a fresh read of the lane id)
         const int lane_e = gg_lane_now(), rbase_e = (wave_s >> 1) * (BM / NWM), cbase_e = (wave_s & 1) * (BN / 2);
-        const int clane = FP8 ? (lane_e >> 5) * 4 : (lane_e >> 4) * 4;  // first column of the lane's run inside 8 (fp8) / 16 (bf16) columns
+        const int lsub = FP8 ? (lane_e >> 5) : (lane_e >> 4);  // which of the lanes that share a tile row this one is
         bool ok[TM];
         bf16_t* crow[TM];
         float rs[TM];
@@ -593,71 +661,65 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             ok[i] = ok[i] && crow_i >= 0;  // a negative map entry: the row has no place in the output
             crow[i] = C + (p.c_map ? (size_t)max(crow_i, 0) : grow) * p.ldc + (DW ? (size_t)g * p.c_group_stride : (size_t)0);
         }
-        float4 sc0[NQ], sc1[NQ];  // fp8: channel scales of the lane's columns (gate / only; up)
 #pragma unroll
-        for (int o = 0; o < TM * TN; ++o) {
-            // fp8: column tiles outermost (the channel scales of a column tile are fetched once and serve the
-            // wave's TM row tiles); bf16: row tiles outermost, so that the stores of one row tile fill whole
+        for (int o = 0; o < TM * NG; ++o) {
+            // fp8: column groups outermost; bf16: row tiles outermost, so that the stores of one row tile fill whole
             // cache lines back to back (the other order wrote 50 % more bytes to memory: lines left the L2
             // half written)
-            const int i = FP8 ? o % TM : o / TN, j = FP8 ? o / TM : o % TN;
+            const int i = FP8 ? o % TM : o / NG, jg = FP8 ? o / TM : o % NG;
             if constexpr (EPI == EPI_SWIGLU) {
-                if ((j / UPJ) % 2 == 1) continue;  // an up tile: consumed together with its gate tile
+                if (jg % 2 == 1) continue;  // an up group: consumed together with its gate group
             }
-            const int pcol = nt * BN + cbase_e + j * MT;  // first packed column of the tile
-            const int colj = (EPI == EPI_SWIGLU ? (pcol / 64) * 32 + pcol % 32 : pcol) + clane;
-            if constexpr (FP8) {
-                // the column scales of the lane's columns, by packed column inside the tile (an LDS read: cheap enough
-                // to repeat for every row tile instead of holding eight vectors across them)
+            const int pcol = nt * BN + cbase_e + jg * 32;  // first packed column of the group
+            const int colg = EPI == EPI_SWIGLU ? (pcol / 64) * 32 : pcol;  // its first output column
 #pragma unroll
-                for (int q = 0; q < NQ; ++q) {
-                    const int tc = cbase_e + j * MT + 8 * q + clane;
-                    sc0[q] = *(const float4*)(s_col_scale + tc);
-                    sc1[q] = make_float4(1.f, 1.f, 1.f, 1.f);
-                    if constexpr (EPI == EPI_SWIGLU) sc1[q] = *(const float4*)(s_col_scale + tc + 32);
-                }
-            }
-            {
+            for (int u = 0; u < NU; ++u) {
+                // the lane's eight consecutive columns: two runs of four accumulators (bf16: the group's two tiles;
+                // fp8: the register quads 2u and 2u + 1 of the group's one tile)
+                const int col = colg + (FP8 ? 16 * u : 0) + 8 * lsub;
+                float x[8];
 #pragma unroll
-                for (int q = 0; q < NQ; ++q) {
-                    const int col = colj + 8 * q;
-                    float x[4];
-                    if constexpr (EPI == EPI_SWIGLU) {
-                        constexpr int ju_ = UPJ;  // offset of the up tile
-                        float cg[4] = {1.f, 1.f, 1.f, 1.f}, cu[4] = {1.f, 1.f, 1.f, 1.f};
-                        if constexpr (FP8) {
-                            cg[0] = sc0[q].x; cg[1] = sc0[q].y; cg[2] = sc0[q].z; cg[3] = sc0[q].w;
-                            cu[0] = sc1[q].x; cu[1] = sc1[q].y; cu[2] = sc1[q].z; cu[3] = sc1[q].w;
-                        }
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            float gv = acc[i][j][4 * q + e], uv = acc[i][(j + ju_) % TN][4 * q + e];
-                            if constexpr (FP8) { gv *= cg[e] * rs[i]; uv *= cu[e] * rs[i]; }
-                            x[e] = act_silu_fast(gv) * uv;
-                        }
-                    } else {
-                        float cs[4] = {1.f, 1.f, 1.f, 1.f};
-                        if constexpr (FP8) { cs[0] = sc0[q].x; cs[1] = sc0[q].y; cs[2] = sc0[q].z; cs[3] = sc0[q].w; }
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            float v = acc[i][j][4 * q + e];
-                            if constexpr (FP8) v *= cs[e] * rs[i];
-                            if constexpr (EPI == EPI_GELU) v = act_gelu(v);
-                            if constexpr (EPI == EPI_SILU) v = act_silu_fast(v);
-                            x[e] = v;
+                for (int t = 0; t < 2; ++t) {
+                    const int j = FP8 ? jg : jg * GT + t;       // MFMA tile of the run
+                    const int qd = FP8 ? 2 * u + t : 0;         // its register quad
+                    const int ju = j + GT;                      // SwiGLU: the up tile (32 packed columns further)
+                    float cg[4] = {1.f, 1.f, 1.f, 1.f}, cu[4] = {1.f, 1.f, 1.f, 1.f};
+                    if constexpr (FP8) {
+                        // channel scales by row of the weight tile (an LDS read: cheap enough to repeat for every row tile)
+                        const int tc = cbase_e + j * MT + 8 * qd + 4 * lsub;
+                        const float4 s0 = *(const float4*)(s_col_scale + tc);
+                        cg[0] = s0.x; cg[1] = s0.y; cg[2] = s0.z; cg[3] = s0.w;
+                        if constexpr (EPI == EPI_SWIGLU) {
+                            const float4 s1 = *(const float4*)(s_col_scale + tc + 32);
+                            cu[0] = s1.x; cu[1] = s1.y; cu[2] = s1.z; cu[3] = s1.w;
                         }
                     }
-                    if (ok[i] && col < p.N) {
-                        uint2 o;
-                        o.x = gg_pack_bf16(x[0], x[1]);
-                        o.y = gg_pack_bf16(x[2], x[3]);
-                        *(uint2*)(crow[i] + col) = o;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        float v = acc[i][j][4 * qd + e];
+                        if constexpr (FP8) v *= cg[e] * rs[i];
+                        if constexpr (EPI == EPI_SWIGLU) {
+                            float uv = acc[i][ju % TN][4 * qd + e];
+                            if constexpr (FP8) uv *= cu[e] * rs[i];
+                            v = act_silu_fast(v) * uv;
+                        }
+                        if constexpr (EPI == EPI_GELU) v = act_gelu(v);
+                        if constexpr (EPI == EPI_SILU) v = act_silu_fast(v);
+                        x[4 * t + e] = v;
                     }
                 }
-                // keep the accumulator read-out of one tile from being hoisted over the previous tile's stores
-                // (that would need every accumulator in a VGPR at once)
-                if (FP8 || (o % 2 == 1)) __builtin_amdgcn_sched_barrier(0);
+                if (ok[i] && col < p.N) {
+                    uint4 o4;
+                    o4.x = gg_pack_bf16(x[0], x[1]);
+                    o4.y = gg_pack_bf16(x[2], x[3]);
+                    o4.z = gg_pack_bf16(x[4], x[5]);
+                    o4.w = gg_pack_bf16(x[6], x[7]);
+                    *(uint4*)(crow[i] + col) = o4;
+                }
             }
+            // keep the accumulator read-out of one group from being hoisted over the previous group's stores
+            // (that would need every accumulator in a VGPR at once)
+            __builtin_amdgcn_sched_barrier(0);
         }
         cur = nxt;
         Ab = Ab_n;
@@ -666,6 +728,8 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         for (int r = 0; r < RA; ++r) a_off[r] = a_off_n[r];
     }
 #undef GG_TILE_PTRS
+#undef GG_MAPROW_GLOBAL
+#undef GG_MAPROW_LDS
 #undef GG_LD
 #undef GG_STAGE_PTRS
 #undef GG_ISSUE_RANGE
@@ -719,7 +783,7 @@ __global__ __launch_bounds__(256) void gg_reduce_parts_kernel(const GemmParams p
     bf16_t* C = (bf16_t*)p.C;
     const int r_end = min((slab + 1) * (BM / RSL), t.rv);
     for (int r = slab * (BM / RSL) + threadIdx.x / OC4; r < r_end; r += RPP) {
-        const float* w = ws + (size_t)r * BN + pc;
+        const float* w = ws + (size_t)r * BN + gg_packed_row<FP8>(pc);  // (parts are stored by row of the weight tile)
         float4 a = *(const float4*)w, b = make_float4(0.f, 0.f, 0.f, 0.f);
         if constexpr (EPI == EPI_SWIGLU) b = *(const float4*)(w + 32);
         for (int part = 1; part < plan.P; ++part) {
@@ -784,10 +848,12 @@ __global__ __launch_bounds__(256) void prepack_kernel(const T* __restrict__ w, c
         for (int i = threadIdx.x; i < 64 * 64; i += 256) {
             const int nn = i / 64, kk = i % 64;
             const int n = n0 + nn;
-            if (n < N && k0 + kk < K) {
-                const int np = src2 ? ((n >> 5) * 64 + pass * 32 + (n & 31)) : n;
+            // (columns [N, next multiple of 64) leave as the zeros they were loaded as: the rows of a group of 32 are
+            // permuted, so a partly filled group cannot be zeroed as a range of rows)
+            const int np = src2 ? ((n >> 5) * 64 + pass * 32 + (n & 31)) : n;
+            if ((n < N || (!src2 && np < Npad)) && k0 + kk < K) {
                 const int k = k0 + kk;
-                dst[((size_t)(k / SK) * Npad + np) * SK + (k % SK)] = tile[kk][nn];
+                dst[((size_t)(k / SK) * Npad + gg_packed_row<sizeof(T) == 1>(np)) * SK + (k % SK)] = tile[kk][nn];
             }
         }
         __syncthreads();
@@ -796,7 +862,7 @@ __global__ __launch_bounds__(256) void prepack_kernel(const T* __restrict__ w, c
 
 template <typename T>
 __global__ void zero_pad_rows_kernel(T* __restrict__ out, int K, int Nreal, int Npad) {
-    // rows [Nreal, Npad) of every K slab of every expert's packed matrix
+    // rows [Nreal, Npad) of every K slab of every expert's packed matrix (Nreal a multiple of 32: whole groups)
     constexpr int SK = ROWB / (int)sizeof(T);
     const int e = blockIdx.y;
     const size_t per_slab = (size_t)(Npad - Nreal) * SK;
@@ -997,7 +1063,8 @@ __global__ __launch_bounds__(256) void prepack_t_kernel(const T* __restrict__ w,
         const int ns = slab / passes, pass = slab % passes;
         const T* src = (pass ? w_up : w) + (size_t)e * K * N;
         uint4 val = z;
-        if (k < K) val = *reinterpret_cast<const uint4*>(src + (size_t)k * N + (size_t)ns * SK + v * (16 / (int)sizeof(T)));
+        const int kc = gg_packed_col<sizeof(T) == 1>(k);  // the output column of the transposed product this row stands for
+        if (kc < K) val = *reinterpret_cast<const uint4*>(src + (size_t)kc * N + (size_t)ns * SK + v * (16 / (int)sizeof(T)));
         *reinterpret_cast<uint4*>(out + (((size_t)e * nsl * passes + slab) * Kpad + k) * SK + v * (16 / (int)sizeof(T))) = val;
     }
 }
@@ -1053,7 +1120,7 @@ __global__ __launch_bounds__(256) void dw_operand_kernel(const uint16_t* __restr
         if constexpr (SLAB) {
             int oc = c0 + c;
             if (split_F > 0 && oc < 2 * split_F) oc = ((oc % 64) / 32) * split_F + (oc / 64) * 32 + oc % 32;
-            out[((size_t)(sp / SK) * Npad + oc) * SK + sp % SK] = v;
+            out[((size_t)(sp / SK) * Npad + gg_packed_row<false>(oc)) * SK + sp % SK] = v;
         } else {
             out[(size_t)(c0 + c) * ld_out + sp] = v;
         }
@@ -1248,7 +1315,8 @@ template <typename T>
 int launch_prepack(const T* w, const T* w_up, int E_l, int K, int N, T* out, hipStream_t s) {
     const int n_eff = N * (w_up ? 2 : 1);
     const int Npad = round_up(n_eff, GG_BN);
-    if (Npad > n_eff) zero_pad_rows_kernel<T><<<dim3(64, E_l), 256, 0, s>>>(out, K, n_eff, Npad);
+    const int n_zero = w_up ? n_eff : std::min(round_up(N, 64), Npad);  // (the re-tiling kernel writes the zeros up to there)
+    if (Npad > n_zero) zero_pad_rows_kernel<T><<<dim3(64, E_l), 256, 0, s>>>(out, K, n_zero, Npad);
     prepack_kernel<T><<<dim3(ceil_div(N, 64), ceil_div(K, 64), E_l), 256, 0, s>>>(w, w_up, out, K, N, Npad);
     return moe_check_launch("prepack_weights");
 }
