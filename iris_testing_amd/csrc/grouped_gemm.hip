@@ -201,6 +201,33 @@ __device__ __forceinline__ void gg_fill_table(int4* s_tiles, const int* g_tile_s
     }
 }
 
+// The tile of round `round` if the table holds it and it has rows (rv = 0 otherwise: the caller then takes the general
+// walk below).  One LDS read; nothing is advanced, refilled or skipped.
+template <bool SPLIT, bool DW>
+__device__ __forceinline__ GgTile gg_peek(const int4* s_tiles, const int* g_row_start, const GgPlan& pl, int nk, int my, int stride,
+                                          int round, int round0) {
+    GgTile t;
+    t.g = t.nt = t.row0 = 0;
+    t.rv = 0;
+    t.ks0 = 0; t.nks = nk; t.unit = -1;
+    if (round < round0 + GG_TT) {  // (past the end of the walk the table holds empty entries)
+        const int4 e = s_tiles[round - round0];
+        t.g = __builtin_amdgcn_readfirstlane(e.x); t.nt = __builtin_amdgcn_readfirstlane(e.y);
+        t.row0 = __builtin_amdgcn_readfirstlane(e.z); t.rv = max(__builtin_amdgcn_readfirstlane(e.w), 0);
+        if constexpr (DW) {
+            t.ks0 = g_row_start[t.g];
+            t.nks = g_row_start[t.g + 1] - t.ks0;
+        }
+        if constexpr (SPLIT) {
+            const int lin = round * stride + my;
+            t.ks0 = (lin % pl.P) * pl.nkp;
+            t.nks = min(pl.nkp, nk - t.ks0);
+            t.unit = lin;
+        }
+    }
+    return t;
+}
+
 // Next non-empty tile of this workgroup at or after round `round` (advanced past it); rv = 0 when there is none.
 // round0 is the round the table starts at; the table is refilled (by the whole workgroup: every wave makes the same
 // calls) when the walk leaves it.
@@ -327,9 +354,10 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     __shared__ int g_tile_start[GG_MAXG + 1];
     __shared__ int g_row_start[GG_MAXG + 1];
     // what the epilogue needs from global memory per tile row / tile column (fp8 scales, the output row map)
-    __shared__ __align__(16) float s_row_scale[BM];
-    __shared__ __align__(16) float s_col_scale[BN];
-    __shared__ int s_crow[BM];
+    // (two copies, used by alternate tiles: a wave may enter the next tile while another is still in this one's epilogue)
+    __shared__ __align__(16) float s_row_scale[2][BM];
+    __shared__ __align__(16) float s_col_scale[2][BN];
+    __shared__ int s_crow[2][BM];
     __shared__ int s_amap[BM];              // the NEXT tile's input rows (a_map), fetched while this one is multiplied
     __shared__ __align__(16) int4 s_tiles[GG_TT];
     static_assert(BM <= NWM * 2 * WAVE && BN <= NWM * 2 * WAVE, "one thread per tile row and per tile column");
@@ -454,6 +482,14 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         for (int r = 0; r < RA; ++r) a_off[r] = a_off0[r];
         GG_PROLOGUE(Ab, Bb, a_off, (VARK ? cur.nks : nk));
     }
+    // The ring runs on from one tile into the next: the last four blocks of a tile refill their slots with the first
+    // four stages of the NEXT tile (when the table has it at hand), its last block reads that tile's first fragments,
+    // and the next tile then starts with everything in place -- no burst of 32 loads per lane with the matrix pipes
+    // idle, no pair of barriers.  `pre` says that the tile at hand was prepared like that; phi is the ring slot of its
+    // first stage (the ring is not realigned between tiles); tpar picks the copy of the epilogue data.
+    uint4 fA0[TM * CF], fB0[TN * CF], fA1[TM * CF], fB1[TN * CF];
+    bool pre = false;
+    int phi = 0, tpar = 0;
     while (cur.rv > 0) {
         const int g = __builtin_amdgcn_readfirstlane(cur.g), nt = __builtin_amdgcn_readfirstlane(cur.nt);
         const int row0 = __builtin_amdgcn_readfirstlane(cur.row0), rv = __builtin_amdgcn_readfirstlane(cur.rv);
@@ -507,7 +543,21 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     GG_ML((I) + 6, FA_, FB_, NA_, NB_, slot); GG_ML((I) + 7, FA_, FB_, NA_, NB_, slot)
 #define GG_STAGE(FA_, FB_, NA_, NB_, SL, s, last)                                                        \
     do {                                                                                                 \
-        GG_STAGE_PTRS(Ab, Bb, (s) + 4, ap_, bp_, nks)                                                    \
+        if constexpr ((SL) % 2 == 0) {                                                                   \
+            if ((s) == nks - 4) { /* from here on the loads fetch the next tile, if it is at hand */        \
+                const GgTile pk_ = gg_peek<SPLIT, DW>(s_tiles, g_row_start, plan, nk, my, (int)gridDim.x, round, round0); \
+                if (pk_.rv > 0) {                                                                        \
+                    GG_TILE_PTRS(pk_, Ab_s, Bb_s, a_off_s, GG_MAPROW_LDS);                               \
+                    Ab = Ab_s;                                                                           \
+                    Bb = Bb_s;                                                                           \
+                    _Pragma("unroll") for (int r = 0; r < RA; ++r) a_off[r] = a_off_s[r];                \
+                    kbase = nks;                                                                         \
+                    nks_ld = VARK ? pk_.nks : nk;                                                        \
+                    seam = true;                                                                         \
+                }                                                                                        \
+            }                                                                                            \
+        }                                                                                                \
+        GG_STAGE_PTRS(Ab, Bb, (s) + 4 - kbase, ap_, bp_, nks_ld)                                         \
         const uint4* nfa_ = fa + (((SL) + 1) & 3) * ASLOT;                                               \
         const uint4* nfb_ = fb + (((SL) + 1) & 3) * BSLOT;                                               \
         __builtin_amdgcn_sched_barrier(0);                                                               \
@@ -515,23 +565,25 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         GG_ML8(16, FA_, FB_, NA_, NB_, SL); GG_ML8(24, FA_, FB_, NA_, NB_, SL);                           \
         GG_ML8(32, FA_, FB_, NA_, NB_, SL); GG_ML8(40, FA_, FB_, NA_, NB_, SL);                           \
         GG_ML8(48, FA_, FB_, NA_, NB_, SL); GG_ML8(56, FA_, FB_, NA_, NB_, SL);                           \
-        if (!(last)) {                                                                                   \
+        if (!(last) || seam) { /* (the last block hands over too when the next tile's stages are behind it) */ \
             gg_wait<2 * LPS, 0>();                                                                       \
             __builtin_amdgcn_s_barrier();                                                                \
         }                                                                                                \
     } while (0)
+        int kbase = 0, nks_ld = nks;  // the loads of block s fetch stage s + 4 - kbase of the tile (Ab, Bb, a_off) point to
+        bool seam = false;            // ... which is the next tile from block nks - 4 on
         {
-            uint4 fA0[TM * CF], fB0[TN * CF], fA1[TM * CF], fB1[TN * CF];
-            // the four stages of this tile were requested before the previous tile's epilogue (or above, for
-            // the first tile); the epilogue's stores sit behind them in the same counter, so wait for
-            // everything once per tile
-            gg_wait<0, 15>();
-            __syncthreads();
+            if (!pre) {
+                // the four stages of this tile were requested before the previous tile's epilogue (or above, for
+                // the first tile); the epilogue's stores sit behind them in the same counter, so wait for
+                // everything
+                gg_wait<0, 15>();
+                __syncthreads();
+            }
             if (p.a_map) {
-                // the input rows of the NEXT tile, one per thread, straight into LDS: the tile set-up at the end of this
-                // tile's K loop then reads them from there instead of waiting for memory with the matrix pipes idle
-                int round_pk = round;  // (a look ahead: the walk itself advances at the end of the K loop)
-                const GgTile pk = gg_walk<BM, SPLIT, DW>(s_tiles, g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, plan, nk, my, (int)gridDim.x, round_pk, round0, p.dw_rows);
+                // the input rows of the NEXT tile, one per thread, straight into LDS: the switch to the next tile inside
+                // this tile's K loop then reads them from there instead of waiting for memory
+                const GgTile pk = gg_peek<SPLIT, DW>(s_tiles, g_row_start, plan, nk, my, (int)gridDim.x, round, round0);
                 if (pk.rv > 0 && wave_s * WAVE < BM) {
                     const int tid_a = wave_s * WAVE + gg_lane_now();
                     gg_dma4(gg_uniform((const uint8_t*)(p.a_map + pk.row0)), (uint32_t)min(tid_a, pk.rv - 1) * 4u,
@@ -540,46 +592,52 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             }
             if constexpr (!SPLIT) {
                 // What the epilogue needs from global memory per tile row / column (fp8 scales, the output row map) is
-                // requested here, straight into LDS, one value per thread: every wave has left the previous tile's
-                // epilogue, the loads land during the first K stages (they are older than every load the K loop waits
+                // requested here, straight into LDS, one value per thread (into the copy the previous tile does not
+                // use): the loads land during the first K stages (they are older than every load the K loop waits
                 // for), and no epilogue waits for a memory round trip.  No register holds anything across the K loop.
                 const int lane_t = gg_lane_now(), tid_t = wave_s * WAVE + lane_t;  // (a fresh lane id: nothing kept live for this)
                 const uint32_t t4 = (uint32_t)min(tid_t, rv - 1) * 4u;
                 if (wave_s * WAVE < BM) {
                     if constexpr (FP8)
                         gg_dma4(gg_uniform((const uint8_t*)(p.row_scale + row0)), t4,
-                                __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(s_row_scale + wave_s * WAVE)));
+                                __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(s_row_scale[tpar] + wave_s * WAVE)));
                     if (p.c_map)
                         gg_dma4(gg_uniform((const uint8_t*)(p.c_map + row0)), t4,
-                                __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(s_crow + wave_s * WAVE)));
+                                __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(s_crow[tpar] + wave_s * WAVE)));
                 }
                 if constexpr (FP8) {
                     const int pc = gg_packed_col<true>(nt * BN + tid_t);  // packed column of the launch behind this row of the weight tile; the lanes 32..63 of a wave hold up columns
                     int col = EPI == EPI_SWIGLU ? (pc / 64) * 32 + pc % 32 : pc;
                     col = col < p.N ? col : 0;  // (columns past N are never stored: any valid scale will do)
-                    const uint32_t lds_cs = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(s_col_scale + wave_s * WAVE));
+                    const uint32_t lds_cs = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(s_col_scale[tpar] + wave_s * WAVE));
                     const uint32_t c4 = (uint32_t)col * 4u;
                     if (EPI == EPI_SWIGLU && lane_t >= 32) gg_dma4(gg_uniform((const uint8_t*)(p.col_scale2 + (size_t)g * p.ncs)), c4, lds_cs);
                     else gg_dma4(gg_uniform((const uint8_t*)(p.col_scale + (size_t)g * p.ncs)), c4, lds_cs);
                 }
             }
+            if (!pre) {
+                const uint4* fa0 = fa + phi * ASLOT;
+                const uint4* fb0 = fb + phi * BSLOT;
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+                for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int h = 0; h < CF; ++h) fA0[i * CF + h] = fa[i * MT * CHUNKS + (fpos ^ h)];
+                    for (int h = 0; h < CF; ++h) fA0[i * CF + h] = fa0[i * MT * CHUNKS + (fpos ^ h)];
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
+                for (int j = 0; j < TN; ++j)
 #pragma unroll
-                for (int h = 0; h < CF; ++h) fB0[j * CF + h] = fb[j * MT * CHUNKS + (fpos ^ h)];
-            // slot 0 is refilled from the first block on: every wave must hold its stage-0 fragments first
-            gg_wait<63, 0>();
-            __syncthreads();
-            // nk >= 2 and even: a loop that cannot run zero times keeps the accumulators in place from their
-            // zeroing to the epilogue
-            int ks = 0;
+                    for (int h = 0; h < CF; ++h) fB0[j * CF + h] = fb0[j * MT * CHUNKS + (fpos ^ h)];
+                // the first slot is refilled from the first block on: every wave must hold its stage-0 fragments first
+                gg_wait<63, 0>();
+                __syncthreads();
+            }
+            // The blocks are written out for the slots 0 .. 3; a tile whose first stage lies in slot 2 (phi = 2: the
+            // tiles before it left the ring there) enters at the third.  nk >= 2 and even.
+            int ks = -phi;
             do {
-                GG_STAGE(fA0, fB0, fA1, fB1, 0, ks, false);
-                GG_STAGE(fA1, fB1, fA0, fB0, 1, ks + 1, ks + 2 >= nks);
+                if (ks >= 0) {
+                    GG_STAGE(fA0, fB0, fA1, fB1, 0, ks, false);
+                    GG_STAGE(fA1, fB1, fA0, fB0, 1, ks + 1, ks + 2 >= nks);
+                }
                 if (ks + 2 < nks) {
                     GG_STAGE(fA0, fB0, fA1, fB1, 2, ks + 2, false);
                     GG_STAGE(fA1, fB1, fA0, fB0, 3, ks + 3, ks + 4 >= nks);
@@ -594,12 +652,18 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 
         // ---- next tile: decode it and request its first stages now (every slot is free once all waves
         // have passed the barrier: the last fragments of this tile are already in registers)
+        // (when the K loop has switched over, the walk only confirms what the look-ahead saw)
         const GgTile nxt = gg_walk<BM, SPLIT, DW>(s_tiles, g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, plan, nk, my, (int)gridDim.x, round, round0, p.dw_rows);
-        GG_TILE_PTRS(nxt, Ab_n, Bb_n, a_off_n, GG_MAPROW_LDS);
-        if (nxt.rv > 0) {
+        if (!seam && nxt.rv > 0) {
+            GG_TILE_PTRS(nxt, Ab_n, Bb_n, a_off_n, GG_MAPROW_GLOBAL);
+            Ab = Ab_n;
+            Bb = Bb_n;
+#pragma unroll
+            for (int r = 0; r < RA; ++r) a_off[r] = a_off_n[r];
             __syncthreads();
-            GG_PROLOGUE(Ab_n, Bb_n, a_off_n, (VARK ? nxt.nks : nk));
+            GG_PROLOGUE(Ab, Bb, a_off, (VARK ? nxt.nks : nk));
         }
+        const int phi_n = seam ? ((phi + nks) & 3) : 0;
 
         // ---- a part of a tile: its fp32 partial sums go to the workspace as they are (tile row major, 256
         // columns; the lane's runs of four columns as 16-byte stores); the reduction kernel does the rest
@@ -624,10 +688,9 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                 __builtin_amdgcn_sched_barrier(0);
             }
             cur = nxt;
-            Ab = Ab_n;
-            Bb = Bb_n;
-#pragma unroll
-            for (int r = 0; r < RA; ++r) a_off[r] = a_off_n[r];
+            pre = seam;
+            phi = phi_n;
+            tpar ^= 1;
             continue;
         }
 
@@ -656,8 +719,8 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             ok[i] = r < rv;
             const size_t grow = (size_t)(row0 + (ok[i] ? r : 0));
             rs[i] = 1.f;
-            if constexpr (FP8) rs[i] = s_row_scale[r];
-            const int crow_i = p.c_map ? s_crow[r] : 0;
+            if constexpr (FP8) rs[i] = s_row_scale[tpar][r];
+            const int crow_i = p.c_map ? s_crow[tpar][r] : 0;
             ok[i] = ok[i] && crow_i >= 0;  // a negative map entry: the row has no place in the output
             crow[i] = C + (p.c_map ? (size_t)max(crow_i, 0) : grow) * p.ldc + (DW ? (size_t)g * p.c_group_stride : (size_t)0);
         }
@@ -687,10 +750,10 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                     if constexpr (FP8) {
                         // channel scales by row of the weight tile (an LDS read: cheap enough to repeat for every row tile)
                         const int tc = cbase_e + j * MT + 8 * qd + 4 * lsub;
-                        const float4 s0 = *(const float4*)(s_col_scale + tc);
+                        const float4 s0 = *(const float4*)(s_col_scale[tpar] + tc);
                         cg[0] = s0.x; cg[1] = s0.y; cg[2] = s0.z; cg[3] = s0.w;
                         if constexpr (EPI == EPI_SWIGLU) {
-                            const float4 s1 = *(const float4*)(s_col_scale + tc + 32);
+                            const float4 s1 = *(const float4*)(s_col_scale[tpar] + tc + 32);
                             cu[0] = s1.x; cu[1] = s1.y; cu[2] = s1.z; cu[3] = s1.w;
                         }
                     }
@@ -722,10 +785,9 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             __builtin_amdgcn_sched_barrier(0);
         }
         cur = nxt;
-        Ab = Ab_n;
-        Bb = Bb_n;
-#pragma unroll
-        for (int r = 0; r < RA; ++r) a_off[r] = a_off_n[r];
+        pre = seam;
+        phi = phi_n;
+        tpar ^= 1;
     }
 #undef GG_TILE_PTRS
 #undef GG_MAPROW_GLOBAL
