@@ -268,6 +268,14 @@ int moe_grouped_mlp_fp8_mapped(const void* a_base_bf16, int a_rows, const int32_
  * moe_combine_backward: d ret[slot(t,kk)] = gate[t,kk] * d out[t] (padding slots zeroed, like the pack) and
  *   d gate[t,kk] = <d out[t], ret[slot(t,kk)]>.  The gradient of the fixed-M pack is moe_combine with unit gates; that of
  *   the expert-major unpack is moe_return_pack, and the other way round; moe_shuffle_backward is declared above. */
+/* moe_grouped_gemm_act_keep: moe_grouped_gemm_mapped with an activation (act != MOE_ACT_NONE; bf16; rows of `out` are not
+ *   remapped) that ALSO stores the values before the activation, for the backward pass of the expert MLP
+ *   (layers/expert.py:62-64 of the reference is an empty stub): pre_act [S_rows, N] bf16, for SwiGLU [S_rows, 2N] in the
+ *   column order of the fused gate / up product (32 gate columns, their 32 up columns, ...), which is what
+ *   moe_mlp_act_backward takes.  Same values as a launch with MOE_ACT_NONE on the same weights would give. */
+int moe_grouped_gemm_act_keep(const void* a_base, int a_rows, const int32_t* a_row_map, const void* packed,
+                              const int32_t* expert_cnt, int S_rows, int K, int N, int E_l, int act, void* out, void* pre_act,
+                              void* part_ws, size_t part_ws_bytes, moe_stream_t stream);
 int moe_prepack_weights_transposed(const void* w, const void* w_up, int dtype, int E_l, int K, int N, void* packed,
                                    moe_stream_t stream);
 size_t moe_dw_workspace_bytes(int S_rows, int E_l, int K, int N);

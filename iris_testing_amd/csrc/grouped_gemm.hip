@@ -42,6 +42,8 @@ struct GemmParams {
     const uint8_t* A;         // [S_rows, K] activations (bf16 or fp8)
     const uint8_t* B;         // packed weights [E_l, Npad, K]
     void* C;                  // [S_rows, ldc] bf16
+    void* C2;                 // optional (bf16 kernels with an activation): the values BEFORE the activation, bf16, row pitch ldc
+                              // (SwiGLU: 2 ldc, in the packed gate / up column order), kept for the backward pass
     const int32_t* cnt;       // [E_l] rows per group
     const float* row_scale;   // fp8: [S_rows] per-row activation scale
     const float* col_scale;   // fp8: [E_l, ncs] per-output-channel scale (gate for SwiGLU)
@@ -741,6 +743,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                 // fp8: the register quads 2u and 2u + 1 of the group's one tile)
                 const int col = colg + (FP8 ? 16 * u : 0) + 8 * lsub;
                 float x[8];
+                [[maybe_unused]] float pre_g[8], pre_u[8];  // bf16 kernels asked to keep them: the values before the activation
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
                     const int j = FP8 ? jg : jg * GT + t;       // MFMA tile of the run
@@ -761,9 +764,11 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                     for (int e = 0; e < 4; ++e) {
                         float v = acc[i][j][4 * qd + e];
                         if constexpr (FP8) v *= cg[e] * rs[i];
+                        if constexpr (!FP8 && EPI != EPI_NONE) pre_g[4 * t + e] = v;
                         if constexpr (EPI == EPI_SWIGLU) {
                             float uv = acc[i][ju % TN][4 * qd + e];
                             if constexpr (FP8) uv *= cu[e] * rs[i];
+                            if constexpr (!FP8) pre_u[4 * t + e] = uv;
                             v = act_silu_fast(v) * uv;
                         }
                         if constexpr (EPI == EPI_GELU) v = act_gelu(v);
@@ -778,6 +783,23 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                     o4.z = gg_pack_bf16(x[4], x[5]);
                     o4.w = gg_pack_bf16(x[6], x[7]);
                     *(uint4*)(crow[i] + col) = o4;
+                    if constexpr (!FP8 && EPI != EPI_NONE) {
+                        if (p.C2) {
+                            // same row, in a matrix whose rows are as long (SwiGLU: twice as long, packed column order)
+                            constexpr int W2 = EPI == EPI_SWIGLU ? 2 : 1;
+                            bf16_t* r2 = (bf16_t*)p.C2 + (size_t)(crow[i] - C) * W2 + (EPI == EPI_SWIGLU ? pcol + 8 * lsub : col);
+                            uint4 g4;
+                            g4.x = gg_pack_bf16(pre_g[0], pre_g[1]); g4.y = gg_pack_bf16(pre_g[2], pre_g[3]);
+                            g4.z = gg_pack_bf16(pre_g[4], pre_g[5]); g4.w = gg_pack_bf16(pre_g[6], pre_g[7]);
+                            *(uint4*)r2 = g4;
+                            if constexpr (EPI == EPI_SWIGLU) {
+                                uint4 u4;
+                                u4.x = gg_pack_bf16(pre_u[0], pre_u[1]); u4.y = gg_pack_bf16(pre_u[2], pre_u[3]);
+                                u4.z = gg_pack_bf16(pre_u[4], pre_u[5]); u4.w = gg_pack_bf16(pre_u[6], pre_u[7]);
+                                *(uint4*)(r2 + 32) = u4;
+                            }
+                        }
+                    }
                 }
             }
             // keep the accumulator read-out of one group from being hoisted over the previous group's stores
@@ -861,6 +883,19 @@ __global__ __launch_bounds__(256) void gg_reduce_parts_kernel(const GemmParams p
         float rs = 1.f;
         if constexpr (FP8) rs = p.row_scale[grow];
         float av[4] = {a.x, a.y, a.z, a.w}, bv[4] = {b.x, b.y, b.z, b.w};
+        if constexpr (!FP8 && EPI != EPI_NONE) {
+            if (p.C2 && col < p.N) {  // the values before the activation, kept for the backward pass (rows are never remapped there)
+                constexpr int W2 = EPI == EPI_SWIGLU ? 2 : 1;
+                bf16_t* r2 = (bf16_t*)p.C2 + grow * (size_t)p.ldc * W2 + (EPI == EPI_SWIGLU ? gp : col);
+                uint2 o2;
+                o2.x = gg_pack_bf16(av[0], av[1]); o2.y = gg_pack_bf16(av[2], av[3]);
+                *(uint2*)r2 = o2;
+                if constexpr (EPI == EPI_SWIGLU) {
+                    o2.x = gg_pack_bf16(bv[0], bv[1]); o2.y = gg_pack_bf16(bv[2], bv[3]);
+                    *(uint2*)(r2 + 32) = o2;
+                }
+            }
+        }
         const float c0[4] = {sc0.x, sc0.y, sc0.z, sc0.w}, c1[4] = {sc1.x, sc1.y, sc1.z, sc1.w};
         float x[4];
 #pragma unroll
@@ -1469,6 +1504,25 @@ extern "C" int moe_grouped_gemm_mapped(const void* a_base, int a_rows, const int
     GemmParams p{};
     p.A = (const uint8_t*)a_base; p.B = (const uint8_t*)packed; p.C = out; p.cnt = expert_cnt;
     p.a_map = a_row_map; p.c_map = c_row_map;
+    p.E_l = E_l; p.K = K; p.N = N; p.ldc = N; p.S_rows = S_rows;
+    p.Npad = round_up(act == EPI_SWIGLU ? 2 * N : N, GG_BN);
+    return launch_gemm<false>(p, act, (hipStream_t)stream, part_ws, part_ws_bytes);
+}
+
+extern "C" int moe_grouped_gemm_act_keep(const void* a_base, int a_rows, const int32_t* a_row_map, const void* packed,
+                                         const int32_t* expert_cnt, int S_rows, int K, int N, int E_l, int act, void* out,
+                                         void* pre_act, void* part_ws, size_t part_ws_bytes, moe_stream_t stream) {
+    MOE_REQUIRE(S_rows >= 0 && K > 0 && N > 0 && E_l > 0 && E_l <= GG_MAXG, MOE_ERR_INVALID, "grouped_gemm_act_keep: bad shape");
+    MOE_REQUIRE(act > EPI_NONE && act <= EPI_SWIGLU, MOE_ERR_INVALID, "grouped_gemm_act_keep: activation %d", act);
+    MOE_REQUIRE(K % 64 == 0 && N % 8 == 0, MOE_ERR_UNSUPPORTED, "grouped_gemm_act_keep: needs K %% 64 == 0 and N %% 8 == 0 (K=%d N=%d)", K, N);
+    MOE_REQUIRE(a_rows >= 0, MOE_ERR_INVALID, "grouped_gemm_act_keep: negative buffer rows");
+    MOE_REQUIRE(!a_row_map || (unsigned long long)a_rows * (unsigned long long)K * 2ull < (1ull << 32), MOE_ERR_UNSUPPORTED,
+                "grouped_gemm_act_keep: the gathered buffer must be smaller than 4 GiB (%d rows of %d)", a_rows, K);
+    if (S_rows == 0) return MOE_OK;
+    MOE_REQUIRE(a_base && packed && expert_cnt && out && pre_act, MOE_ERR_INVALID, "grouped_gemm_act_keep: null pointer");
+    GemmParams p{};
+    p.A = (const uint8_t*)a_base; p.B = (const uint8_t*)packed; p.C = out; p.C2 = pre_act; p.cnt = expert_cnt;
+    p.a_map = a_row_map;
     p.E_l = E_l; p.K = K; p.N = N; p.ldc = N; p.S_rows = S_rows;
     p.Npad = round_up(act == EPI_SWIGLU ? 2 * N : N, GG_BN);
     return launch_gemm<false>(p, act, (hipStream_t)stream, part_ws, part_ws_bytes);

@@ -153,20 +153,29 @@ class ExpertMLP(torch.autograd.Function):
     @staticmethod
     def forward(ctx, tokens, cnt, ew, w1, w2, w_up):
         tokens = tokens.contiguous()
-        S = tokens.shape[0]
-        hidden = torch.empty((S, ew.ffn), dtype=tokens.dtype, device=tokens.device)
-        out = ops.grouped_mlp(tokens, cnt, ew.act, ew.w1, ew.w2, ew.w_up, F=ew.ffn, hidden_ws=hidden)
-        ctx.save_for_backward(tokens, hidden, cnt, w1, w2, w_up)
+        S, F = tokens.shape[0], ew.ffn
+        hidden = torch.empty((S, F), dtype=tokens.dtype, device=tokens.device)
+        a1 = None
+        if tokens.dtype == torch.bfloat16 and ew.act != "none" and S:
+            # the first GEMM also keeps what it feeds to the activation: the backward pass would otherwise run it again
+            ws = _part_ws(tokens.device)
+            a1 = torch.empty((S, 2 * F if ew.act == "swiglu" else F), dtype=tokens.dtype, device=tokens.device)
+            ops.grouped_gemm_act_keep(tokens, ew.w1, cnt, S, F, ew.act, hidden, a1, part_ws=ws)
+            out = torch.zeros((S, ew.hidden), dtype=tokens.dtype, device=tokens.device)  # (rows past the counted total stay zero)
+            ops.grouped_gemm_mapped(hidden, None, ew.w2, cnt, S, ew.hidden, "none", out, part_ws=ws)
+        else:
+            out = ops.grouped_mlp(tokens, cnt, ew.act, ew.w1, ew.w2, ew.w_up, F=F, hidden_ws=hidden)
+        ctx.save_for_backward(tokens, hidden, cnt, w1, w2, w_up, a1)
         ctx.ew = ew
         return out
 
     @staticmethod
     def backward(ctx, dy):
-        """With a1 the pre-activations (recomputed: the forward keeps only the hidden activation h):
+        """With a1 the pre-activations (bf16: kept by the forward's first GEMM; fp32: recomputed):
           d h  = dy @ W2^T          d W2 = h^T @ dy            (per expert, ragged rows as the reduction dimension)
           d a1 = d h * act'(a1)     (SwiGLU: d g = d h * u * silu'(g), d u = d h * silu(g))
           d x  = d a1 @ W1^T        d W1 = x^T @ d a1          (SwiGLU: both halves in one launch each)"""
-        tokens, hidden, cnt, w1, w2, w_up = ctx.saved_tensors
+        tokens, hidden, cnt, w1, w2, w_up, a1 = ctx.saved_tensors
         ew = ctx.ew
         dy = dy.contiguous()
         S, H, F = tokens.shape[0], ew.hidden, ew.ffn
@@ -185,10 +194,12 @@ class ExpertMLP(torch.autograd.Function):
         NP = 2 * F if swiglu else F
         dh = torch.zeros((S, F), dtype=dy.dtype, device=dy.device)
         dx = torch.zeros((S, H), dtype=dy.dtype, device=dy.device)
-        a1 = torch.zeros((S, NP), dtype=dy.dtype, device=dy.device)
         if S:
             ops.grouped_gemm_mapped(dy, None, _packed_weights_t(w2), cnt, S, F, "none", dh, part_ws=ws)
-            ops.grouped_gemm_mapped(tokens, None, ew.w1, cnt, S, NP, "none", a1, part_ws=ws)
+        if a1 is None:  # (no rows, or an MLP without an activation)
+            a1 = torch.zeros((S, NP), dtype=dy.dtype, device=dy.device)
+            if S:
+                ops.grouped_gemm_mapped(tokens, None, ew.w1, cnt, S, NP, "none", a1, part_ws=ws)
         dw2 = ops.grouped_gemm_dw(hidden, dy, cnt)
         da1 = ops.mlp_act_backward(a1, dh, ew.act)
         if S:

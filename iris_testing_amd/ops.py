@@ -408,6 +408,24 @@ def grouped_gemm_mapped(a_base: torch.Tensor, a_row_map: Optional[torch.Tensor],
     return out
 
 
+def grouped_gemm_act_keep(a_base: torch.Tensor, packed: torch.Tensor, expert_cnt: torch.Tensor, S_rows: int, N: int, act: str,
+                          out: torch.Tensor, pre_act: torch.Tensor, part_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """grouped_gemm_mapped with an activation that also keeps the values before it (for the backward pass):
+    pre_act [S_rows, N], for SwiGLU [S_rows, 2N] in the fused gate / up column order (what mlp_act_backward takes)."""
+    _req_cuda(a_base, "a_base")
+    _req_i32(expert_cnt, "expert_cnt")
+    assert act in ("gelu", "silu", "swiglu"), "an activation to keep the input of"
+    assert a_base.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and pre_act.dtype == torch.bfloat16
+    assert a_base.is_contiguous() and out.is_contiguous() and pre_act.is_contiguous()
+    assert out.shape == (S_rows, N) and pre_act.shape == (S_rows, 2 * N if act == "swiglu" else N)
+    L.check(L.lib().moe_grouped_gemm_act_keep(L.ptr(a_base), a_base.shape[0], None, L.ptr(packed), L.ptr(expert_cnt), S_rows,
+                                              a_base.shape[1], N, expert_cnt.numel(), L.ACT[act], L.ptr(out), L.ptr(pre_act),
+                                              L.ptr(part_ws) if part_ws is not None else None,
+                                              part_ws.numel() * part_ws.element_size() if part_ws is not None else 0,
+                                              L.stream_ptr()))
+    return out
+
+
 def gemm_part_workspace(device) -> torch.Tensor:
     """fp32 scratch for the K-split of grouped_gemm_mapped, sized for any launch."""
     return torch.empty(L.lib().moe_gemm_part_workspace_bytes() // 4, dtype=torch.float32, device=device)

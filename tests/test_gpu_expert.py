@@ -197,6 +197,41 @@ def test_grouped_gemm_k_split_of_the_last_round(E_l, K, N, rows, act):
     print(f"K split: {differs} of {split.numel()} outputs differ in the last bits from the unsplit kernel", flush=True)
 
 
+@pytest.mark.parametrize("E_l,K,N,rows,act", [(3, 256, 384, (300, 0, 77), "swiglu"), (2, 512, 256, (70, 333), "gelu"),
+                                              (1, 1024, 2048, (443,), "silu"), (1, 1024, 4096, (20836,), "swiglu")])
+@pytest.mark.parametrize("split", [False, True], ids=["whole_tiles", "k_split"])
+def test_grouped_gemm_act_keep_also_stores_the_pre_activations(E_l, K, N, rows, act, split):
+    """The launch that keeps the values before the activation for the backward pass: its output is bit for bit that
+    of the ordinary launch, and what it keeps is bit for bit what a launch without activation produces (SwiGLU: in
+    the fused gate / up column order) -- with and without the K split of the last round."""
+    rng = np.random.default_rng(K + N + len(rows))
+    cnt = np.array(rows, dtype=np.int32)
+    S_tot = int(cnt.sum())
+    x = _randn(rng, S_tot, K)
+    w = _randn(rng, E_l, K, N, scale=K ** -0.5)
+    wu = _randn(rng, E_l, K, N, scale=K ** -0.5) if act == "swiglu" else None
+    packed = ops.prepack_weights(_t(w, "bf16"), None if wu is None else _t(wu, "bf16"))
+    cnt_t, x_t = torch.from_numpy(cnt).to(DEV), _t(x, "bf16")
+    ws = ops.gemm_part_workspace(DEV) if split else None
+    NP = 2 * N if act == "swiglu" else N
+    plain = torch.full((S_tot, N), -7.0, dtype=torch.bfloat16, device=DEV)
+    ops.grouped_gemm_mapped(x_t, None, packed, cnt_t, S_tot, N, act, plain, part_ws=ws)
+    pre_ref = torch.full((S_tot, NP), -7.0, dtype=torch.bfloat16, device=DEV)
+    ops.grouped_gemm_mapped(x_t, None, packed, cnt_t, S_tot, NP, "none", pre_ref, part_ws=ws)
+    out = torch.full((S_tot, N), -7.0, dtype=torch.bfloat16, device=DEV)
+    pre = torch.full((S_tot, NP), -7.0, dtype=torch.bfloat16, device=DEV)
+    ops.grouped_gemm_act_keep(x_t, packed, cnt_t, S_tot, N, act, out, pre, part_ws=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.int16), plain.view(torch.int16)), "the output changed with the second store"
+    assert torch.equal(pre.view(torch.int16), pre_ref.view(torch.int16)), "kept pre-activations differ from a launch without activation"
+    # and they are the oracle's product
+    want = O.grouped_gemm(x, w, cnt, "bf16")
+    got = to_np(pre)
+    if act == "swiglu":  # fused order: 32 gate columns, their 32 up columns, ...
+        got = got.reshape(S_tot, N // 32, 2, 32)[:, :, 0, :].reshape(S_tot, N)
+    _check(got, want, BF16_RTOL, BF16_ATOL, "kept pre-activations")
+
+
 @pytest.mark.parametrize("W,E_l,M,H,F,fill", [(4, 3, 300, 128, 256, "ragged"), (8, 5, 64, 256, 128, "empty"),
                                               (2, 1, 40, 128, 128, "full")])
 def test_copy_free_destination_equals_operator_chain(W, E_l, M, H, F, fill):
