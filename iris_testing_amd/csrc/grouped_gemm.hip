@@ -1369,9 +1369,15 @@ int launch_gemm(const GemmParams& p_in, int epi, hipStream_t s, void* part_ws = 
         if (p.max_units >= 2) p.part_ws = (float*)part_ws;
     }
     const int red_blocks = (grid / 4) * GG_RED_SLABS;
+    // A launch so small that all its tiles are certain to be split (whatever the row counts turn out to be, there are at most
+    // ub of them: every group adds at most one partly filled row of tiles) has no whole tile: the first kernel is left out.
+    // gg_plan finds two parts or more whenever 4 tail <= grid, the K range has 16 stages and the workspace holds 2 tail units.
+    const int bm = small_m ? 128 : 256, nk = p.K * (FP8 ? 1 : 2) / ROWB;
+    const long long ub = ((long long)(p.S_rows + bm - 1) / bm + p.E_l) * nt;
+    const bool all_split = p.part_ws && red_blocks > 0 && 4 * ub <= grid && nk >= 2 * GG_MIN_PART_STAGES && p.max_units >= 2 * ub;
 #define GG_LAUNCH(BMv, NWMv, EPIv)                                                                        \
     do {                                                                                                  \
-        grouped_gemm_kernel<BMv, NWMv, EPIv, FP8, false><<<grid, NWMv * 2 * WAVE, 0, s>>>(p);              \
+        if (!all_split) grouped_gemm_kernel<BMv, NWMv, EPIv, FP8, false><<<grid, NWMv * 2 * WAVE, 0, s>>>(p); \
         if (p.part_ws && red_blocks > 0) {                                                                \
             grouped_gemm_kernel<BMv, NWMv, EPIv, FP8, true><<<grid, NWMv * 2 * WAVE, 0, s>>>(p);           \
             gg_reduce_parts_kernel<BMv, EPIv, FP8><<<red_blocks, 256, 0, s>>>(p, grid);                    \
