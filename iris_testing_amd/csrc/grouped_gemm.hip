@@ -546,7 +546,9 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 #define GG_STAGE(FA_, FB_, NA_, NB_, SL, s, last)                                                        \
     do {                                                                                                 \
         if constexpr ((SL) % 2 == 0) {                                                                   \
-            if ((s) == nks - 4) { /* from here on the loads fetch the next tile, if it is at hand */        \
+            /* from block nks - 4 on the loads fetch the next tile, if it is at hand; not in a tile's first block: the  \
+               row map that the tile's top requested must have landed and been handed over (one block end at least) */ \
+            if ((s) == nks - 4 && (s) > 0) {                                                             \
                 const GgTile pk_ = gg_peek<SPLIT, DW>(s_tiles, g_row_start, plan, nk, my, (int)gridDim.x, round, round0); \
                 if (pk_.rv > 0) {                                                                        \
                     GG_TILE_PTRS(pk_, Ab_s, Bb_s, a_off_s, GG_MAPROW_LDS);                               \

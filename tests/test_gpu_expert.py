@@ -114,7 +114,11 @@ def test_expert_mlp(dtype, act, E_l, H, F, S):
     _check(out, want.astype(np.float64), r, a, f"expert_mlp {dtype} {act} E_l={E_l} H={H} F={F}")
 
 
-@pytest.mark.parametrize("E_l,K,N,S,act", [(3, 128, 264, 900, "none"), (4, 256, 512, 1500, "swiglu")])
+@pytest.mark.parametrize("E_l,K,N,S,act", [(3, 128, 264, 900, "none"), (4, 256, 512, 1500, "swiglu"),
+                                           # more tiles than workgroups, short K: the ring runs on from tile to tile (K = 192,
+                                           # 320: six and ten stages, so consecutive tiles start in different ring slots) or,
+                                           # with four stages (K = 128), every tile is set up on its own
+                                           (3, 128, 2048, 9000, "none"), (2, 192, 2048, 9500, "none"), (5, 320, 1024, 17000, "swiglu")])
 def test_grouped_gemm_mapped(E_l, K, N, S, act):
     """Row indirection on both sides: logical row r is read from a scattered row of a larger buffer and its
     result is written to a scattered row of a larger output.  The result must be bit for bit what the plain
