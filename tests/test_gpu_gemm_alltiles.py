@@ -192,3 +192,23 @@ def test_projection_check_sees_a_wrong_tile():
     short[0:256, 0:256] = (X[0:256, 32:].float() @ W[0, 32:, 0:256].float()).bfloat16()
     with pytest.raises(AssertionError):
         _freivalds(short, X, W, [S], "one tile short of a K stage")
+
+
+def test_more_rounds_than_the_tile_table_holds():
+    """A workgroup decodes its tiles 256 rounds at a time into a table; a launch of more than 256 rounds (66 048 tiles
+    here: 258 row tiles x 256 column tiles on 256 workgroups, K = 64 to keep it cheap) must refill it.  The output rows are
+    mapped away (negative map entries store nothing) except a sample that holds every row of the rounds past the first
+    table, which is compared with a plain fp32 product."""
+    torch.manual_seed(5)
+    S, K, N = 66000, 64, 65536
+    x = torch.randn((S, K), device=DEV).bfloat16()
+    w = (torch.randn((1, K, N), device=DEV) * K ** -0.5).bfloat16()
+    cnt = torch.tensor([S], dtype=torch.int32, device=DEV)
+    keep = torch.cat([torch.arange(0, 300), torch.arange(30000, 30300), torch.arange(65536 - 200, S)]).to(DEV)
+    c_map = torch.full((S,), -1, dtype=torch.int32, device=DEV)
+    c_map[keep] = torch.arange(keep.numel(), dtype=torch.int32, device=DEV)
+    out = torch.full((keep.numel(), N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.grouped_gemm_mapped(x, None, ops.prepack_weights(w), cnt, S, N, "none", out, c_row_map=c_map)
+    torch.cuda.synchronize()
+    ref = x[keep].float() @ w[0].float()
+    _close(out, ref, "rows of the first, a middle and the last rounds")
