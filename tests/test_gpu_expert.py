@@ -161,6 +161,24 @@ def test_grouped_gemm_mapped(E_l, K, N, S, act):
     assert rc != 0 and b"4 GiB" in lib.moe_last_error()
 
 
+def test_grouped_gemm_counts_that_claim_more_rows_than_there_are():
+    """Row counts are device data the kernels cannot trust: a group that claims rows past S_rows is cut there (its tiles
+    beyond have no rows and are skipped by the walk), the groups after it get nothing, and nothing is read or written
+    past row S_rows."""
+    rng = np.random.default_rng(77)
+    E_l, K, N, S_rows = 3, 256, 1024, 700
+    cnt = np.array([300, 5000, 40], dtype=np.int32)
+    x = _randn(rng, S_rows, K)
+    w = _randn(rng, E_l, K, N, scale=K ** -0.5)
+    packed = ops.prepack_weights(_t(w, "bf16"))
+    out = torch.full((S_rows + 300, N), -7.0, dtype=torch.bfloat16, device=DEV)
+    ops.grouped_gemm_mapped(_t(x, "bf16"), None, packed, torch.from_numpy(cnt).to(DEV), S_rows, N, "none", out)
+    torch.cuda.synchronize()
+    want = O.grouped_gemm(x, w, np.array([300, 400, 0], dtype=np.int32), "bf16")
+    _check(to_np(out[:S_rows]), want, BF16_RTOL, BF16_ATOL, "clamped groups")
+    assert bool((out[S_rows:] == -7.0).all()), "rows past S_rows were written"
+
+
 @pytest.mark.parametrize("E_l,K,N,rows,act", [(2, 512, 1024, (200, 150), "none"), (2, 2048, 4096, (230, 213), "silu"),
                                               (3, 1024, 512, (300, 0, 77), "swiglu"), (1, 4096, 2048, (443,), "gelu"),
                                               (1, 1024, 4096, (20836,), "swiglu")])
