@@ -386,8 +386,11 @@ __global__ __launch_bounds__(WPB * WAVE) void gather_rows_kernel(const u32x4* __
 }
 
 // ---- pack, token-major: every token row is read once and stored to its k send slots ------------------
-// Rows [0, T) of the launch are tokens, rows [T, T + W*M) are send slots that only get zeros when they are
-// padding.  Same bytes in send_buf as the slot-major gather (SRC_PACK), with x read once instead of k times.
+// Units [0, T) of the launch are tokens (one wave each); the units after them are runs of PACK_ZR consecutive send
+// slots each, which only get zeros where they are padding (a wave per slot was mostly wave start-up: with skewed
+// routing most of the send buffer is padding).  Same bytes in send_buf as the slot-major gather (SRC_PACK), with x
+// read once instead of k times.
+constexpr int PACK_ZR = 8;
 template <int WPB>
 __global__ __launch_bounds__(WPB * WAVE) void pack_tokens_kernel(const u32x4* __restrict__ x, u32x4* __restrict__ send,
                                                                   const int32_t* __restrict__ idx, const int32_t* __restrict__ pos,
@@ -395,16 +398,22 @@ __global__ __launch_bounds__(WPB * WAVE) void pack_tokens_kernel(const u32x4* __
                                                                   const int32_t* __restrict__ dst_offsets, int T, int k, int E_l,
                                                                   int W, int M, int row_vec, int32_t* __restrict__ status) {
     const int wave = threadIdx.x / WAVE, lane = lane_id();
-    const int n_rows = T + W * M;
-    for (int r = blockIdx.x * WPB + wave; r < n_rows; r += gridDim.x * WPB) {
+    const int n_slots = W * M;
+    const int n_units = T + (n_slots + PACK_ZR - 1) / PACK_ZR;
+    for (int r = blockIdx.x * WPB + wave; r < n_units; r += gridDim.x * WPB) {
         if (r >= T) {
-            const int d = (r - T) / M, m = (r - T) % M;
-            const int cnt = dst_sizes[d];
-            if (m == 0 && cnt > M && status && lane == 0) *status = 1;
-            if (m < cnt) continue;
-            u32x4* o = send + (size_t)(r - T) * row_vec;
+            const int s0 = (r - T) * PACK_ZR, s1 = min(s0 + PACK_ZR, n_slots);
+            int d = s0 / M, m = s0 % M;
+            int cnt = dst_sizes[d];
             const u32x4 z = {0u, 0u, 0u, 0u};
-            for (int c = lane; c < row_vec; c += WAVE) __builtin_nontemporal_store(z, o + c);
+            for (int sl = s0; sl < s1; ++sl) {
+                if (m == 0 && cnt > M && status && lane == 0) *status = 1;
+                if (m >= cnt) {
+                    u32x4* o = send + (size_t)sl * row_vec;
+                    for (int c = lane; c < row_vec; c += WAVE) __builtin_nontemporal_store(z, o + c);
+                }
+                if (++m == M && sl + 1 < s1) { m = 0; cnt = dst_sizes[++d]; }
+            }
             continue;
         }
         // destination rows of the token's k slots (-1: beyond the pair capacity, dropped like the gather drops it)
@@ -640,21 +649,30 @@ __global__ __launch_bounds__(256) void row_map_kernel(const int32_t* __restrict_
     map[r] = m < M ? s * M + m : -1;
 }
 
-// rows [size_s, M) of every slot s of a [W,M,row] buffer <- 0, size_s = sum over e of rc[s,e] (one wave per row)
-__global__ __launch_bounds__(256) void zero_padding_rows_kernel(u32x4* __restrict__ buf, const int32_t* __restrict__ rc, int W,
-                                                                 int E_l, int M, int row_vecs) {
-    const int wave = threadIdx.x / WAVE, lane = lane_id();
-    const int r = blockIdx.x * (blockDim.x / WAVE) + wave;
-    if (r >= W * M) return;
-    const int s = r / M, m = r % M;
+// rows [size_s, M) of every slot s of a [W,M,row] buffer <- 0, size_s = sum over e of rc[s,e]; one wave per run of
+// PACK_ZR consecutive rows (the slot's size is summed once per run, or twice when the run crosses into the next slot)
+__device__ __forceinline__ int slot_size(const int32_t* __restrict__ rc, int s, int E_l, int lane) {
     int size = 0;
     for (int e = lane; e < E_l; e += WAVE) size += rc[s * E_l + e];
 #pragma unroll
     for (int off = WAVE / 2; off >= 1; off >>= 1) size += __shfl_xor(size, off, WAVE);
-    if (m < size) return;
-    u32x4* row = buf + (size_t)r * row_vecs;
+    return size;
+}
+__global__ __launch_bounds__(256) void zero_padding_rows_kernel(u32x4* __restrict__ buf, const int32_t* __restrict__ rc, int W,
+                                                                 int E_l, int M, int row_vecs) {
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const int r0 = (blockIdx.x * (blockDim.x / WAVE) + wave) * PACK_ZR, r1 = min(r0 + PACK_ZR, W * M);
+    if (r0 >= r1) return;
+    int s = r0 / M, m = r0 % M;
+    int size = slot_size(rc, s, E_l, lane);
     const u32x4 z = {0u, 0u, 0u, 0u};
-    for (int c = lane; c < row_vecs; c += WAVE) __builtin_nontemporal_store(z, row + c);
+    for (int r = r0; r < r1; ++r) {
+        if (m >= size) {
+            u32x4* row = buf + (size_t)r * row_vecs;
+            for (int c = lane; c < row_vecs; c += WAVE) __builtin_nontemporal_store(z, row + c);
+        }
+        if (++m == M && r + 1 < r1) { m = 0; size = slot_size(rc, ++s, E_l, lane); }
+    }
 }
 
 // map_ws of the recv-driven entry points: three prefix tables plus room for a transposed copy of the counts
@@ -808,8 +826,8 @@ extern "C" int moe_pack_tokens(const void* x, int dtype, int T, int H, const int
     MOE_REQUIRE((long long)W * M + T < (1ll << 31), MOE_ERR_UNSUPPORTED, "pack_tokens: W*M + T too large");
     MOE_REQUIRE(send_buf && dst_sizes && dst_offsets, MOE_ERR_INVALID, "pack_tokens: null pointer");
     MOE_REQUIRE(T == 0 || (x && topk_idx && pos), MOE_ERR_INVALID, "pack_tokens: null pointer");
-    const int n_rows = T + W * M;
-    const int blocks = min(ceil_div(n_rows, 4), 65535 * 8);
+    const int n_units = T + ceil_div(W * M, PACK_ZR);
+    const int blocks = min(ceil_div(n_units, 4), 65535 * 8);
     pack_tokens_kernel<4><<<blocks, 4 * WAVE, 0, (hipStream_t)stream>>>((const u32x4*)x, (u32x4*)send_buf, topk_idx, pos, dst_sizes,
                                                                         dst_offsets, T, k, E_l, W, M,
                                                                         H * dtype_size(dtype) / 16, status);
@@ -895,7 +913,7 @@ extern "C" int moe_zero_padding_rows(void* buf, int dtype, int W, int M, int H, 
     if (rc) return rc;
     MOE_REQUIRE(W > 0 && E_l > 0 && M >= 1 && buf && recv_counts, MOE_ERR_INVALID, "zero_padding_rows: bad arguments");
     MOE_REQUIRE((long long)W * M < (1ll << 31), MOE_ERR_UNSUPPORTED, "zero_padding_rows: too many rows");
-    zero_padding_rows_kernel<<<ceil_div(W * M, 4), 256, 0, (hipStream_t)stream>>>((u32x4*)buf, recv_counts, W, E_l, M,
+    zero_padding_rows_kernel<<<ceil_div(ceil_div(W * M, PACK_ZR), 4), 256, 0, (hipStream_t)stream>>>((u32x4*)buf, recv_counts, W, E_l, M,
                                                                                   H * dtype_size(dtype) / 16);
     return moe_check_launch("zero_padding_rows");
 }
