@@ -714,6 +714,12 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         // (the lane-derived constants of the epilogue are derived here, once per tile, from a fresh read of the lane id)
         const int lane_e = gg_lane_now(), rbase_e = (wave_s >> 1) * (BM / NWM), cbase_e = (wave_s & 1) * (BN / 2);
         const int lsub = FP8 ? (lane_e >> 5) : (lane_e >> 4);  // which of the lanes that share a tile row this one is
+        // What the tile's top requested into LDS (scales, row map) is behind two block ends of the K loop at least -- the
+        // second one has waited for it in every wave -- unless the tile has only two stages:
+        if (nks < 4 && (FP8 || p.c_map)) {
+            gg_wait<0, 15>();
+            __syncthreads();
+        }
         bool ok[TM];
         bf16_t* crow[TM];
         float rs[TM];

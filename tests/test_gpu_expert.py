@@ -118,7 +118,8 @@ def test_expert_mlp(dtype, act, E_l, H, F, S):
                                            # more tiles than workgroups, short K: the ring runs on from tile to tile (K = 192,
                                            # 320: six and ten stages, so consecutive tiles start in different ring slots) or,
                                            # with four stages (K = 128), every tile is set up on its own
-                                           (3, 128, 2048, 9000, "none"), (2, 192, 2048, 9500, "none"), (5, 320, 1024, 17000, "swiglu")])
+                                           (3, 128, 2048, 9000, "none"), (2, 192, 2048, 9500, "none"), (5, 320, 1024, 17000, "swiglu"),
+                                           (2, 64, 2048, 9100, "none")])  # two stages per tile: the shortest K
 def test_grouped_gemm_mapped(E_l, K, N, S, act):
     """Row indirection on both sides: logical row r is read from a scattered row of a larger buffer and its
     result is written to a scattered row of a larger output.  The result must be bit for bit what the plain
