@@ -429,25 +429,21 @@ __global__ __launch_bounds__(WPB * WAVE) void pack_tokens_kernel(const u32x4* __
             }
         }
         const u32x4* src = x + (size_t)r * row_vec;
-        int c = lane;
-        for (; c + 7 * WAVE < row_vec; c += 8 * WAVE) {
+        // eight 16-byte loads in flight per lane (fewer at the end of a row, or when the row is shorter than 8 KB)
+        for (int c = lane; c < row_vec; c += 8 * WAVE) {
             u32x4 v[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(src + c + u * WAVE);
+            for (int u = 0; u < 8; ++u)
+                if (c + u * WAVE < row_vec) v[u] = __builtin_nontemporal_load(src + c + u * WAVE);
 #pragma unroll
             for (int j = 0; j < MOE_MAX_TOPK; ++j) {
                 if (j < k && drow[j] >= 0) {
                     u32x4* o = send + (size_t)drow[j] * row_vec + c;
 #pragma unroll
-                    for (int u = 0; u < 8; ++u) __builtin_nontemporal_store(v[u], o + u * WAVE);
+                    for (int u = 0; u < 8; ++u)
+                        if (c + u * WAVE < row_vec) __builtin_nontemporal_store(v[u], o + u * WAVE);
                 }
             }
-        }
-        for (; c < row_vec; c += WAVE) {
-            const u32x4 v = __builtin_nontemporal_load(src + c);
-#pragma unroll
-            for (int j = 0; j < MOE_MAX_TOPK; ++j)
-                if (j < k && drow[j] >= 0) __builtin_nontemporal_store(v, send + (size_t)drow[j] * row_vec + c);
         }
     }
 }
