@@ -212,3 +212,107 @@ def test_more_rounds_than_the_tile_table_holds():
     torch.cuda.synchronize()
     ref = x[keep].float() @ w[0].float()
     _close(out, ref, "rows of the first, a middle and the last rounds")
+
+
+def test_bf16_gemm_over_random_shapes_and_maps():
+    """Thirty seeded launches over the corners of the kernel's shape space -- K from two ring stages up, column counts that
+    are no multiple of a tile or of a 32-column group, empty and one-row groups, more tiles than workgroups or fewer, row
+    maps on either side with dropped (negative) rows, every epilogue, with and without the K-split workspace -- each
+    compared element by element with a plain fp32 product of the same operands."""
+    rng = np.random.default_rng(2024)
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    ws = ops.gemm_part_workspace(DEV)
+    try:
+        for case in range(30):
+            E_l = int(rng.integers(1, 7))
+            K = 64 * int(rng.choice([1, 2, 3, 4, 5, 8, 11, 16]))
+            act = str(rng.choice(["none", "none", "swiglu", "gelu", "silu"]))
+            N = int(rng.choice([32, 96, 264, 1024, 2080, 4096])) if act != "swiglu" else int(rng.choice([32, 96, 512, 1504, 4096]))
+            big = rng.random() < 0.4
+            cnt = rng.integers(0, 4000 if big else 300, size=E_l).astype(np.int32)
+            cnt[rng.integers(0, E_l)] = int(rng.choice([0, 1, 255, 256, 257]))
+            S = int(cnt.sum())
+            if S == 0:
+                cnt[0] = 5
+                S = 5
+            n_in, n_out = S + 37, S + 11
+            use_amap, use_cmap, split = rng.random() < 0.6, rng.random() < 0.6, rng.random() < 0.5
+            print(f"case {case}: E_l={E_l} K={K} N={N} act={act} cnt={cnt.tolist()} a_map={use_amap} c_map={use_cmap} split={split}", flush=True)
+            base = torch.from_numpy(rng.standard_normal((n_in, K)).astype(np.float32)).to(DEV).bfloat16()
+            w = torch.from_numpy((rng.standard_normal((E_l, K, N)) * K ** -0.5).astype(np.float32)).to(DEV).bfloat16()
+            wu = torch.from_numpy((rng.standard_normal((E_l, K, N)) * K ** -0.5).astype(np.float32)).to(DEV).bfloat16() if act == "swiglu" else None
+            a_map = rng.permutation(n_in)[:S].astype(np.int32) if use_amap else np.arange(S, dtype=np.int32)
+            c_map = rng.permutation(n_out)[:S].astype(np.int32) if use_cmap else np.arange(S, dtype=np.int32)
+            dropped = rng.random(S) < 0.02 if use_cmap else np.zeros(S, bool)
+            c_map_dev = np.where(dropped, -1, c_map).astype(np.int32)
+            out = torch.full((n_out, N), -7.0, dtype=torch.bfloat16, device=DEV)
+            ops.grouped_gemm_mapped(base, torch.from_numpy(a_map).to(DEV) if use_amap else None, ops.prepack_weights(w, wu),
+                                    torch.from_numpy(cnt).to(DEV), S, N, act, out,
+                                    torch.from_numpy(c_map_dev).to(DEV) if use_cmap else None, part_ws=ws if split else None)
+            torch.cuda.synchronize()
+            x = base[torch.from_numpy(a_map).long().to(DEV)].float()
+            ref = torch.empty((S, N), dtype=torch.float32, device=DEV)
+            r0 = 0
+            for e, c in enumerate(cnt.tolist()):
+                if c:
+                    g = x[r0:r0 + c] @ w[e].float()
+                    if act == "swiglu":
+                        g = torch.nn.functional.silu(g) * (x[r0:r0 + c] @ wu[e].float())
+                    elif act == "gelu":
+                        g = torch.nn.functional.gelu(g)
+                    elif act == "silu":
+                        g = torch.nn.functional.silu(g)
+                    ref[r0:r0 + c] = g
+                r0 += c
+            kept = torch.from_numpy(~dropped).to(DEV)
+            got = out[torch.from_numpy(c_map).long().to(DEV)]
+            _close(got[kept], ref[kept], f"case {case}")
+            written = np.zeros(n_out, bool)
+            written[c_map[~dropped]] = True
+            assert bool((out[torch.from_numpy(~written).to(DEV)] == -7.0).all()), f"case {case}: a row outside the map (or a dropped one) was written"
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prev
+
+
+def test_fp8_mlp_over_random_shapes():
+    """Twelve seeded fp8 expert MLPs (H, F multiples of 128 from the shortest K up; empty, tiny and large groups; more tiles
+    than workgroups or fewer; with and without the K-split workspace), each GEMM compared element by element with an fp32
+    product of the decoded codes and scales the kernels themselves used."""
+    from helpers import O
+    rng = np.random.default_rng(77)
+    part = ops.gemm_part_workspace(DEV)
+    for case in range(12):
+        E_l = int(rng.integers(1, 6))
+        H = 128 * int(rng.choice([1, 2, 3, 5, 8, 16]))
+        F = 128 * int(rng.choice([1, 2, 3, 11, 16]))
+        big = rng.random() < 0.4
+        cnt = rng.integers(0, 5000 if big else 300, size=E_l).astype(np.int32)
+        cnt[rng.integers(0, E_l)] = int(rng.choice([0, 1, 255, 257]))
+        if int(cnt.sum()) == 0:
+            cnt[0] = 9
+        S = int(cnt.sum())
+        split = rng.random() < 0.5
+        print(f"case {case}: E_l={E_l} H={H} F={F} cnt={cnt.tolist()} split={split}", flush=True)
+        x = torch.from_numpy((rng.standard_normal((S, H)) * rng.uniform(0.3, 3.0, (S, 1))).astype(np.float32)).to(DEV).bfloat16()
+        qs = [O.quantize_cols_fp8((rng.standard_normal(sh) * sc).astype(np.float32))
+              for sh, sc in (((E_l, H, F), H ** -0.5), ((E_l, H, F), H ** -0.5), ((E_l, F, H), F ** -0.5))]
+        (gq, gs), (uq, us), (dq, ds) = [(torch.from_numpy(q).to(DEV), torch.from_numpy(s).to(DEV)) for q, s in qs]
+        p1, p2 = ops.prepack_weights_fp8(gq, uq), ops.prepack_weights_fp8(dq)
+        ws = ops.fp8_workspace(S, H, F, DEV)
+        y = ops.grouped_mlp_fp8(x, torch.from_numpy(cnt).to(DEV), F, p1, gs, us, p2, ds, ws=ws, part_ws=part if split else None)
+        torch.cuda.synchronize()
+        xd, hd = _dec(ws["xq"]), _dec(ws["hq"])
+        h_ref = torch.empty((S, F), dtype=torch.float32, device=DEV)
+        y_ref = torch.empty((S, H), dtype=torch.float32, device=DEV)
+        r0 = 0
+        for e, c in enumerate(cnt.tolist()):
+            if c:
+                sx = ws["xs"][r0:r0 + c, None]
+                g = (xd[r0:r0 + c] @ _dec(gq[e])) * sx * gs[e][None, :]
+                u = (xd[r0:r0 + c] @ _dec(uq[e])) * sx * us[e][None, :]
+                h_ref[r0:r0 + c] = torch.nn.functional.silu(g) * u
+                y_ref[r0:r0 + c] = (hd[r0:r0 + c] @ _dec(dq[e])) * ws["hs"][r0:r0 + c, None] * ds[e][None, :]
+            r0 += c
+        _close(ws["h"], h_ref, f"case {case} gate/up + SwiGLU")
+        _close(y, y_ref, f"case {case} down")
