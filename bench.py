@@ -257,7 +257,7 @@ def main():
         v, secs, threads, desc = cpu_baseline(cfg, (x_np, router_np, bias_np, w_np), sample)
         out["cpu_baseline"] = {"value": round(v, 1), "unit": "tokens/s", "cores": threads, "kind": "port",
                                "sample": desc, "seconds": round(secs, 2), "host_cpus": os.cpu_count(),
-                               "per_element_loop_config1": per_element_loop_baseline()}
+                               "per_element_loop_plumbing": per_element_loop_baseline()}
     print(json.dumps(out), flush=True)
 
 
