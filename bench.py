@@ -111,6 +111,9 @@ def main():
     ap.add_argument("--config", default="mixtral")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="skip the HIP-graph replay timing")
+    ap.add_argument("--bf16-dispatch", action="store_true",
+                    help="fp8 workloads: send the tokens as bf16 and quantise them at the destination (default: quantise "
+                         "them where they are packed and send fp8 codes and scales)")
     ap.add_argument("--unfused", action="store_true",
                     help="run the destination side as unpack + MLP + return pack (the reference's operator split) "
                          "instead of gathering / scattering inside the GEMMs")
@@ -136,7 +139,8 @@ def main():
     # ---- untimed set-up: W seeded shards routed and packed, rank 0's receive buffer assembled
     world = harness.build_world(cfg, dev)
     ew, raw, qs = harness.expert_weights(cfg, 0, dev)
-    pipe = DispatchPipeline(world, ew, fused=False if args.unfused else None)
+    pipe = DispatchPipeline(world, ew, fused=False if args.unfused else None,
+                            fp8_dispatch=False if (args.unfused or args.bf16_dispatch) else None)
     # the returned buffer: slot 0 is rank 0's own return slot; the other slots stand in for what the
     # other ranks' experts would send back (same shape and dtype, arbitrary finite contents)
     pipe.step()
@@ -208,7 +212,9 @@ def main():
     dom = "mlp_up"  # the gate/up grouped GEMM: most of the flops of a step
     traffic, traffic_source = profiled_traffic(cfg.name, dom)
     if cfg.quant == "fp8":
-        kname = "moe_grouped_mlp_fp8 (row quantisation + gate/up GEMM + SwiGLU + re-quantisation + down GEMM)"
+        kname = ("moe_grouped_mlp_fp8_q (gate/up GEMM + SwiGLU + re-quantisation + down GEMM; the tokens arrive quantised)"
+                 if pipe.fp8_dispatch else
+                 "moe_grouped_mlp_fp8 (row quantisation + gate/up GEMM + SwiGLU + re-quantisation + down GEMM)")
     elif cfg.dtype == "f32":
         kname = "moe_grouped_mlp fp32 (both GEMMs)"
     else:
@@ -234,6 +240,7 @@ def main():
         "host_wall_ms_per_step": round(wall * 1e3 / args.steps, 4),
         "launch": launch,
         "destination_side": "gather/scatter inside the GEMMs" if pipe.fused else "unpack + MLP + return pack",
+        "dispatch": "fp8 codes + row scales (quantised while packing)" if pipe.fp8_dispatch else cfg.dtype,
         "ms_per_step_stream": round(stream_ms_per_step, 4),
         "ms_per_step_graph": None if ms_graph is None else round(ms_graph, 4),
         "roofline": roofline,

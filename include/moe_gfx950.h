@@ -118,6 +118,15 @@ int moe_pack_tokens(const void* x, int dtype, int T, int H, const int32_t* topk_
                     int E_l, const int32_t* dst_sizes, const int32_t* dst_offsets, int W, int M, void* send_buf,
                     int32_t* status, moe_stream_t stream);
 
+/* The fp8 form of the same send buffer (BASELINE workload "quantized skew sweep": activations quantised per token to
+ * e4m3 for the fp8 grouped GEMM).  Per-row quantisation commutes with moving rows, so the tokens can be quantised where
+ * they are packed: send_q [W,M,H] codes and send_scale [W,M] hold, slot for slot, what moe_quantize_rows_fp8 would make
+ * of moe_pack_tokens' bf16 buffer (padding slots: codes 0, scale 1), half the bytes cross, and the destination hands both
+ * to moe_grouped_mlp_fp8_q_mapped without a quantisation pass of its own.  x is bf16.  Same README.md:5-7 layout. */
+int moe_pack_tokens_fp8(const void* x_bf16, int T, int H, const int32_t* topk_idx, const int32_t* pos, int k, int E_l,
+                        const int32_t* dst_sizes, const int32_t* dst_offsets, int W, int M, uint8_t* send_q,
+                        float* send_scale, int32_t* status, moe_stream_t stream);
+
 /* ---- a9: receive layout (reference baseline.py:178-222; kernels.py:93-102,124-125) ------------
  * recv [W,M,H]: slot s holds what source s sent to this rank ((el, token) order, zero padded);
  * recv_counts [W,E_l]: recv_counts[s,e] rows from source s for local expert e.
@@ -249,6 +258,16 @@ int moe_grouped_mlp_fp8_mapped(const void* a_base_bf16, int a_rows, const int32_
                                const float* sd, uint8_t* xq_ws, float* xs_ws, void* h_ws, uint8_t* hq_ws, float* hs_ws,
                                void* out, int out_rows, const int32_t* c_row_map, void* part_ws, size_t part_ws_bytes,
                                moe_stream_t stream);
+
+/* moe_grouped_mlp_fp8_mapped for rows that arrive quantised (moe_pack_tokens_fp8): a_q [a_rows,H] codes and a_scale
+ * [a_rows] scales, gathered through a_row_map (nullable) by the first GEMM as it loads them; xs_ws [S_rows] receives the
+ * scales in the GEMM's row order.  Everything else as in moe_grouped_mlp_fp8_mapped, whose result it reproduces bit for
+ * bit when a_q / a_scale are the quantised rows of that call's input. */
+int moe_grouped_mlp_fp8_q_mapped(const uint8_t* a_q, const float* a_scale, int a_rows, const int32_t* a_row_map,
+                                 const int32_t* expert_cnt, int S_rows, int H, int F, int E_l, const uint8_t* wgu_packed,
+                                 const float* sg, const float* su, const uint8_t* wd_packed, const float* sd, float* xs_ws,
+                                 void* h_ws, uint8_t* hq_ws, float* hs_ws, void* out, int out_rows,
+                                 const int32_t* c_row_map, void* part_ws, size_t part_ws_bytes, moe_stream_t stream);
 
 /* ---- gradients (every backward of the reference is an empty stub: layers/expert.py:62-64,
  * layers/token_shuffle.py:58-60, layers/all_to_all.py:121-123) -----------------------------------------------------

@@ -60,6 +60,9 @@ _SIGNATURES = {
     "moe_return_pack": (c_int, [P, c_int, c_int, c_int, P, c_int, c_int, c_int, P, P, P]),
     "moe_recv_row_map": (c_int, [P, c_int, c_int, c_int, c_int, P, P, P, P]),
     "moe_grouped_gemm_mapped": (c_int, [P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P, c_int, P, P, c_size_t, P]),
+    "moe_pack_tokens_fp8": (c_int, [P, c_int, c_int, P, P, c_int, c_int, P, P, c_int, c_int, P, P, P, P]),
+    "moe_grouped_mlp_fp8_q_mapped": (c_int, [P, P, c_int, P, P, c_int, c_int, c_int, c_int, P, P, P, P, P, P, P, P, P, P, c_int,
+                                             P, P, c_size_t, P]),
     "moe_grouped_gemm_act_keep": (c_int, [P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P, P, c_size_t, P]),
     "moe_gemm_part_workspace_bytes": (c_size_t, []),
     "moe_prepack_weights_transposed": (c_int, [P, P, c_int, c_int, c_int, c_int, P, P]),

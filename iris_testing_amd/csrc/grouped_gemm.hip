@@ -1151,6 +1151,107 @@ __global__ __launch_bounds__(256) void quantize_rows_fp8_kernel(const bf16_t* __
     }
 }
 
+// ---- quantise and pack in one pass: the token rows leave the source as fp8 codes and one scale per row -----------------
+// Per-row quantisation commutes with moving rows: send_q / send_scale hold, slot for slot, what quantize_rows_fp8 would make
+// of the bf16 send buffer (padding slots: codes 0, scale 1, as for an all-zero row) -- so the destination can feed them to
+// the fp8 GEMM as they arrive, and half the bytes cross.  Units [0, T) of the launch are tokens (one wave each: the row is
+// read once, quantised in registers, stored to its k slots); the units after them are runs of PACKQ_ZR slots that are
+// written only where they are padding.
+constexpr int PACKQ_ZR = 8;
+template <int NV>
+__global__ __launch_bounds__(256) void pack_tokens_fp8_kernel(const bf16_t* __restrict__ x, int T, int cols,
+                                                               const int32_t* __restrict__ idx, const int32_t* __restrict__ pos,
+                                                               const int32_t* __restrict__ dst_sizes,
+                                                               const int32_t* __restrict__ dst_offsets, int k, int E_l, int W, int M,
+                                                               uint8_t* __restrict__ send_q, float* __restrict__ send_scale,
+                                                               int32_t* __restrict__ status) {
+    const int wave = threadIdx.x / WAVE, lane = lane_id();
+    const int nv = cols / 8;  // 16-byte vectors of bf16 per row = 8-byte vectors of codes
+    const int n_slots = W * M;
+    const int n_units = T + (n_slots + PACKQ_ZR - 1) / PACKQ_ZR;
+    for (int r = blockIdx.x * 4 + wave; r < n_units; r += gridDim.x * 4) {
+        if (r >= T) {
+            const int s0 = (r - T) * PACKQ_ZR, s1 = min(s0 + PACKQ_ZR, n_slots);
+            int d = s0 / M, m = s0 % M;
+            int cnt = dst_sizes[d];
+            for (int sl = s0; sl < s1; ++sl) {
+                if (m == 0 && cnt > M && status && lane == 0) *status = 1;
+                if (m >= cnt) {
+                    uint2* o = (uint2*)(send_q + (size_t)sl * cols);
+                    for (int c = lane; c < nv; c += WAVE) o[c] = make_uint2(0u, 0u);
+                    if (lane == 0) send_scale[sl] = 1.f;
+                }
+                if (++m == M && sl + 1 < s1) { m = 0; cnt = dst_sizes[++d]; }
+            }
+            continue;
+        }
+        int drow[MOE_MAX_TOPK];
+#pragma unroll
+        for (int j = 0; j < MOE_MAX_TOPK; ++j) {
+            drow[j] = -1;
+            if (j < k) {
+                const int d = idx[(size_t)r * k + j] / E_l;
+                const bool d_ok = (unsigned)d < (unsigned)W;
+                const int m = pos[(size_t)r * k + j] - dst_offsets[d_ok ? d : 0];
+                if (d_ok && (unsigned)m < (unsigned)M) drow[j] = d * M + m;
+            }
+        }
+        const uint4* src = (const uint4*)(x + (size_t)r * cols);
+        uint4 held[NV > 0 ? NV : 1];
+        float amax = 0.f;
+        if constexpr (NV > 0) {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int c = lane + i * WAVE;
+                held[i] = c < nv ? src[c] : make_uint4(0, 0, 0, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < NV; ++i) amax = fp8_row_amax(held[i], amax);
+        } else {
+            for (int c = lane; c < nv; c += WAVE) amax = fp8_row_amax(src[c], amax);
+        }
+#pragma unroll
+        for (int off = WAVE / 2; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, WAVE));
+        const bool zero = amax == 0.f;
+        const float inv = zero ? 1.f : __fdiv_rn(448.f, amax);
+        const float sc = zero ? 1.f : __fdiv_rn(amax, 448.f);
+        if constexpr (NV > 0) {
+            uint2 code[NV];
+#pragma unroll
+            for (int i = 0; i < NV; ++i) code[i] = fp8_row_convert(held[i], inv);
+#pragma unroll
+            for (int j = 0; j < MOE_MAX_TOPK; ++j) {
+                if (j < k && drow[j] >= 0) {
+                    uint2* o = (uint2*)(send_q + (size_t)drow[j] * cols);
+#pragma unroll
+                    for (int i = 0; i < NV; ++i) {
+                        const int c = lane + i * WAVE;
+                        if (c < nv) o[c] = code[i];
+                    }
+                    if (lane == 0) send_scale[drow[j]] = sc;
+                }
+            }
+        } else {
+            for (int c = lane; c < nv; c += WAVE) {
+                const uint2 code = fp8_row_convert(src[c], inv);
+#pragma unroll
+                for (int j = 0; j < MOE_MAX_TOPK; ++j)
+                    if (j < k && drow[j] >= 0) ((uint2*)(send_q + (size_t)drow[j] * cols))[c] = code;
+            }
+#pragma unroll
+            for (int j = 0; j < MOE_MAX_TOPK; ++j)
+                if (j < k && drow[j] >= 0 && lane == 0) send_scale[drow[j]] = sc;
+        }
+    }
+}
+
+// out[r] = scale[map[r]] (map NULL: scale[r]; a negative entry takes row 0, like the GEMM's row gather)
+__global__ __launch_bounds__(256) void gather_scale_kernel(const float* __restrict__ scale, const int32_t* __restrict__ map, int n,
+                                                            float* __restrict__ out) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r < n) out[r] = scale[map ? max(map[r], 0) : r];
+}
+
 // ---- backward pass helpers -----------------------------------------------------------------------------------------
 // Re-tiling of w [E_l,K,N] as the weights of the TRANSPOSED product (d tokens = d out @ w^T: reduction over N, K output
 // columns): out[e][n / SK][k][n % SK] = w[e][k][n], rows k in [K, Kpad) zero.  No transposition is involved: the 64-byte
@@ -1636,6 +1737,60 @@ extern "C" int moe_grouped_mlp_fp8(const void* tokens_bf16, const int32_t* exper
                                    void* out, moe_stream_t stream) {
     return moe_grouped_mlp_fp8_mapped(tokens_bf16, S_rows, nullptr, expert_cnt, S_rows, H, F, E_l, wgu_packed, sg, su, wd_packed,
                                       sd, xq_ws, xs_ws, h_ws, hq_ws, hs_ws, out, S_rows, nullptr, nullptr, 0, stream);
+}
+
+extern "C" int moe_pack_tokens_fp8(const void* x_bf16, int T, int H, const int32_t* topk_idx, const int32_t* pos, int k, int E_l,
+                                   const int32_t* dst_sizes, const int32_t* dst_offsets, int W, int M, uint8_t* send_q,
+                                   float* send_scale, int32_t* status, moe_stream_t stream) {
+    MOE_REQUIRE(T >= 0 && H > 0 && H % 8 == 0 && W > 0 && M >= 1 && E_l > 0, MOE_ERR_INVALID, "pack_tokens_fp8: bad shape");
+    MOE_REQUIRE(k >= 1 && k <= MOE_MAX_TOPK, MOE_ERR_UNSUPPORTED, "pack_tokens_fp8: topk=%d outside [1,%d]", k, MOE_MAX_TOPK);
+    MOE_REQUIRE((long long)W * M + T < (1ll << 31), MOE_ERR_UNSUPPORTED, "pack_tokens_fp8: W*M + T too large");
+    MOE_REQUIRE(send_q && send_scale && dst_sizes && dst_offsets, MOE_ERR_INVALID, "pack_tokens_fp8: null pointer");
+    MOE_REQUIRE(T == 0 || (x_bf16 && topk_idx && pos), MOE_ERR_INVALID, "pack_tokens_fp8: null pointer");
+    const int n_units = T + ceil_div(W * M, PACKQ_ZR);
+    const int blocks = min(ceil_div(n_units, 4), 65535 * 8);
+    const int nv = ceil_div(H / 8, WAVE);
+    hipStream_t s = (hipStream_t)stream;
+#define GG_PQ(NVv) pack_tokens_fp8_kernel<NVv><<<blocks, 256, 0, s>>>((const bf16_t*)x_bf16, T, H, topk_idx, pos, dst_sizes, dst_offsets, k, E_l, W, M, send_q, send_scale, status)
+    if (nv <= 2) GG_PQ(2);
+    else if (nv <= 4) GG_PQ(4);
+    else if (nv <= 8) GG_PQ(8);
+    else if (nv <= 16) GG_PQ(16);
+    else GG_PQ(0);
+#undef GG_PQ
+    return moe_check_launch("pack_tokens_fp8");
+}
+
+extern "C" int moe_grouped_mlp_fp8_q_mapped(const uint8_t* a_q, const float* a_scale, int a_rows, const int32_t* a_row_map,
+                                            const int32_t* expert_cnt, int S_rows, int H, int F, int E_l,
+                                            const uint8_t* wgu_packed, const float* sg, const float* su,
+                                            const uint8_t* wd_packed, const float* sd, float* xs_ws, void* h_ws, uint8_t* hq_ws,
+                                            float* hs_ws, void* out, int out_rows, const int32_t* c_row_map, void* part_ws,
+                                            size_t part_ws_bytes, moe_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    MOE_REQUIRE(S_rows >= 0 && H > 0 && F > 0 && E_l > 0 && E_l <= GG_MAXG, MOE_ERR_INVALID, "grouped_mlp_fp8_q: bad shape");
+    MOE_REQUIRE(H % 128 == 0 && F % 128 == 0, MOE_ERR_UNSUPPORTED, "grouped_mlp_fp8_q: needs H, F multiples of 128 (H=%d F=%d)", H, F);
+    MOE_REQUIRE(a_rows >= 0 && out_rows >= 0, MOE_ERR_INVALID, "grouped_mlp_fp8_q: negative buffer rows");
+    MOE_REQUIRE(!a_row_map || (unsigned long long)a_rows * (unsigned long long)H < (1ull << 32), MOE_ERR_UNSUPPORTED,
+                "grouped_mlp_fp8_q: the gathered buffer must be smaller than 4 GiB (%d rows of %d)", a_rows, H);
+    if (S_rows == 0) return MOE_OK;
+    MOE_REQUIRE(a_q && a_scale && expert_cnt && wgu_packed && sg && su && wd_packed && sd && xs_ws && h_ws && hq_ws && hs_ws && out,
+                MOE_ERR_INVALID, "grouped_mlp_fp8_q: null pointer");
+    // the row scales in the order of the GEMM's rows (the codes themselves are gathered by the GEMM as it loads them)
+    gather_scale_kernel<<<ceil_div(S_rows, 256), 256, 0, s>>>(a_scale, a_row_map, S_rows, xs_ws);
+    GemmParams p{};
+    p.A = a_q; p.B = wgu_packed; p.C = h_ws; p.cnt = expert_cnt; p.row_scale = xs_ws; p.col_scale = sg; p.col_scale2 = su;
+    p.a_map = a_row_map;
+    p.E_l = E_l; p.K = H; p.N = F; p.Npad = round_up(2 * F, GG_BN); p.ldc = F; p.S_rows = S_rows; p.ncs = F;
+    int rc = launch_gemm<true>(p, EPI_SWIGLU, s, part_ws, part_ws_bytes);
+    if (rc) return rc;
+    rc = launch_quantize(h_ws, nullptr, S_rows, F, hq_ws, hs_ws, nullptr, s);
+    if (rc) return rc;
+    GemmParams q{};
+    q.A = hq_ws; q.B = wd_packed; q.C = out; q.cnt = expert_cnt; q.row_scale = hs_ws; q.col_scale = sd;
+    q.c_map = c_row_map;
+    q.E_l = E_l; q.K = F; q.N = H; q.Npad = round_up(H, GG_BN); q.ldc = H; q.S_rows = S_rows; q.ncs = H;
+    return launch_gemm<true>(q, EPI_NONE, s, part_ws, part_ws_bytes);
 }
 
 // ---- backward pass entry points --------------------------------------------------------------------------------------

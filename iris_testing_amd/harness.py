@@ -37,6 +37,10 @@ class World:
     recv: torch.Tensor               # [W,M,H] what rank 0 receives
     recv_counts: torch.Tensor        # [W,E_l] i32: recv_counts[s,e] rows from source s for local expert e
     S: int                           # rows received by rank 0
+    # fp8 workloads: the same receive buffer as the sources send it when they quantise their tokens while packing
+    # (ops.pack_tokens_fp8): per-row codes [W,M,H] and scales [W,M]
+    recv_q: Optional[torch.Tensor] = None
+    recv_scale: Optional[torch.Tensor] = None
 
 
 def route_shard(cfg: MoEConfig, x: torch.Tensor, router: torch.Tensor, bias: Optional[torch.Tensor]) -> ShardRoute:
@@ -73,6 +77,11 @@ def build_world(cfg: MoEConfig, device="cuda", dst_rank: int = 0, keep_shards: b
         recv_counts[s] = routes[s].counts.send_counts[dst_rank]
     S = int(recv_counts.sum().item())
     w = World(cfg, router, bias, shards[0], routes, M, CAP, recv, recv_counts, S)
+    if cfg.quant == "fp8":
+        # (per-row quantisation commutes with moving rows: quantising the assembled buffer row by row gives what W
+        # quantise-and-pack launches would have sent)
+        q, sc = ops.quantize_rows_fp8(recv.view(cfg.world * M, cfg.hidden))
+        w.recv_q, w.recv_scale = q.view(cfg.world, M, cfg.hidden), sc.view(cfg.world, M)
     return (w, shards) if keep_shards else w
 
 

@@ -139,6 +139,30 @@ def pack_tokens(x: torch.Tensor, topk_idx: torch.Tensor, pos: torch.Tensor, dst_
     return out
 
 
+def pack_tokens_fp8(x: torch.Tensor, topk_idx: torch.Tensor, pos: torch.Tensor, dst_sizes: torch.Tensor,
+                    dst_offsets: torch.Tensor, e_local: int, M: int, out_q: Optional[torch.Tensor] = None,
+                    out_scale: Optional[torch.Tensor] = None, status: Optional[torch.Tensor] = None):
+    """pack_tokens with the per-token fp8 quantisation done on the way: ([W,M,H] uint8 codes, [W,M] fp32 scales) -- slot for
+    slot what quantize_rows_fp8 makes of pack_tokens' bf16 buffer."""
+    _req_cuda(x, "tokens")
+    assert x.dtype == torch.bfloat16 and x.is_contiguous()
+    for t, n in ((topk_idx, "topk_idx"), (pos, "pos"), (dst_sizes, "dst_sizes"), (dst_offsets, "dst_offsets")):
+        _req_i32(t, n)
+    T, H = x.shape
+    W = dst_sizes.numel()
+    k = topk_idx.shape[1] if topk_idx.dim() == 2 else 1
+    assert topk_idx.numel() == T * k and pos.numel() == T * k
+    if out_q is None:
+        out_q = torch.empty((W, M, H), dtype=torch.uint8, device=x.device)
+    if out_scale is None:
+        out_scale = torch.empty((W, M), dtype=torch.float32, device=x.device)
+    assert out_q.shape == (W, M, H) and out_q.dtype == torch.uint8 and out_q.is_contiguous()
+    assert out_scale.shape == (W, M) and out_scale.dtype == torch.float32 and out_scale.is_contiguous()
+    L.check(L.lib().moe_pack_tokens_fp8(L.ptr(x), T, H, L.ptr(topk_idx), L.ptr(pos), k, e_local, L.ptr(dst_sizes),
+                                        L.ptr(dst_offsets), W, M, L.ptr(out_q), L.ptr(out_scale), L.ptr(status), L.stream_ptr()))
+    return out_q, out_scale
+
+
 # ---- a9 / a10 -------------------------------------------------------------------------------
 def _map_ws(W, E_l, n_out, device, map_ws=None):
     need = L.lib().moe_recv_map_ints(W, E_l, n_out)
@@ -338,6 +362,29 @@ def grouped_mlp_fp8(tokens: torch.Tensor, expert_cnt: torch.Tensor, F: int, wgu_
                                                    L.ptr(ws["xs"]), L.ptr(ws["h"]), L.ptr(ws["hq"]), L.ptr(ws["hs"]), L.ptr(out), S,
                                                    None, L.ptr(part_ws), part_ws.numel() * part_ws.element_size(),
                                                    L.stream_ptr()))
+    return out
+
+
+
+def grouped_mlp_fp8_q(a_q: torch.Tensor, a_scale: torch.Tensor, a_row_map: Optional[torch.Tensor], expert_cnt: torch.Tensor,
+                      S_rows: int, F: int, wgu_packed, sg, su, wd_packed, sd, ws: dict, out: torch.Tensor,
+                      c_row_map: Optional[torch.Tensor] = None, part_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """grouped_mlp_fp8 for rows that arrive as fp8 codes and scales (pack_tokens_fp8): a_q [rows,H] uint8, a_scale [rows];
+    ws as from fp8_workspace (its "xq" is not used, "xs" receives the scales in row order)."""
+    _req_cuda(a_q, "a_q")
+    _req_i32(expert_cnt, "expert_cnt")
+    assert a_q.dtype == torch.uint8 and a_q.dim() == 2 and a_q.is_contiguous() and a_scale.dtype == torch.float32
+    assert a_scale.numel() == a_q.shape[0] and out.dtype == torch.bfloat16 and out.dim() == 2 and out.is_contiguous()
+    H = a_q.shape[1]
+    assert out.shape[1] == H
+    L.check(L.lib().moe_grouped_mlp_fp8_q_mapped(L.ptr(a_q), L.ptr(a_scale), a_q.shape[0],
+                                                 L.ptr(a_row_map) if a_row_map is not None else None, L.ptr(expert_cnt), S_rows, H, F,
+                                                 expert_cnt.numel(), L.ptr(wgu_packed), L.ptr(sg), L.ptr(su), L.ptr(wd_packed),
+                                                 L.ptr(sd), L.ptr(ws["xs"]), L.ptr(ws["h"]), L.ptr(ws["hq"]), L.ptr(ws["hs"]),
+                                                 L.ptr(out), out.shape[0], L.ptr(c_row_map) if c_row_map is not None else None,
+                                                 L.ptr(part_ws) if part_ws is not None else None,
+                                                 part_ws.numel() * part_ws.element_size() if part_ws is not None else 0,
+                                                 L.stream_ptr()))
     return out
 
 

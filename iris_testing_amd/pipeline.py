@@ -7,6 +7,8 @@ A step = what rank 0 does for one batch:
 With ``fused=True`` (bf16 or fp8 experts) the destination side skips the two row copies: "unpack" only builds the
 row map, the first GEMM gathers its input rows from the receive buffer, the second scatters its result rows
 into the returned layout, and "return_pack" only zeroes the padding rows.
+With ``fp8_dispatch=True`` (fp8 experts, fused) the tokens are quantised per row where they are packed: the send and
+receive buffers hold fp8 codes and one scale per row, and the destination runs no quantisation pass over its input.
 The two transfers in between are not part of a one-GPU build: the receive buffer and the returned
 buffer are assembled beforehand (harness.build_world) and stay fixed.  Each stage is one C-ABI call
 on the current stream; no stage synchronises or allocates.
@@ -26,7 +28,7 @@ STAGES = ["route", "count", "pack", "unpack", "mlp_up", "mlp_down", "return_pack
 
 class DispatchPipeline:
     def __init__(self, world: World, weights: ExpertWeights, returned: Optional[torch.Tensor] = None,
-                 fused: Optional[bool] = None):
+                 fused: Optional[bool] = None, fp8_dispatch: Optional[bool] = None):
         cfg = world.cfg
         # gather / scatter inside the GEMMs needs the bf16 MFMA path and a receive buffer under 4 GiB
         can_fuse = weights.dtype in (torch.bfloat16, torch.uint8) and \
@@ -34,6 +36,10 @@ class DispatchPipeline:
         self.fused = can_fuse if fused is None else bool(fused)
         if self.fused and not can_fuse:
             raise ValueError("the fused destination path needs bf16 or fp8 expert weights and a receive buffer under 4 GiB")
+        can_q = self.fused and weights.dtype == torch.uint8 and world.recv_q is not None and cfg.torch_dtype == torch.bfloat16
+        self.fp8_dispatch = can_q if fp8_dispatch is None else bool(fp8_dispatch)
+        if self.fp8_dispatch and not can_q:
+            raise ValueError("fp8 dispatch needs fp8 experts, bf16 tokens, the fused destination side and a quantised receive buffer")
         self.world, self.cfg, self.weights = world, cfg, weights
         dev = world.x0.device
         T, H, E, k, W, E_l, F = cfg.tokens, cfg.hidden, cfg.experts, cfg.topk, cfg.world, cfg.e_local, cfg.ffn
@@ -54,6 +60,9 @@ class DispatchPipeline:
         self.count_ws_bytes = lib.moe_count_workspace_bytes(T, k, E)
         self.count_ws = torch.empty(self.count_ws_bytes, dtype=torch.uint8, device=dev)
         self.send = torch.empty((W, M, H), dtype=dt, device=dev)
+        if self.fp8_dispatch:
+            self.send_q = torch.empty((W, M, H), dtype=torch.uint8, device=dev)
+            self.send_scale = torch.empty((W, M), dtype=torch.float32, device=dev)
         self.status = torch.zeros(1, dtype=torch.int32, device=dev)
         # destination side
         self.rows = torch.empty((S, H), dtype=dt, device=dev)
@@ -93,6 +102,11 @@ class DispatchPipeline:
 
     def pack(self, s):
         c, w = self.cfg, self.world
+        if self.fp8_dispatch:
+            L.check(L.lib().moe_pack_tokens_fp8(self._p(w.x0), c.tokens, c.hidden, self._p(self.idx), self._p(self.pos), c.topk,
+                                                c.e_local, self._p(self.dst_sizes), self._p(self.dst_offsets), c.world, w.M,
+                                                self._p(self.send_q), self._p(self.send_scale), self._p(self.status), s))
+            return
         L.check(L.lib().moe_pack_tokens(self._p(w.x0), self.code, c.tokens, c.hidden, self._p(self.idx), self._p(self.pos),
                                         c.topk, c.e_local, self._p(self.dst_sizes), self._p(self.dst_offsets), c.world, w.M,
                                         self._p(self.send), self._p(self.status), s))
@@ -115,6 +129,14 @@ class DispatchPipeline:
             # the fp8 entry point runs quantise + gate/up + quantise + down in one call; fused: input rows gathered from
             # the receive buffer, result rows scattered into the returned layout
             w = self.world
+            if self.fp8_dispatch:
+                L.check(lib.moe_grouped_mlp_fp8_q_mapped(self._p(w.recv_q), self._p(w.recv_scale), c.world * w.M,
+                                                         self._p(self.row_map), self._p(self.expert_cnt), self.S, c.hidden, c.ffn,
+                                                         c.e_local, self._p(ew.w1), self._p(sg), self._p(su), self._p(ew.w2),
+                                                         self._p(sd), self._p(self.xs), self._p(self.hidden), self._p(self.hq),
+                                                         self._p(self.hs), self._p(self.ret), c.world * w.M, self._p(self.row_map),
+                                                         self._p(self.part_ws), self.part_ws_bytes, s))
+                return
             src, n_src, a_map = (w.recv, c.world * w.M, self.row_map) if self.fused else (self.rows, self.S, None)
             dst, n_dst, c_map = (self.ret, c.world * w.M, self.row_map) if self.fused else (self.y, self.S, None)
             L.check(lib.moe_grouped_mlp_fp8_mapped(self._p(src), n_src, self._p(a_map), self._p(self.expert_cnt), self.S, c.hidden,
@@ -212,7 +234,7 @@ class DispatchPipeline:
             ret = dict(bound="hbm", amount=S * H * B + W * M * H * B)
         return {
             "route": dict(bound="hbm", amount=T * H * B + H * E * B + T * k * 8),
-            "pack": dict(bound="hbm", amount=T * H * B + W * M * H * B),
+            "pack": dict(bound="hbm", amount=T * H * B + W * M * (H + 4) if self.fp8_dispatch else T * H * B + W * M * H * B),
             "unpack": unpack,
             **mlp,
             "return_pack": ret,

@@ -382,6 +382,19 @@ def pack_fixed_m(payload: np.ndarray, dst_offsets: np.ndarray, dst_sizes: np.nda
 # --------------------------------------------------------------------------------------
 # a9: receive layout  (reference baseline.py:178-222; kernels.py:100-102,124-125)
 # --------------------------------------------------------------------------------------
+
+def pack_fixed_m_fp8(payload: np.ndarray, dst_offsets: np.ndarray, dst_sizes: np.ndarray, M: int,
+                     drop: bool = False) -> Tuple[np.ndarray, np.ndarray]:
+    """The fixed [W,M,H] send layout (README.md:5-7 of the reference) of tokens quantised per row to fp8 before they are
+    sent: (codes [W,M,H] uint8, scales [W,M] fp32) = quantize_rows_fp8 of every row of pack_fixed_m's buffer; a padding
+    slot is an all-zero row (codes 0, scale 1).  Not in the reference, which sends the token dtype: the workload
+    description asks for per-token fp8 activations, and per-row quantisation commutes with moving rows (checked in
+    tests/test_oracle_dispatch.py), so quantising at the source changes no result."""
+    send = pack_fixed_m(payload, dst_offsets, dst_sizes, M, drop=drop)
+    W, _, H = send.shape
+    q, sc = quantize_rows_fp8(send.reshape(W * M, H))
+    return q.reshape(W, M, H), sc.reshape(W, M)
+
 def reorder_flat_to_token_buf(flat: np.ndarray, recv_counts: np.ndarray, capacity: int,
                               token_buf_out: np.ndarray) -> np.ndarray:
     """token_buf[e, src, :c] = next c rows of ``flat`` for src-major, expert-minor blocks;

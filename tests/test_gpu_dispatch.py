@@ -349,3 +349,49 @@ def test_kernels_reproduce_the_frozen_dispatch_vectors():
     assert_bits_equal(ops.return_pack(rows * 2.0, rc, M), g["ret"], "return buffer")
     out = ops.combine(dev(g["send0"]) * 2.0, idx0, c0.pos, dev(g["gate0"]), c0.dst_offsets, E // W)
     assert_bits_equal(out, g["combined"], "combined output")
+
+
+@pytest.mark.parametrize("T,H,E,k,W,slack", [(90, 64, 12, 3, 4, 2), (700, 2048, 60, 8, 4, 0), (300, 7168, 16, 1, 8, 5), (64, 16384, 8, 2, 2, 1)])
+def test_pack_tokens_fp8_is_the_quantised_send_buffer(T, H, E, k, W, slack):
+    """Quantise-and-pack against the oracle (quantize_rows_fp8 of every row of the bf16 send buffer): codes and scales
+    bit-exact, padding slots codes 0 / scale 1; and against the kernels' own two-step path (pack, then quantise)."""
+    rng = np.random.default_rng(T + H)
+    x = O.bf16_round((rng.standard_normal((T, H)) * rng.uniform(0.1, 4.0, (T, 1))).astype(np.float32))
+    x[3] = 0.0
+    idx = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+    counts = O.send_counts(idx, W, E)
+    sizes, offs = O.dst_sizes_offsets(counts)
+    pos, row_token = O.payload_positions(idx, E)
+    M = O.pair_capacity(sizes) + slack
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(DEV)  # noqa: E731
+    xt = torch.from_numpy(x).bfloat16().to(DEV)
+    q = torch.full((W, M, H), 0xAB, dtype=torch.uint8, device=DEV)
+    sc = torch.full((W, M), -3.0, dtype=torch.float32, device=DEV)
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    ops.pack_tokens_fp8(xt, dev(idx), dev(pos), dev(sizes), dev(offs), E // W, M, out_q=q, out_scale=sc, status=status)
+    want_q, want_s = O.pack_fixed_m_fp8(O.send_payload(x, row_token), offs, sizes, M)
+    assert_bits_equal(q, want_q, "fp8 send codes")
+    assert_bits_equal(sc, want_s, "fp8 send scales")
+    assert int(status.item()) == 0
+    send = ops.pack_tokens(xt, dev(idx), dev(pos), dev(sizes), dev(offs), E // W, M)
+    q2, s2 = ops.quantize_rows_fp8(send.view(W * M, H))
+    assert torch.equal(q.view(W * M, H), q2) and torch.equal(sc.view(-1), s2)
+
+
+def test_pack_tokens_fp8_drops_what_the_bf16_pack_drops():
+    """An undersized M: the same rows are dropped, the status word is raised, nothing is written outside the buffers."""
+    rng = np.random.default_rng(12)
+    T, H, E, k, W = 200, 256, 8, 2, 4
+    x = O.bf16_round(rng.standard_normal((T, H)).astype(np.float32))
+    idx = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+    counts = O.send_counts(idx, W, E)
+    sizes, offs = O.dst_sizes_offsets(counts)
+    pos, row_token = O.payload_positions(idx, E)
+    M = int(sizes.max()) - 7
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(DEV)  # noqa: E731
+    status = torch.zeros(1, dtype=torch.int32, device=DEV)
+    q, sc = ops.pack_tokens_fp8(torch.from_numpy(x).bfloat16().to(DEV), dev(idx), dev(pos), dev(sizes), dev(offs), E // W, M, status=status)
+    want_q, want_s = O.pack_fixed_m_fp8(O.send_payload(x, row_token), offs, sizes, M, drop=True)
+    assert_bits_equal(q, want_q, "fp8 send codes (overflow)")
+    assert_bits_equal(sc, want_s, "fp8 send scales (overflow)")
+    assert int(status.item()) == 1

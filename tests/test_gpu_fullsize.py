@@ -114,3 +114,16 @@ def test_fused_destination_equals_copies(name):
     assert torch.equal(fused.expert_cnt, ref.expert_cnt)
     assert torch.equal(fused.ret.view(torch.int16), ref.ret.view(torch.int16)), "returned buffer differs"
     assert torch.equal(fused.out.view(torch.int16), ref.out.view(torch.int16)), "combined output differs"
+    if cfg.quant == "fp8":
+        # fused takes the tokens as fp8 codes and row scales, quantised where they were packed; the same with bf16 on the wire
+        assert fused.fp8_dispatch
+        wire = DispatchPipeline(world, ew, fused=True, fp8_dispatch=False)
+        wire.returned.copy_(back)
+        wire.ret.fill_(float("nan"))
+        wire.step()
+        torch.cuda.synchronize()
+        assert torch.equal(wire.ret.view(torch.int16), ref.ret.view(torch.int16)), "returned buffer differs (bf16 dispatch)"
+        q, sc = ops.quantize_rows_fp8(ref.send.view(-1, cfg.hidden))
+        assert torch.equal(fused.send_q.view(-1, cfg.hidden), q) and torch.equal(fused.send_scale.view(-1), sc), \
+            "quantise-and-pack differs from pack, then quantise"
+        assert torch.equal(fused.hidden.view(torch.int16), wire.hidden.view(torch.int16)), "hidden activations differ"

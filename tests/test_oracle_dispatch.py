@@ -275,3 +275,36 @@ def test_capacity_overflow_drops_the_same_rows_everywhere():
             if m < M:
                 acc = (acc + gate[t, kk] * xs[0][t]).astype(np.float32)
         assert np.array_equal(out[t], acc)
+
+
+def test_quantising_rows_commutes_with_packing_them():
+    """pack_fixed_m_fp8 (tokens quantised to fp8 where they are packed) against the other order: quantise every token row
+    first -- with torch's own e4m3 cast, as test_oracle_expert pins quantize_rows_fp8 -- then move the codes and the
+    scales as payload.  Padding slots are all-zero rows: codes 0, scale 1.  Includes an all-zero token."""
+    import torch
+    rng = np.random.default_rng(8)
+    T, H, E, k, W = 70, 48, 12, 3, 4
+    x = O.bf16_round((rng.standard_normal((T, H)) * rng.uniform(0.1, 4.0, (T, 1))).astype(np.float32))
+    x[5] = 0.0
+    idx = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+    counts = O.send_counts(idx, W, E)
+    sizes, offs = O.dst_sizes_offsets(counts)
+    pos, row_token = O.payload_positions(idx, E)
+    M = O.pair_capacity(sizes) + 3
+    q, sc = O.pack_fixed_m_fp8(O.send_payload(x, row_token), offs, sizes, M)
+    # the other order, with torch's cast
+    xt = torch.from_numpy(x)
+    amax = xt.abs().amax(dim=1)
+    zero = amax == 0
+    safe = torch.where(zero, torch.ones_like(amax), amax)
+    scale_t = torch.where(zero, torch.ones_like(amax), safe / 448.0).numpy()
+    codes_t = (xt * torch.where(zero, torch.ones_like(amax), 448.0 / safe)[:, None]).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    want_q = np.zeros((W, M, H), np.uint8)
+    want_s = np.ones((W, M), np.float32)
+    for t in range(T):
+        for j in range(k):
+            d = idx[t, j] // (E // W)
+            m = pos[t, j] - offs[d]
+            want_q[d, m], want_s[d, m] = codes_t[t], scale_t[t]
+    assert np.array_equal(q, want_q) and np.array_equal(sc, want_s)
+    assert (sc[0, sizes[0]:] == 1.0).all() and (q[0, sizes[0]:] == 0).all()
