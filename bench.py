@@ -210,7 +210,7 @@ def main():
         stages[n] = {"ms": round(ms, 4), "ms_min": round(stage_spread[n][0], 4), "ms_median": round(stage_spread[n][1], 4),
                      "bound": wk["bound"], "achieved": round(ach, 2), "peak": peak, "unit": unit, "frac": round(ach / peak, 4)}
     dom = "mlp_up"  # the gate/up grouped GEMM: most of the flops of a step
-    traffic, traffic_source = profiled_traffic(cfg.name, dom)
+    traffic, traffic_source = profiled_traffic(cfg.name, dom + "_fp8_dispatch" if pipe.fp8_dispatch else dom)
     if cfg.quant == "fp8":
         kname = ("moe_grouped_mlp_fp8_q (gate/up GEMM + SwiGLU + re-quantisation + down GEMM; the tokens arrive quantised)"
                  if pipe.fp8_dispatch else
