@@ -215,7 +215,7 @@ int moe_grouped_mlp_fp8(const void* tokens_bf16, const int32_t* expert_cnt, int 
  *   moe_recv_row_map        row_map[r] = row of the [W,M,H] receive buffer that holds expert-major row r
  *                           (r < n_rows; rows past the received total map to row 0; rows dropped by the
  *                           sender's pack, at or past row M of their slot, map to -1), expert_cnt (nullable)
- *                           as in moe_unpack_expert_major; map_ws >= moe_recv_map_ints(W,E_l,n_rows) ints.
+ *                           as in moe_unpack_expert_major; map_ws: unused (kept for ABI stability; may be NULL).
  *                           The same map is the destination of result row r in the returned buffer.
  *   moe_grouped_gemm_mapped moe_grouped_gemm_packed with row indirection: logical row r is read from row
  *                           a_row_map[r] of a_base (a_rows rows of K, under 4 GiB) and written to row

@@ -626,25 +626,50 @@ int gather_rows(const void* src, void* dst, const RowSource& a, int n_rows, int 
     return moe_check_launch("gather_rows");
 }
 
-// Expert-major row r of the receive side -> row of the [W,M,H] buffer that holds it (one thread per row,
-// binary search in the (expert, source)-major prefix).  The same index serves the way back: the result
-// row of r returns to the slot its input came from.  Rows past the received total map to row 0; rows the pack
-// dropped (position in the sender's slot at or past the pair capacity M) map to -1: the GEMMs read row 0 for them
-// and store nothing.
-__global__ __launch_bounds__(256) void row_map_kernel(const int32_t* __restrict__ row_off, const int32_t* __restrict__ src_off,
-                                                       int W, int E_l, int M, int n_rows, int32_t* __restrict__ map) {
+// Expert-major row r of the receive side -> row of the [W,M,H] buffer that holds it (one thread per row, binary search in
+// the (expert, source)-major prefix).  The same index serves the way back: the result row of r returns to the slot its input
+// came from.  Rows past the received total map to row 0; rows the pack dropped (position in the sender's slot at or past
+// the pair capacity M) map to -1: the GEMMs read row 0 for them and store nothing.
+// One launch: every block derives the two prefix tables it needs from recv_counts in LDS (at most
+// MOE_MAX_EXPERTS entries: a wave's scan) instead of waiting for a table kernel; block 0 also leaves the per-expert totals.
+__global__ __launch_bounds__(256) void row_map_from_counts_kernel(const int32_t* __restrict__ rc, int W, int E_l, int M, int n_rows,
+                                                                   int32_t* __restrict__ map, int32_t* __restrict__ expert_cnt) {
+    __shared__ int32_t s_row_off[MOE_MAX_EXPERTS + 1];
+    __shared__ int32_t s_src_off[MOE_MAX_EXPERTS];
+    const int n = W * E_l;
+    if (threadIdx.x < WAVE) {
+        const int lane = lane_id();
+        const int per = (n + WAVE - 1) / WAVE;
+        const int lo = min(lane * per, n), hi = min(lo + per, n);
+        int sum = 0;
+        for (int i = lo; i < hi; ++i) sum += rc[(i % W) * E_l + (i / W)];
+        const int incl = wave_incl_scan(sum);
+        int run = incl - sum;
+        for (int i = lo; i < hi; ++i) { s_row_off[i] = run; run += rc[(i % W) * E_l + (i / W)]; }
+        if (lane == WAVE - 1) s_row_off[n] = incl;
+        for (int sr = lane; sr < W; sr += WAVE) {
+            int r = 0;
+            for (int e = 0; e < E_l; ++e) { s_src_off[sr * E_l + e] = r; r += rc[sr * E_l + e]; }
+        }
+        if (blockIdx.x == 0 && expert_cnt)
+            for (int e = lane; e < E_l; e += WAVE) {
+                int c = 0;
+                for (int sr = 0; sr < W; ++sr) c += rc[sr * E_l + e];
+                expert_cnt[e] = c;
+            }
+    }
+    __syncthreads();
     const int r = blockIdx.x * blockDim.x + threadIdx.x;
     if (r >= n_rows) return;
-    const int n = W * E_l;
-    if (r >= row_off[n]) { map[r] = 0; return; }
-    int lo = 0, hi = n;  // row_off[0] = 0 <= r; the last of a run of equal offsets owns the row
+    if (r >= s_row_off[n]) { map[r] = 0; return; }
+    int lo = 0, hi = n;  // s_row_off[0] = 0 <= r; the last of a run of equal offsets owns the row
     while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;
-        if (row_off[mid] <= r) lo = mid; else hi = mid;
+        if (s_row_off[mid] <= r) lo = mid; else hi = mid;
     }
-    const int e = lo / W, s = lo % W;
-    const int m = src_off[s * E_l + e] + (r - row_off[lo]);
-    map[r] = m < M ? s * M + m : -1;
+    const int e = lo / W, sr = lo % W;
+    const int m = s_src_off[sr * E_l + e] + (r - s_row_off[lo]);
+    map[r] = m < M ? sr * M + m : -1;
 }
 
 // rows [size_s, M) of every slot s of a [W,M,row] buffer <- 0, size_s = sum over e of rc[s,e]; one wave per run of
@@ -892,16 +917,11 @@ extern "C" int moe_recv_row_map(const int32_t* recv_counts, int W, int E_l, int 
                                 int32_t* expert_cnt, int32_t* map_ws, moe_stream_t stream) {
     hipStream_t s = (hipStream_t)stream;
     MOE_REQUIRE(W > 0 && E_l > 0 && W * E_l <= MOE_MAX_EXPERTS, MOE_ERR_INVALID, "recv_row_map: bad W=%d E_l=%d", W, E_l);
-    MOE_REQUIRE(M >= 1 && n_rows >= 0 && recv_counts && map_ws, MOE_ERR_INVALID, "recv_row_map: bad arguments");
-    const int n = W * E_l;
-    int32_t* src_off = map_ws;
-    int32_t* row_off = map_ws + (n + 1);
-    int32_t* flat_off = map_ws + 2 * (n + 1);
-    recv_tables_kernel<<<1, WAVE, 0, s>>>(recv_counts, W, E_l, src_off, row_off, flat_off, nullptr, expert_cnt);
-    if (n_rows > 0) {
-        MOE_REQUIRE(row_map, MOE_ERR_INVALID, "recv_row_map: null pointer");
-        row_map_kernel<<<ceil_div(n_rows, 256), 256, 0, s>>>(row_off, src_off, W, E_l, M, n_rows, row_map);
-    }
+    MOE_REQUIRE(M >= 1 && n_rows >= 0 && recv_counts, MOE_ERR_INVALID, "recv_row_map: bad arguments");
+    (void)map_ws;  // (the tables of earlier versions live in LDS now)
+    MOE_REQUIRE(n_rows == 0 || row_map, MOE_ERR_INVALID, "recv_row_map: null pointer");
+    // (one launch: every block rebuilds the prefix tables in LDS; at least one block, for the per-expert totals)
+    row_map_from_counts_kernel<<<max(ceil_div(n_rows, 256), 1), 256, 0, s>>>(recv_counts, W, E_l, M, n_rows, row_map, expert_cnt);
     return moe_check_launch("recv_row_map");
 }
 
