@@ -108,6 +108,32 @@ __global__ __launch_bounds__(WAVE) void offsets_kernel(const int32_t* __restrict
     offsets_body(counts, E, W, es, expert_start, send_counts, expert_offs, dst_sizes, dst_offsets, caps);
 }
 
+// Steps 2 and 3 in one launch when the histogram is small enough for one workgroup (every wave scans the experts
+// w, w + 16, ...; then one wave derives the offsets): a launch saved on a stage that is all launches.
+constexpr int SCAN1_MAXCELLS = 1 << 16;
+__global__ __launch_bounds__(1024) void scan_offsets_kernel(const int32_t* __restrict__ hist, int32_t* __restrict__ base,
+                                                             int32_t* __restrict__ counts, int NB, int E, int W,
+                                                             int32_t* __restrict__ expert_start, int32_t* __restrict__ send_counts,
+                                                             int32_t* __restrict__ expert_offs, int32_t* __restrict__ dst_sizes,
+                                                             int32_t* __restrict__ dst_offsets, int32_t* __restrict__ caps) {
+    __shared__ int32_t es[MOE_MAX_EXPERTS + 1];
+    __shared__ int32_t s_counts[MOE_MAX_EXPERTS];
+    const int wave = threadIdx.x / WAVE, nw = blockDim.x / WAVE;
+    for (int e = wave; e < E; e += nw) {
+        int running = 0;
+        for (int c = 0; c < NB; c += WAVE) {
+            const int b = c + lane_id();
+            const int v = b < NB ? hist[(size_t)e * NB + b] : 0;
+            const int inc = wave_incl_scan(v);
+            if (b < NB) base[(size_t)e * NB + b] = running + inc - v;
+            running += __shfl(inc, WAVE - 1, WAVE);
+        }
+        if (lane_id() == 0) { counts[e] = running; s_counts[e] = running; }
+    }
+    __syncthreads();
+    if (wave == 0) offsets_body(s_counts, E, W, es, expert_start, send_counts, expert_offs, dst_sizes, dst_offsets, caps);
+}
+
 // ---- 4. stable positions: one wave per 64-token block ----------------------------------------------
 // One wave ranks the slots of token block b: the rank of a slot among the block's slots of the same expert is the
 // number of lower lanes that hold that expert (a token holds an expert at most once), read off a 64-bit lane
@@ -740,8 +766,13 @@ extern "C" int moe_count_and_offsets(const int32_t* topk_idx, int T, int k, int 
         return moe_check_launch("count_and_offsets");
     }
     block_hist_kernel<<<ceil_div(NB, 4), 256, 4 * E * sizeof(int32_t), s>>>(topk_idx, hist, T, k, E, NB);
-    scan_blocks_kernel<<<E, WAVE, 0, s>>>(hist, base, counts, NB);
-    offsets_kernel<<<1, WAVE, 0, s>>>(counts, E, W, expert_start, send_counts, expert_offs, dst_sizes, dst_offsets, caps);
+    if ((long long)E * NB <= SCAN1_MAXCELLS) {
+        scan_offsets_kernel<<<1, 1024, 0, s>>>(hist, base, counts, NB, E, W, expert_start, send_counts, expert_offs, dst_sizes,
+                                               dst_offsets, caps);
+    } else {
+        scan_blocks_kernel<<<E, WAVE, 0, s>>>(hist, base, counts, NB);
+        offsets_kernel<<<1, WAVE, 0, s>>>(counts, E, W, expert_start, send_counts, expert_offs, dst_sizes, dst_offsets, caps);
+    }
     if (T > 0) rank_kernel<<<ceil_div(NB, 4), 256, 0, s>>>(topk_idx, base, expert_start, pos, row_token, T, k, E, NB);
     return moe_check_launch("count_and_offsets");
 }
