@@ -371,7 +371,11 @@ int launch_logits(const XT* x, const XT* w, float* part, int T, int H, int E, hi
         if (E <= 4) RT_LAUNCH(4, 2, 1, 1, CPR, 1);
         else if (E <= 8) RT_LAUNCH(4, 2, 1, 2, CPR, 1);
         else if (E <= 16) RT_LAUNCH(4, 2, 1, 4, CPR, 1);
-        else if (E <= 64) RT_LAUNCH(16, 2, 1, 4, CPR, 1);
+        else if (E <= 64) {
+            // (fp32 tokens: two token blocks per wave do not fit the registers at this shape -- 18 would be spilled)
+            if constexpr (sizeof(XT) == 4) RT_LAUNCH(16, 1, 1, 4, CPR, 1);
+            else RT_LAUNCH(16, 2, 1, 4, CPR, 1);
+        }
         else RT_LAUNCH(16, 2, 1, 8, CPR, ceil_div(E, 128));
     }
 #undef RT_LAUNCH

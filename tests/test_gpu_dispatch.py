@@ -119,6 +119,26 @@ def test_route_logits_rounding_matches_fmaf_chain(kind, E):
     assert_bits_equal(idx, o_idx, f"top-k ({kind})")
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("E", [3, 8, 16, 40, 130])
+def test_route_block_shapes_for_many_tokens(E, dtype):
+    """More than 2048 tokens take the block shapes with two token blocks per wave (one for fp32 tokens at 17 to 64
+    experts), one per range of E: each of them, in both token dtypes, with a row length that is no multiple of the
+    segment length, bit-exact against the oracle."""
+    T, H, k = 2500, 200, min(3, E)
+    g = torch.Generator().manual_seed(E)
+    x = torch.randn(T, H, generator=g)
+    w = torch.randn(H, E, generator=g) * H ** -0.5
+    b = torch.randn(E, generator=g)
+    if dtype == "bf16":
+        x, w = x.bfloat16(), w.bfloat16()
+    idx, gate, logits = ops.route_topk(x.to(DEV), w.to(DEV).contiguous(), k, b.to(DEV))
+    o_idx, o_gate, o_logits = O.route(to_np(x), to_np(w), k, b.numpy())
+    assert_bits_equal(logits, o_logits, f"logits E={E} {dtype}")
+    assert_bits_equal(idx, o_idx, f"top-k E={E} {dtype}")
+    np.testing.assert_allclose(to_np(gate), o_gate, rtol=1e-5, atol=1e-30)
+
+
 @pytest.mark.parametrize("E,k,W", [(8, 8, 4), (512, 16, 64), (6, 1, 3), (60, 7, 1)])
 def test_route_edge_shapes(E, k, W):
     T, H = 77, 72
