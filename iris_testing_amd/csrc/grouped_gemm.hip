@@ -1503,8 +1503,9 @@ int launch_gemm(const GemmParams& p_in, int epi, hipStream_t s, void* part_ws = 
     } while (0)
     switch (epi) {
         case EPI_NONE: GG_EPI(EPI_NONE); break;
-        case EPI_GELU: GG_EPI(EPI_GELU); break;
-        case EPI_SILU: GG_EPI(EPI_SILU); break;
+        // (no fp8 entry point asks for these two: not instantiated)
+        case EPI_GELU: if constexpr (FP8) return moe_fail(MOE_ERR_UNSUPPORTED, "grouped_gemm: fp8 with activation %d", epi); else GG_EPI(EPI_GELU); break;
+        case EPI_SILU: if constexpr (FP8) return moe_fail(MOE_ERR_UNSUPPORTED, "grouped_gemm: fp8 with activation %d", epi); else GG_EPI(EPI_SILU); break;
         case EPI_SWIGLU: GG_EPI(EPI_SWIGLU); break;
         default: return moe_fail(MOE_ERR_INVALID, "grouped_gemm: activation %d", epi);
     }
