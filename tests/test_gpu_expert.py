@@ -300,7 +300,7 @@ def test_copy_free_destination_equals_operator_chain(W, E_l, M, H, F, fill):
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
 
 
-@pytest.mark.parametrize("R,C", [(5, 64), (300, 2048), (77, 1408)])
+@pytest.mark.parametrize("R,C", [(5, 64), (300, 2048), (77, 1408), (40, 4096), (33, 7168), (9, 16384)])  # every register-held row length and the streamed one
 def test_quantize_rows_fp8_bit_exact(R, C):
     rng = np.random.default_rng(R)
     x = _randn(rng, R, C, scale=3.0)
