@@ -415,3 +415,32 @@ def test_pack_tokens_fp8_drops_what_the_bf16_pack_drops():
     assert_bits_equal(q, want_q, "fp8 send codes (overflow)")
     assert_bits_equal(sc, want_s, "fp8 send scales (overflow)")
     assert int(status.item()) == 1
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("k", [3, 7, 16])
+def test_pack_and_combine_at_other_top_k(k, dtype):
+    """top-k values without a compiled-in variant (the kernels then loop over a run-time k): pack, both ways, and
+    combine, bit-exact against the oracle."""
+    rng = np.random.default_rng(k)
+    T, H, E, W = 130, 72, 48, 4
+    E_l = E // W
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    if dtype == "bf16":
+        x = O.bf16_round(x)
+    idx = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+    gate = rng.random((T, k)).astype(np.float32)
+    counts = O.send_counts(idx, W, E)
+    sizes, offs = O.dst_sizes_offsets(counts)
+    pos, row_token = O.payload_positions(idx, E)
+    M = O.pair_capacity(sizes) + 1
+    tdt = torch.float32 if dtype == "f32" else torch.bfloat16
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(DEV)  # noqa: E731
+    xt = torch.from_numpy(x).to(tdt).to(DEV)
+    want = O.pack_fixed_m(O.send_payload(x, row_token), offs, sizes, M)
+    send = ops.pack_tokens(xt, dev(idx), dev(pos), dev(sizes), dev(offs), E_l, M)
+    assert_bits_equal(send, want, "send (token-major pack)")
+    assert_bits_equal(ops.pack_fixed_m(xt, dev(row_token), dev(sizes), dev(offs), M), want, "send (slot-major pack)")
+    ret = O.bf16_round(rng.standard_normal((W, M, H)).astype(np.float32)) if dtype == "bf16" else rng.standard_normal((W, M, H)).astype(np.float32)
+    out = ops.combine(torch.from_numpy(ret).to(tdt).to(DEV), dev(idx), dev(pos), dev(gate), dev(offs), E_l)
+    assert_bits_equal(out, O.combine(ret, idx, pos, gate, offs, E_l, dtype), "combine")
