@@ -55,7 +55,7 @@ const char* moe_last_error(void);
  * order.  Selection on the logits, descending, ties to the lower expert id; topk_gate = softmax
  * probability of each selected expert (not renormalised).  x [T,H], router [H,E] in `dtype`; bias fp32
  * [E] or NULL.  logits: fp32 [T,E] output (the raw logits).  ws: moe_route_workspace_bytes(T,E) bytes of
- * scratch (the segments' partial sums). */
+ * scratch (the segments' partial sums).   ws and logits must be 16-byte aligned. */
 #define MOE_ROUTE_SEGMENTS 8
 size_t moe_route_workspace_bytes(int T, int E);
 int moe_route_topk(const void* x, const void* router, const float* bias, int dtype, int T, int H, int E,

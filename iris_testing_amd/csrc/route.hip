@@ -265,8 +265,9 @@ __global__ __launch_bounds__(NWV * WAVE, (NWV == 4 && TB == 2 ? 2 : 1)) void rou
     }
 }
 
-// Softmax gates + top-k.  G lanes cooperate on one token (G = 8,16,32,64); lane gl holds experts
-// gl, gl+G, gl+2G, ...  Selection key: (logit descending, expert id ascending).
+// Softmax gates + top-k.  G lanes cooperate on one token (G = 8,16,32,64); lane gl holds the eight consecutive experts
+// 8 gl .. 8 gl + 7 (two 16-byte loads per segment plane when the rows are 16-byte multiples).  Selection key: (logit
+// descending, expert id ascending).
 constexpr int TK_MAXV = 8;  // values per lane -> E <= 8*G
 
 template <int G>
@@ -285,23 +286,48 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict_
         const int t = tbase + lane / G;
         const bool live = t < T;
         float v[TK_MAXV];
+        const int e0 = gl * TK_MAXV;
+        const bool vec = (E & 3) == 0;  // every row of the planes starts at a multiple of 16 bytes (and e0 is a multiple of 8)
 #pragma unroll
-        for (int i = 0; i < TK_MAXV; ++i) {
-            const int e = gl + i * G;
-            v[i] = NEG_INF;
-            if (live && e < E) {
+        for (int h = 0; h < TK_MAXV / 4; ++h) {
+            const int eh = e0 + 4 * h;
+            float sum[4] = {NEG_INF, NEG_INF, NEG_INF, NEG_INF};
+            if (live && eh < E) {
                 // the segments' partial sums in segment order, then the bias: this fixes the logit's bits
-                const float* pp = part + (size_t)t * E + e;
-                float s[RT_P];
+                const float* pp = part + (size_t)t * E + eh;
+                if (vec) {  // (eh + 3 < E then)
+                    float4 sp[RT_P];
 #pragma unroll
-                for (int p = 0; p < RT_P; ++p) s[p] = pp[(size_t)p * T * E];
-                float sum = s[0];
+                    for (int p = 0; p < RT_P; ++p) sp[p] = *reinterpret_cast<const float4*>(pp + (size_t)p * T * E);
+                    sum[0] = sp[0].x; sum[1] = sp[0].y; sum[2] = sp[0].z; sum[3] = sp[0].w;
 #pragma unroll
-                for (int p = 1; p < RT_P; ++p) sum = __fadd_rn(sum, s[p]);
-                if (bias) sum = __fadd_rn(sum, bias[e]);
-                v[i] = sum;
-                logits[(size_t)t * E + e] = sum;
+                    for (int p = 1; p < RT_P; ++p) {
+                        sum[0] = __fadd_rn(sum[0], sp[p].x); sum[1] = __fadd_rn(sum[1], sp[p].y);
+                        sum[2] = __fadd_rn(sum[2], sp[p].z); sum[3] = __fadd_rn(sum[3], sp[p].w);
+                    }
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        if (eh + c < E) {
+                            float a = pp[c];
+#pragma unroll
+                            for (int p = 1; p < RT_P; ++p) a = __fadd_rn(a, pp[(size_t)p * T * E + c]);
+                            sum[c] = a;
+                        }
+                    }
+                }
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    if (eh + c < E && bias) sum[c] = __fadd_rn(sum[c], bias[eh + c]);
+                if (vec) *reinterpret_cast<float4*>(logits + (size_t)t * E + eh) = make_float4(sum[0], sum[1], sum[2], sum[3]);
+                else {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+                        if (eh + c < E) logits[(size_t)t * E + eh + c] = sum[c];
+                }
             }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) v[4 * h + c] = (live && eh + c < E) ? sum[c] : NEG_INF;
         }
         unsigned taken = 0;
         float row_max = 0.f;
@@ -314,7 +340,7 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict_
                 int be = 0x7fffffff;
 #pragma unroll
                 for (int i = 0; i < TK_MAXV; ++i) {
-                    const int e = gl + i * G;
+                    const int e = e0 + i;
                     const bool ok = (e < E) && !((taken >> i) & 1u);
                     // ascending e within the lane: strict > keeps the lower id on ties
                     if (ok && (be == 0x7fffffff || v[i] > bv)) { bv = v[i]; be = e; }
@@ -325,7 +351,7 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict_
                     const int oe = __shfl_xor(be, off, WAVE);
                     if (oe != 0x7fffffff && (be == 0x7fffffff || ov > bv || (ov == bv && oe < be))) { bv = ov; be = oe; }
                 }
-                if (be != 0x7fffffff && (be % G) == gl) taken |= 1u << (be / G);
+                if (be != 0x7fffffff && (be / TK_MAXV) == gl) taken |= 1u << (be % TK_MAXV);
                 sel_v[j] = bv;
                 sel_e[j] = be;
                 if (j == 0) row_max = bv;
@@ -335,7 +361,7 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict_
         float part = 0.f;
 #pragma unroll
         for (int i = 0; i < TK_MAXV; ++i) {
-            const int e = gl + i * G;
+            const int e = e0 + i;
             if (e < E) part += expf(v[i] - row_max);
         }
 #pragma unroll
@@ -402,6 +428,7 @@ extern "C" int moe_route_topk(const void* x, const void* router, const float* bi
     MOE_REQUIRE(x && router && logits && topk_idx && topk_gate && ws, MOE_ERR_INVALID, "route_topk: null pointer");
     MOE_REQUIRE(ws_bytes >= moe_route_workspace_bytes(T, E), MOE_ERR_WORKSPACE, "route_topk: workspace %zu < %zu", ws_bytes,
                 moe_route_workspace_bytes(T, E));
+    MOE_REQUIRE((((uintptr_t)ws | (uintptr_t)logits) & 15) == 0, MOE_ERR_INVALID, "route_topk: ws and logits must be 16-byte aligned");
     float* part = (float*)ws;
     int rc = dtype == MOE_F32 ? launch_logits<float>((const float*)x, (const float*)router, part, T, H, E, s)
                               : launch_logits<bf16_t>((const bf16_t*)x, (const bf16_t*)router, part, T, H, E, s);
