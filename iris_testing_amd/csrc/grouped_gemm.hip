@@ -724,19 +724,24 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             gg_wait<0, 15>();
             __syncthreads();
         }
-        bool ok[TM];
-        bf16_t* crow[TM];
+        // fp8: a lane stores to TWO rows of a row tile (its accumulators change lanes first, below); bf16: to its own
+        constexpr int NR = FP8 ? 2 : 1;
+        bool ok[TM][NR];
+        bf16_t* crow[TM][NR];
         float rs[TM];
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            const int r = rbase_e + i * MT + (lane_e & (MT - 1));
-            ok[i] = r < rv;
-            const size_t grow = (size_t)(row0 + (ok[i] ? r : 0));
             rs[i] = 1.f;
-            if constexpr (FP8) rs[i] = s_row_scale[tpar][r];
-            const int crow_i = p.c_map ? s_crow[tpar][r] : 0;
-            ok[i] = ok[i] && crow_i >= 0;  // a negative map entry: the row has no place in the output
-            crow[i] = C + (p.c_map ? (size_t)max(crow_i, 0) : grow) * p.ldc + (DW ? (size_t)g * p.c_group_stride : (size_t)0);
+            if constexpr (FP8) rs[i] = s_row_scale[tpar][rbase_e + i * MT + (lane_e & (MT - 1))];  // (of the row it computed)
+#pragma unroll
+            for (int h = 0; h < NR; ++h) {
+                const int r = rbase_e + i * MT + (FP8 ? (lane_e & 15) + 16 * h : (lane_e & (MT - 1)));
+                ok[i][h] = r < rv;
+                const size_t grow = (size_t)(row0 + (ok[i][h] ? r : 0));
+                const int crow_i = p.c_map ? s_crow[tpar][r] : 0;
+                ok[i][h] = ok[i][h] && crow_i >= 0;  // a negative map entry: the row has no place in the output
+                crow[i][h] = C + (p.c_map ? (size_t)max(crow_i, 0) : grow) * p.ldc + (DW ? (size_t)g * p.c_group_stride : (size_t)0);
+            }
         }
 #pragma unroll
         for (int o = 0; o < TM * NG; ++o) {
@@ -749,6 +754,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             }
             const int pcol = nt * BN + cbase_e + jg * 32;  // first packed column of the group
             const int colg = EPI == EPI_SWIGLU ? (pcol / 64) * 32 : pcol;  // its first output column
+            [[maybe_unused]] uint4 pk[2];  // fp8: the lane's two 16-byte units of the group, stored after they changed lanes
 #pragma unroll
             for (int u = 0; u < NU; ++u) {
                 // the lane's eight consecutive columns: two runs of four accumulators (bf16: the group's two tiles;
@@ -788,18 +794,20 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                         x[4 * t + e] = v;
                     }
                 }
-                if (ok[i] && col < p.N) {
-                    uint4 o4;
-                    o4.x = gg_pack_bf16(x[0], x[1]);
-                    o4.y = gg_pack_bf16(x[2], x[3]);
-                    o4.z = gg_pack_bf16(x[4], x[5]);
-                    o4.w = gg_pack_bf16(x[6], x[7]);
-                    *(uint4*)(crow[i] + col) = o4;
-                    if constexpr (!FP8 && EPI != EPI_NONE) {
+                uint4 o4;
+                o4.x = gg_pack_bf16(x[0], x[1]);
+                o4.y = gg_pack_bf16(x[2], x[3]);
+                o4.z = gg_pack_bf16(x[4], x[5]);
+                o4.w = gg_pack_bf16(x[6], x[7]);
+                if constexpr (FP8) {
+                    pk[u] = o4;
+                } else if (ok[i][0] && col < p.N) {
+                    *(uint4*)(crow[i][0] + col) = o4;
+                    if constexpr (EPI != EPI_NONE) {
                         if (p.C2) {
                             // same row, in a matrix whose rows are as long (SwiGLU: twice as long, packed column order)
                             constexpr int W2 = EPI == EPI_SWIGLU ? 2 : 1;
-                            bf16_t* r2 = (bf16_t*)p.C2 + (size_t)(crow[i] - C) * W2 + (EPI == EPI_SWIGLU ? pcol + 8 * lsub : col);
+                            bf16_t* r2 = (bf16_t*)p.C2 + (size_t)(crow[i][0] - C) * W2 + (EPI == EPI_SWIGLU ? pcol + 8 * lsub : col);
                             uint4 g4;
                             g4.x = gg_pack_bf16(pre_g[0], pre_g[1]); g4.y = gg_pack_bf16(pre_g[2], pre_g[3]);
                             g4.z = gg_pack_bf16(pre_g[4], pre_g[5]); g4.w = gg_pack_bf16(pre_g[6], pre_g[7]);
@@ -812,6 +820,30 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                             }
                         }
                     }
+                }
+            }
+            if constexpr (FP8) {
+                // A lane holds 16 bytes of each half of its row's 64 (columns 8 lsub .. and 16 + 8 lsub ..) and the lane 16
+                // further the same of the row 16 further.  They trade one half each (v_permlane16_swap: lanes 16-31 and
+                // 48-63 of the first operand against lanes 0-15 and 32-47 of the second), after which the first operand
+                // holds whole 64-byte segments of rows 0-15 of the row tile and the second those of rows 16-31: a store
+                // instruction then covers 16 rows instead of 32 -- the store path's cost follows the number of row
+                // segments per instruction, not the bytes.
+#define GG_SWAP16(a_, b_)                                                          \
+    do {                                                                           \
+        const auto sw_ = __builtin_amdgcn_permlane16_swap((a_), (b_), false, false); \
+        (a_) = sw_[0];                                                             \
+        (b_) = sw_[1];                                                             \
+    } while (0)
+                GG_SWAP16(pk[0].x, pk[1].x);
+                GG_SWAP16(pk[0].y, pk[1].y);
+                GG_SWAP16(pk[0].z, pk[1].z);
+                GG_SWAP16(pk[0].w, pk[1].w);
+#undef GG_SWAP16
+                const int col = colg + 16 * ((lane_e >> 4) & 1) + 8 * lsub;
+                if (col < p.N) {
+                    if (ok[i][0]) *(uint4*)(crow[i][0] + col) = pk[0];
+                    if (ok[i][NR - 1]) *(uint4*)(crow[i][NR - 1] + col) = pk[1];
                 }
             }
             // keep the accumulator read-out of one group from being hoisted over the previous group's stores
