@@ -133,18 +133,31 @@ __device__ __forceinline__ float act_gelu(float x) { return 0.5f * x * (1.0f + e
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 // bf16: one 16x16x32 MFMA; lanes 16q .. 16q+15 hold K elements 8q .. 8q+7 (16 bytes) of rows 0 .. 15 of both operands
+// (Z: the sum starts here -- the MFMA takes a constant zero as its C operand, so no accumulator is cleared beforehand)
+template <bool Z = false>
 __device__ __forceinline__ void mma_bf16_k32(floatx4& acc, const uint4& a, const uint4& b) {
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
+    if constexpr (Z) {
+        const floatx4 z = {0.f, 0.f, 0.f, 0.f};
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), z, 0, 0, 0);
+    } else {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), acc, 0, 0, 0);
+    }
 }
 
 // fp8: one 32x32x64 MFMA on 32 bytes of K per lane and operand (two 16-byte LDS chunks); both operands
 // are split over the lanes and registers in the same way, so every k is multiplied exactly once
 typedef int gg_i32x8 __attribute__((ext_vector_type(8)));
+template <bool Z = false>
 __device__ __forceinline__ void mma_fp8_k64(floatx16& acc, const uint4& a_lo, const uint4& a_hi, const uint4& b_lo, const uint4& b_hi) {
     const gg_i32x8 a = {(int)a_lo.x, (int)a_lo.y, (int)a_lo.z, (int)a_lo.w, (int)a_hi.x, (int)a_hi.y, (int)a_hi.z, (int)a_hi.w};
     const gg_i32x8 b = {(int)b_lo.x, (int)b_lo.y, (int)b_lo.z, (int)b_lo.w, (int)b_hi.x, (int)b_hi.y, (int)b_hi.z, (int)b_hi.w};
     // format selectors 0/0 = fp8 (e4m3) for both operands, no block scales
-    acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc, 0, 0, 0, 0, 0, 0);
+    if constexpr (Z) {
+        const floatx16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, z, 0, 0, 0, 0, 0, 0);
+    } else {
+        acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc, 0, 0, 0, 0, 0, 0);
+    }
 }
 
 __device__ __forceinline__ int seg_of(const int* off, int n, int r) {
@@ -503,13 +516,15 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         const int unit = SPLIT ? __builtin_amdgcn_readfirstlane(cur.unit) : -1;
 
         typedef typename std::conditional<FP8, floatx16, floatx4>::type acc_t;
-        acc_t acc[TM][TN];
+        acc_t acc[TM][TN];  // (not cleared where the MFMAs of the tile's first block start the sums)
+        if constexpr (VARK) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
+                for (int j = 0; j < TN; ++j)
 #pragma unroll
-                for (int v = 0; v < (FP8 ? 16 : 4); ++v) acc[i][j][v] = 0.f;
+                    for (int v = 0; v < (FP8 ? 16 : 4); ++v) acc[i][j][v] = 0.f;
+        }
 
         // ---- One MFMA block per 64-byte stage.  Block s multiplies the fragments of stage s, reads those of
         // stage s+1 (all issued in the first half of the block, so they have landed when the block ends) and
@@ -527,12 +542,12 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         if constexpr (ro_ < TM) NA_[ro_ * CF + rh_] = nfa_[ro_ * MT * CHUNKS + (fpos ^ rh_)];            \
         else NB_[(ro_ - TM) * CF + rh_] = nfb_[(ro_ - TM) * MT * CHUNKS + (fpos ^ rh_)];                 \
     } while (0)
-#define GG_ML(I, FA_, FB_, NA_, NB_, slot)                                                               \
+#define GG_ML(I, FA_, FB_, NA_, NB_, slot, Z_)                                                             \
     do {                                                                                                 \
         if constexpr ((I) < NT) {                                                                        \
             constexpr int pa_ = (I) / TN, pb_ = (I) % TN;                                                \
-            if constexpr (FP8) mma_fp8_k64(acc[pa_][pb_], FB_[2 * pb_], FB_[2 * pb_ + 1], FA_[2 * pa_], FA_[2 * pa_ + 1]); \
-            else mma_bf16_k32(acc[pa_][pb_], FB_[pb_], FA_[pa_]);                                        \
+            if constexpr (FP8) mma_fp8_k64<Z_>(acc[pa_][pb_], FB_[2 * pb_], FB_[2 * pb_ + 1], FA_[2 * pa_], FA_[2 * pa_ + 1]); \
+            else mma_bf16_k32<Z_>(acc[pa_][pb_], FB_[pb_], FA_[pa_]);                                    \
             __builtin_amdgcn_sched_barrier(0);                                                           \
             constexpr int ld_ = (I) >= LFIRST && ((I) - LFIRST) % LSTEP == 0 ? ((I) - LFIRST) / LSTEP : LPS;  /* load behind this MFMA */ \
             if constexpr (ld_ < LPS) GG_LD((ld_ < LPS ? ld_ : 0), ap_, bp_, a_off, slot);                \
@@ -542,14 +557,14 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             __builtin_amdgcn_sched_barrier(0);                                                           \
         }                                                                                                \
     } while (0)
-#define GG_ML8(I, FA_, FB_, NA_, NB_, slot)                                                              \
-    GG_ML((I) + 0, FA_, FB_, NA_, NB_, slot); GG_ML((I) + 1, FA_, FB_, NA_, NB_, slot);                   \
-    GG_ML((I) + 2, FA_, FB_, NA_, NB_, slot); GG_ML((I) + 3, FA_, FB_, NA_, NB_, slot);                   \
-    GG_ML((I) + 4, FA_, FB_, NA_, NB_, slot); GG_ML((I) + 5, FA_, FB_, NA_, NB_, slot);                   \
-    GG_ML((I) + 6, FA_, FB_, NA_, NB_, slot); GG_ML((I) + 7, FA_, FB_, NA_, NB_, slot)
-#define GG_STAGE(FA_, FB_, NA_, NB_, SL, s, last)                                                        \
+#define GG_ML8(I, FA_, FB_, NA_, NB_, slot, Z_)                                                          \
+    GG_ML((I) + 0, FA_, FB_, NA_, NB_, slot, Z_); GG_ML((I) + 1, FA_, FB_, NA_, NB_, slot, Z_);           \
+    GG_ML((I) + 2, FA_, FB_, NA_, NB_, slot, Z_); GG_ML((I) + 3, FA_, FB_, NA_, NB_, slot, Z_);           \
+    GG_ML((I) + 4, FA_, FB_, NA_, NB_, slot, Z_); GG_ML((I) + 5, FA_, FB_, NA_, NB_, slot, Z_);           \
+    GG_ML((I) + 6, FA_, FB_, NA_, NB_, slot, Z_); GG_ML((I) + 7, FA_, FB_, NA_, NB_, slot, Z_)
+#define GG_STAGE(FA_, FB_, NA_, NB_, SL, EVEN_, s, last, Z_)                                                      \
     do {                                                                                                 \
-        if constexpr ((SL) % 2 == 0) {                                                                   \
+        if constexpr (EVEN_) { /* (a block in an even slot) */                                           \
             /* from block nks - 4 on the loads fetch the next tile, if it is at hand; not in a tile's first block: the  \
                row map that the tile's top requested must have landed and been handed over (one block end at least) */ \
             if ((s) == nks - 4 && (s) > 0) {                                                             \
@@ -569,10 +584,10 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         const uint4* nfa_ = fa + (((SL) + 1) & 3) * ASLOT;                                               \
         const uint4* nfb_ = fb + (((SL) + 1) & 3) * BSLOT;                                               \
         __builtin_amdgcn_sched_barrier(0);                                                               \
-        GG_ML8(0, FA_, FB_, NA_, NB_, SL); GG_ML8(8, FA_, FB_, NA_, NB_, SL);                             \
-        GG_ML8(16, FA_, FB_, NA_, NB_, SL); GG_ML8(24, FA_, FB_, NA_, NB_, SL);                           \
-        GG_ML8(32, FA_, FB_, NA_, NB_, SL); GG_ML8(40, FA_, FB_, NA_, NB_, SL);                           \
-        GG_ML8(48, FA_, FB_, NA_, NB_, SL); GG_ML8(56, FA_, FB_, NA_, NB_, SL);                           \
+        GG_ML8(0, FA_, FB_, NA_, NB_, SL, Z_); GG_ML8(8, FA_, FB_, NA_, NB_, SL, Z_);                     \
+        GG_ML8(16, FA_, FB_, NA_, NB_, SL, Z_); GG_ML8(24, FA_, FB_, NA_, NB_, SL, Z_);                   \
+        GG_ML8(32, FA_, FB_, NA_, NB_, SL, Z_); GG_ML8(40, FA_, FB_, NA_, NB_, SL, Z_);                   \
+        GG_ML8(48, FA_, FB_, NA_, NB_, SL, Z_); GG_ML8(56, FA_, FB_, NA_, NB_, SL, Z_);                   \
         if (!(last) || seam) { /* (the last block hands over too when the next tile's stages are behind it) */ \
             gg_wait<2 * LPS, 0>();                                                                       \
             __builtin_amdgcn_s_barrier();                                                                \
@@ -640,18 +655,41 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             }
             // The blocks are written out for the slots 0 .. 3; a tile whose first stage lies in slot 2 (phi = 2: the
             // tiles before it left the ring there) enters at the third.  nk >= 2 and even.
-            int ks = -phi;
-            do {
-                if (ks >= 0) {
-                    GG_STAGE(fA0, fB0, fA1, fB1, 0, ks, false);
-                    GG_STAGE(fA1, fB1, fA0, fB0, 1, ks + 1, ks + 2 >= nks);
+            if constexpr (!VARK) {
+                // The tile's first two blocks are written out apart, with the slot as a run-time value: the MFMAs of the
+                // very first start the sums (constant zero as their C operand), so that no accumulator has to be cleared
+                // between two tiles.  (Not where the stage count varies from tile to tile: the register allocation of
+                // those instantiations does not survive it.)
+                const int phi_s = __builtin_amdgcn_readfirstlane(phi);
+                GG_STAGE(fA0, fB0, fA1, fB1, phi_s, true, 0, false, true);
+                GG_STAGE(fA1, fB1, fA0, fB0, phi_s + 1, false, 1, 2 >= nks, false);
+                int ks = phi_s ? 2 : 0;             // phi = 0: on with the slots 2, 3 (the first half of the loop body is
+                const int kmin = phi_s ? 2 : 4;     // skipped once); phi = 2: with the slots 0, 1
+                while (ks < nks) {
+                    if (ks >= kmin) {
+                        GG_STAGE(fA0, fB0, fA1, fB1, 0, true, ks, false, false);
+                        GG_STAGE(fA1, fB1, fA0, fB0, 1, false, ks + 1, ks + 2 >= nks, false);
+                    }
+                    if (ks + 2 < nks) {
+                        GG_STAGE(fA0, fB0, fA1, fB1, 2, true, ks + 2, false, false);
+                        GG_STAGE(fA1, fB1, fA0, fB0, 3, false, ks + 3, ks + 4 >= nks, false);
+                    }
+                    ks += 4;
                 }
-                if (ks + 2 < nks) {
-                    GG_STAGE(fA0, fB0, fA1, fB1, 2, ks + 2, false);
-                    GG_STAGE(fA1, fB1, fA0, fB0, 3, ks + 3, ks + 4 >= nks);
-                }
-                ks += 4;
-            } while (ks < nks);
+            } else {
+                int ks = -phi;
+                do {
+                    if (ks >= 0) {
+                        GG_STAGE(fA0, fB0, fA1, fB1, 0, true, ks, false, false);
+                        GG_STAGE(fA1, fB1, fA0, fB0, 1, false, ks + 1, ks + 2 >= nks, false);
+                    }
+                    if (ks + 2 < nks) {
+                        GG_STAGE(fA0, fB0, fA1, fB1, 2, true, ks + 2, false, false);
+                        GG_STAGE(fA1, fB1, fA0, fB0, 3, false, ks + 3, ks + 4 >= nks, false);
+                    }
+                    ks += 4;
+                } while (ks < nks);
+            }
         }
 #undef GG_STAGE
 #undef GG_ML8
