@@ -270,6 +270,19 @@ __global__ __launch_bounds__(NWV * WAVE, (NWV == 4 && TB == 2 ? 2 : 1)) void rou
 // descending, expert id ascending).
 constexpr int TK_MAXV = 8;  // values per lane -> E <= 8*G
 
+// The value of the lane `off` away in the butterfly of a reduction over 2 off lanes (off a power of two).  Up to 8 it is
+// a DPP move (xor 1, xor 2, then the mirror images within 8 and within 16 lanes: by then the two halves are uniform, so
+// any lane of the other half will do); beyond that a cross-lane read.
+__device__ __forceinline__ unsigned tk_xchg(int off, unsigned x) {
+    switch (off) {
+        case 1: return (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xF, 0xF, false);   // quad_perm [1,0,3,2]
+        case 2: return (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, false);   // quad_perm [2,3,0,1]
+        case 4: return (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x141, 0xF, 0xF, false);  // row_half_mirror
+        case 8: return (unsigned)__builtin_amdgcn_update_dpp(0, (int)x, 0x140, 0xF, 0xF, false);  // row_mirror
+        default: return (unsigned)__shfl_xor((int)x, off, WAVE);
+    }
+}
+
 template <int G>
 __global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict__ part /*[RT_P][T][E]*/,
                                                          const float* __restrict__ bias, float* __restrict__ logits,
@@ -329,35 +342,53 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict_
 #pragma unroll
             for (int c = 0; c < 4; ++c) v[4 * h + c] = (live && eh + c < E) ? sum[c] : NEG_INF;
         }
-        unsigned taken = 0;
+        // Selection on order-preserving keys: (logit bits mapped to an unsigned that sorts like the float, -0 counted as
+        // +0) in the upper word, ~expert in the lower: the 64-bit maximum is the largest logit and, among equals, the
+        // lowest expert.  A taken or absent entry has key 0, below every logit (-inf maps to 0x007fffff).
+        unsigned kh[TK_MAXV], kl[TK_MAXV];
+#pragma unroll
+        for (int i = 0; i < TK_MAXV; ++i) {
+            const int e = e0 + i;
+            const unsigned u = __float_as_uint(v[i] + 0.f);
+            const bool there = live && e < E;
+            kh[i] = there ? (u ^ (((unsigned)((int)u >> 31)) | 0x80000000u)) : 0u;
+            kl[i] = ~(unsigned)e;
+        }
         float row_max = 0.f;
-        float sel_v[MOE_MAX_TOPK];
-        int sel_e[MOE_MAX_TOPK];
+        float my_v = 0.f;  // lane gl keeps selection gl (and gl + G, ...) for the gate it computes below
+        int my_e = 0;
+        float my_v2 = 0.f;
+        int my_e2 = 0;
 #pragma unroll
         for (int j = 0; j < MOE_MAX_TOPK; ++j) {
             if (j < k) {
-                float bv = NEG_INF;
-                int be = 0x7fffffff;
+                unsigned long long best = 0;
 #pragma unroll
                 for (int i = 0; i < TK_MAXV; ++i) {
-                    const int e = e0 + i;
-                    const bool ok = (e < E) && !((taken >> i) & 1u);
-                    // ascending e within the lane: strict > keeps the lower id on ties
-                    if (ok && (be == 0x7fffffff || v[i] > bv)) { bv = v[i]; be = e; }
+                    const unsigned long long c = ((unsigned long long)kh[i] << 32) | kl[i];
+                    best = c > best ? c : best;
                 }
 #pragma unroll
-                for (int off = G / 2; off >= 1; off >>= 1) {
-                    const float ov = __shfl_xor(bv, off, WAVE);
-                    const int oe = __shfl_xor(be, off, WAVE);
-                    if (oe != 0x7fffffff && (be == 0x7fffffff || ov > bv || (ov == bv && oe < be))) { bv = ov; be = oe; }
+                for (int off = 1; off < G; off <<= 1) {
+                    const unsigned oh = tk_xchg(off, (unsigned)(best >> 32)), ol = tk_xchg(off, (unsigned)best);
+                    const unsigned long long o = ((unsigned long long)oh << 32) | ol;
+                    best = o > best ? o : best;
                 }
-                if (be != 0x7fffffff && (be / TK_MAXV) == gl) taken |= 1u << (be % TK_MAXV);
-                sel_v[j] = bv;
-                sel_e[j] = be;
+                const unsigned bh = (unsigned)(best >> 32);
+                const int be = (int)~(unsigned)best;
+                // (the owner drops it from its candidates)
+#pragma unroll
+                for (int i = 0; i < TK_MAXV; ++i)
+                    if (be == e0 + i) kh[i] = 0u;
+                const float bv = __uint_as_float((bh & 0x80000000u) ? (bh ^ 0x80000000u) : ~bh);
                 if (j == 0) row_max = bv;
+                if ((j % G) == gl) {
+                    if (j < G) { my_v = bv; my_e = be; }
+                    else { my_v2 = bv; my_e2 = be; }
+                }
             }
         }
-        // softmax denominator: per-lane ascending partial sum, then xor butterfly
+        // softmax denominator: per-lane ascending partial sum, then a butterfly over the token's lanes
         float part = 0.f;
 #pragma unroll
         for (int i = 0; i < TK_MAXV; ++i) {
@@ -365,15 +396,15 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict_
             if (e < E) part += expf(v[i] - row_max);
         }
 #pragma unroll
-        for (int off = G / 2; off >= 1; off >>= 1) part += __shfl_xor(part, off, WAVE);
-        if (live && gl == 0) {
-#pragma unroll
-            for (int j = 0; j < MOE_MAX_TOPK; ++j) {
-                if (j < k) {
-                    idx[(size_t)t * k + j] = sel_e[j] == 0x7fffffff ? 0 : sel_e[j];
-                    gate[(size_t)t * k + j] = expf(sel_v[j] - row_max) / part;
-                }
-            }
+        for (int off = 1; off < G; off <<= 1) part += __uint_as_float(tk_xchg(off, __float_as_uint(part)));
+        // lane gl writes selection gl (and gl + G when k > G): one exp and one division per lane instead of k in one lane
+        if (live && gl < k) {
+            idx[(size_t)t * k + gl] = my_e;
+            gate[(size_t)t * k + gl] = expf(my_v - row_max) / part;
+        }
+        if (live && gl + G < k) {
+            idx[(size_t)t * k + gl + G] = my_e2;
+            gate[(size_t)t * k + gl + G] = expf(my_v2 - row_max) / part;
         }
     }
 }
