@@ -545,7 +545,8 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 #define GG_ML(I, FA_, FB_, NA_, NB_, slot, Z_)                                                             \
     do {                                                                                                 \
         if constexpr ((I) < NT) {                                                                        \
-            constexpr int pa_ = (I) / TN, pb_ = (I) % TN;                                                \
+            /* boustrophedon over the wave's MFMA tiles: every instruction keeps one operand of the one before it */ \
+            constexpr int pa_ = (I) / TN, pb_ = (pa_ & 1) ? TN - 1 - (I) % TN : (I) % TN;                \
             if constexpr (FP8) mma_fp8_k64<Z_>(acc[pa_][pb_], FB_[2 * pb_], FB_[2 * pb_ + 1], FA_[2 * pa_], FA_[2 * pa_ + 1]); \
             else mma_bf16_k32<Z_>(acc[pa_][pb_], FB_[pb_], FA_[pa_]);                                    \
             __builtin_amdgcn_sched_barrier(0);                                                           \
