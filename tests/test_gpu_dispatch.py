@@ -92,6 +92,25 @@ def test_route_ties_prefer_lower_expert():
     assert (cls == cls[:, :1]).all() and (np.diff(o_idx, axis=1) == 4).all()
 
 
+def test_route_zeros_of_either_sign_tie():
+    """Products that underflow (1e-30 * +-1e-30) give logits of +0 or -0 by the sign of the router column: they compare
+    equal, so the selection is the k lowest expert ids whatever the signs (the selection keys count -0 as +0), and
+    every gate is 1 / E."""
+    T, H, E, k = 70, 64, 24, 6
+    x = torch.full((T, H), 1e-30)
+    w = torch.full((H, E), 1e-30)
+    w[:, ::3] = -1e-30   # every step of the chain adds -1e-60, which rounds to -0: these experts' logits are -0
+    b = torch.full((E,), -0.0)
+    idx, gate, logits = ops.route_topk(x.to(DEV), w.to(DEV).contiguous(), k, b.to(DEV))
+    o_idx, o_gate, o_logits = O.route(x.numpy(), w.numpy(), k, b.numpy())
+    assert_bits_equal(logits, o_logits, "signed-zero logits")
+    lg = to_np(logits)
+    assert np.signbit(lg[:, ::3]).all() and not np.signbit(lg[:, 1::3]).any(), "the case does not produce both zeros"
+    assert_bits_equal(idx, o_idx, "top-k among zeros")
+    assert (to_np(idx) == np.arange(k)[None, :]).all()
+    np.testing.assert_allclose(to_np(gate), np.full((T, k), 1.0 / E, np.float32), rtol=1e-6)
+
+
 @pytest.mark.parametrize("kind", ["wide", "subnormal", "cancel"])
 @pytest.mark.parametrize("E", [8, 20, 200])
 def test_route_logits_rounding_matches_fmaf_chain(kind, E):
@@ -139,7 +158,7 @@ def test_route_block_shapes_for_many_tokens(E, dtype):
     np.testing.assert_allclose(to_np(gate), o_gate, rtol=1e-5, atol=1e-30)
 
 
-@pytest.mark.parametrize("E,k,W", [(8, 8, 4), (512, 16, 64), (6, 1, 3), (60, 7, 1)])
+@pytest.mark.parametrize("E,k,W", [(8, 8, 4), (512, 16, 64), (6, 1, 3), (60, 7, 1), (40, 12, 4), (16, 16, 2)])  # (the last two: more selections than lanes per token)
 def test_route_edge_shapes(E, k, W):
     T, H = 77, 72
     g = torch.Generator().manual_seed(E * 31 + k)
