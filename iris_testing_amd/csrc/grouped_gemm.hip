@@ -38,7 +38,7 @@ constexpr int GG_BN = 256;
 #define GG_BIG_NWM 2  // waves along M of the 256-row tile (x 2 along N)
 #endif
 #ifndef GG_FP8_NWM
-#define GG_FP8_NWM 4  // fp8: 4 x 2 waves of 64 x 128 each, two per SIMD (measured 1.4 to 3.7 % faster over the fp8 workloads than 2 x 2
+#define GG_FP8_NWM 4  // fp8: 4 x 2 waves of 64 x 128 each, two per SIMD (measured 3.5 to 7 % faster over the fp8 workloads than 2 x 2
                       // waves of 128 x 128; the same shape costs bf16 5 %)
 #endif
 
