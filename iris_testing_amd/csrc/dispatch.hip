@@ -64,7 +64,10 @@ __global__ __launch_bounds__(WAVE) void scan_blocks_kernel(const int32_t* __rest
 }
 
 // ---- 3. expert prefix -> all count/offset outputs (one wave) ---------------------------------------
-// (every wave of the calling block runs this with the same inputs and writes the same values: es is shared)
+// ONE_WAVE = false: every wave of the calling block runs this with the same inputs and writes the same values (es is
+// shared; the barrier inside is a block barrier that all of them reach).  ONE_WAVE = true: a single wave runs it, whatever
+// else the block holds, and the hand-over through es is a wave-local one (no block barrier in divergent control flow).
+template <bool ONE_WAVE>
 __device__ __forceinline__ void offsets_body(const int32_t* counts, int E, int W, int32_t* es /*[E+1], LDS*/,
                                              int32_t* expert_start /*[E+1]*/, int32_t* __restrict__ send_counts,
                                              int32_t* __restrict__ expert_offs, int32_t* __restrict__ dst_sizes,
@@ -80,7 +83,14 @@ __device__ __forceinline__ void offsets_body(const int32_t* counts, int E, int W
     if (lane == WAVE - 1) es[E] = incl;
 #pragma unroll
     for (int off = WAVE / 2; off >= 1; off >>= 1) cmax = max(cmax, __shfl_xor(cmax, off, WAVE));
-    __syncthreads();
+    if constexpr (ONE_WAVE) {
+        // the lanes' LDS writes above are read by other lanes of the same wave below
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    } else {
+        __syncthreads();
+    }
     const int E_l = E / W;
     for (int e = lane; e <= E; e += WAVE) expert_start[e] = es[e];
     for (int e = lane; e < E; e += WAVE) {
@@ -105,7 +115,7 @@ __global__ __launch_bounds__(WAVE) void offsets_kernel(const int32_t* __restrict
                                                         int32_t* __restrict__ dst_sizes, int32_t* __restrict__ dst_offsets,
                                                         int32_t* __restrict__ caps) {
     __shared__ int32_t es[MOE_MAX_EXPERTS + 1];
-    offsets_body(counts, E, W, es, expert_start, send_counts, expert_offs, dst_sizes, dst_offsets, caps);
+    offsets_body<true>(counts, E, W, es, expert_start, send_counts, expert_offs, dst_sizes, dst_offsets, caps);
 }
 
 // Steps 2 and 3 in one launch when the histogram is small enough for one workgroup (every wave scans the experts
@@ -131,7 +141,7 @@ __global__ __launch_bounds__(1024) void scan_offsets_kernel(const int32_t* __res
         if (lane_id() == 0) { counts[e] = running; s_counts[e] = running; }
     }
     __syncthreads();
-    if (wave == 0) offsets_body(s_counts, E, W, es, expert_start, send_counts, expert_offs, dst_sizes, dst_offsets, caps);
+    if (wave == 0) offsets_body<true>(s_counts, E, W, es, expert_start, send_counts, expert_offs, dst_sizes, dst_offsets, caps);
 }
 
 // ---- 4. stable positions: one wave per 64-token block ----------------------------------------------
@@ -211,7 +221,7 @@ __global__ __launch_bounds__(256) void count_small_kernel(const int32_t* __restr
         counts[e] = run;
     }
     __syncthreads();
-    offsets_body(counts, E, W, es, expert_start, send_counts, expert_offs, dst_sizes, dst_offsets, caps);
+    offsets_body<false>(counts, E, W, es, expert_start, send_counts, expert_offs, dst_sizes, dst_offsets, caps);
     __syncthreads();
     for (int b0 = 0; b0 < NB; b0 += 4)  // (uniform trip count: rank_block holds block barriers)
         rank_block(idx, base, expert_start, pos, row_token, T, k, E, NB, b0 + wave, b0 + wave < NB, masks[wave]);
@@ -450,8 +460,9 @@ __global__ __launch_bounds__(WPB * WAVE) void pack_tokens_kernel(const u32x4* __
             drow[j] = -1;
             if (j < k) {
                 const int d = idx[(size_t)r * k + j] / E_l;
-                const int m = pos[(size_t)r * k + j] - dst_offsets[d];
-                if ((unsigned)d < (unsigned)W && (unsigned)m < (unsigned)M) drow[j] = d * M + m;
+                const bool d_ok = (unsigned)d < (unsigned)W;  // (an expert id outside [0, W E_l): no slot, and no read of its offset)
+                const int m = pos[(size_t)r * k + j] - dst_offsets[d_ok ? d : 0];
+                if (d_ok && (unsigned)m < (unsigned)M) drow[j] = d * M + m;
             }
         }
         const u32x4* src = x + (size_t)r * row_vec;

@@ -400,6 +400,9 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                 ts += c > 0 ? ((p.dw_rows + BM - 1) / BM) * Nt : 0;
                 rs += ((c + 63) / 64) * 2;
             } else {
+                // (counts that claim more rows than the buffers hold are cut at S_rows: the host's bound on the number of
+                // tiles, which decides whether the whole-tile launch is left out, counts on it)
+                c = min(c, max(p.S_rows - rs, 0));
                 ts += ((c + BM - 1) / BM) * Nt;
                 rs += c;
             }
@@ -920,7 +923,7 @@ __global__ __launch_bounds__(256) void gg_reduce_parts_kernel(const GemmParams p
         for (int g = 0; g < p.E_l; ++g) {
             g_tile_start[g] = ts;
             g_row_start[g] = rs;
-            const int c = max(p.cnt[g], 0);
+            const int c = min(max(p.cnt[g], 0), max(p.S_rows - rs, 0));  // (clamped like the GEMM launch clamps it)
             ts += ((c + BM - 1) / BM) * Nt;
             rs += c;
         }

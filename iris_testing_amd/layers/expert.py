@@ -125,17 +125,37 @@ class ExpertWeights:
     # the tensors prepare() was given, in the reference layout: (w1, w2, w_up); the backward pass differentiates with
     # respect to them and re-tiles their transposes on first use
     raw: Optional[tuple] = field(default=None, repr=False)
+    # version counters of the raw tensors when w1 / w2 / w_up were last derived from them (refresh() compares)
+    raw_versions: Optional[tuple] = field(default=None, repr=False)
+
+    @staticmethod
+    def _derive(raw):
+        """(w1, w2, w_up) as the kernels take them, from the tensors in the reference layout."""
+        w1, w2, w_up = raw
+        if w1.dtype == torch.float32:
+            return w1.contiguous(), w2.contiguous(), None if w_up is None else w_up.contiguous()
+        return (ops.prepack_weights(w1.contiguous(), None if w_up is None else w_up.contiguous()),
+                ops.prepack_weights(w2.contiguous()), None)
+
+    @staticmethod
+    def _versions(raw):
+        return tuple(None if t is None else t._version for t in raw)
 
     @classmethod
     def prepare(cls, act: str, w1: torch.Tensor, w2: torch.Tensor, w_up: Optional[torch.Tensor] = None):
         e_l, H, F = w1.shape
         raw = (w1, w2, w_up)
-        if w1.dtype == torch.float32:
-            return cls(act, H, F, e_l, w1.dtype, w1.contiguous(), w2.contiguous(),
-                       None if w_up is None else w_up.contiguous(), raw=raw)
-        p1 = ops.prepack_weights(w1.contiguous(), None if w_up is None else w_up.contiguous())
-        p2 = ops.prepack_weights(w2.contiguous())
-        return cls(act, H, F, e_l, w1.dtype, p1, p2, raw=raw)
+        p1, p2, pu = cls._derive(raw)
+        return cls(act, H, F, e_l, w1.dtype, p1, p2, pu, raw=raw, raw_versions=cls._versions(raw))
+
+    def refresh(self) -> "ExpertWeights":
+        """Derive the kernels' copies again if a tensor prepare() was given has been updated in place since (an optimizer
+        step): the forward pass would otherwise multiply with the weights of before the update while the backward pass,
+        which re-tiles the transposes by tensor version, uses the new ones."""
+        if self.raw is not None and self._versions(self.raw) != self.raw_versions:
+            self.w1, self.w2, self.w_up = self._derive(self.raw)
+            self.raw_versions = self._versions(self.raw)
+        return self
 
     @classmethod
     def prepare_fp8(cls, wg_q, sg, wu_q, su, wd_q, sd):
@@ -217,7 +237,7 @@ def expert_mlp(tokens: torch.Tensor, weights: ExpertWeights, local_expert_cnt: t
     if weights.dtype == torch.uint8:
         sg, su, sd = weights.scales
         return ops.grouped_mlp_fp8(tokens.contiguous(), local_expert_cnt, weights.ffn, weights.w1, sg, su, weights.w2, sd)
-    raw = weights.raw
+    raw = weights.refresh().raw
     if torch.is_grad_enabled() and raw is not None and (tokens.requires_grad or any(t is not None and t.requires_grad for t in raw)):
         return ExpertMLP.apply(tokens, local_expert_cnt.contiguous(), weights, raw[0], raw[1], raw[2])
     return ops.grouped_mlp(tokens.contiguous(), local_expert_cnt, weights.act, weights.w1, weights.w2, weights.w_up,

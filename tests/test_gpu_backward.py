@@ -138,3 +138,49 @@ def test_combine_and_pack_gradients_match_float64_autograd():
         send.backward(gs.to(DEV))
         want = gs.double().view(W * M, H)[slot].sum(1)
         assert _rel(xd.grad, want) < tol
+
+
+def test_expert_mlp_follows_in_place_weight_updates():
+    """An optimizer step updates the raw weights in place between two calls: the second forward must multiply with the
+    updated weights (the kernels' re-tiled copies are derived again), and its gradients must be those of the updated ones."""
+    rng = np.random.default_rng(11)
+    H, F, cnt = 128, 256, np.array([90, 0, 37], dtype=np.int32)
+    E_l, S = len(cnt), int(cnt.sum())
+    mk = lambda *s, sc=1.0: torch.from_numpy((rng.standard_normal(s) * sc).astype(np.float32)).bfloat16()  # noqa: E731
+    x, w1, wu, w2 = mk(S, H), mk(E_l, H, F, sc=H ** -0.5), mk(E_l, H, F, sc=H ** -0.5), mk(E_l, F, H, sc=F ** -0.5)
+    step1, step2 = mk(E_l, H, F, sc=0.5 * H ** -0.5), mk(E_l, F, H, sc=0.5 * F ** -0.5)
+    g = mk(S, H)
+    xd = x.to(DEV).requires_grad_(True)
+    w1d, wud, w2d = (t.to(DEV).requires_grad_(True) for t in (w1, wu, w2))
+    ew = ExpertWeights.prepare("swiglu", w1d, w2d, wud)
+    cnt_d = torch.from_numpy(cnt).to(DEV)
+
+    def ref64(w1_, wu_, w2_):
+        leaves = [t.double().requires_grad_(True) for t in (x, w1_, wu_, w2_)]
+        x64, a, u, d = leaves
+        parts, r = [], 0
+        for e, c in enumerate(cnt):
+            xe = x64[r:r + c]
+            parts.append((torch.nn.functional.silu(xe @ a[e]) * (xe @ u[e])) @ d[e])
+            r += c
+        out = torch.cat(parts)
+        out.backward(g.double())
+        return out.detach(), [t.grad for t in leaves]
+
+    out0 = expert_mlp(xd, ew, cnt_d)
+    want0, _ = ref64(w1, wu, w2)
+    assert _rel(out0, want0) < 2.0 ** -6
+    with torch.no_grad():  # the in-place update (bumps the tensors' version counters)
+        w1d.add_(step1.to(DEV))
+        w2d.sub_(step2.to(DEV))
+    out1 = expert_mlp(xd, ew, cnt_d)
+    out1.backward(g.to(DEV))
+    w1n, w2n = (w1.float() + step1.float()).bfloat16(), (w2.float() - step2.float()).bfloat16()
+    want1, grads = ref64(w1n, wu, w2n)
+    assert _rel(out1, want1) < 2.0 ** -6, "the forward pass used the weights of before the update"
+    assert _rel(out1, want0) > 2.0 ** -4, "the update must be large enough to tell the two apart"
+    for name, got, want in zip(("d tokens", "d w1", "d w_up", "d w2"), (xd.grad, w1d.grad, wud.grad, w2d.grad), grads):
+        assert _rel(got, want) < 2.0 ** -5, name
+    # inference path (no autograd) sees the update too
+    with torch.no_grad():
+        assert _rel(expert_mlp(xd, ew, cnt_d), want1) < 2.0 ** -6

@@ -285,6 +285,16 @@ def test_overflowed_pack_drops_rows_consistently_down_the_path():
     o_bad = s0["idx"].copy()
     o_bad[3, 1] = E + 5 * E_l
     assert_bits_equal(out, O.combine(o_send0 * 2, o_bad, s0["pos"], s0["gate"], s0["offs"], E_l, cfg.dtype), "combine, bad id")
+    # ... and by the token-major pack: the slot of the bad id stays as it was (its offset is never read), all others are written
+    t_bad, m_bad = 3, int(s0["pos"][3, 1] - s0["offs"][s0["idx"][3, 1] // E_l])
+    guard = torch.full((W * M + 8, H), 7.0, dtype=cfg.torch_dtype, device=DEV)
+    ops.pack_tokens(x0, bad_idx, pos0, sizes0, offs0, E_l, M, out=guard[:W * M].view(W, M, H))
+    want = o_send0.copy()
+    d_bad = int(s0["idx"][t_bad, 1]) // E_l
+    if m_bad < M:
+        want[d_bad, m_bad] = 7.0
+    assert_bits_equal(guard[:W * M].view(W, M, H), want, "token-major pack, bad id")
+    assert (guard[W * M:] == 7.0).all()
 
 
 UNPACK_CASES = [("plumbing", None), ("small", None), ("mixtral", 1024), ("finegrained", 512), ("zipf_k4", 1024)]
