@@ -2,6 +2,7 @@
 """Routed tokens/s through the MoE dispatch + expert + combine hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config mixtral] [--no-cpu-baseline]
+                    [--unfused | --gated | --padding-free] [--backward] [--stream-ceiling]
 
 A "step" is one pass of rank 0's share of the path over one batch of synthetic tokens (see
 iris_testing_amd/pipeline.py): route + count + pack as a source, unpack + grouped expert MLP + return
@@ -22,41 +23,61 @@ sys.path.insert(0, ROOT)
 PEAK = {"hbm": 8000.0, "mfma_bf16": 2500.0, "mfma_fp8": 5000.0, "fp32": 157.3}  # GB/s, TFLOP/s
 
 
-def cpu_baseline(cfg, world_np, budget_tokens: int):
-    """The CPU oracle timed on a bounded sample of the same workload: the first `budget_tokens`
-    tokens of shard 0 through route + count + pack, their routed rows through rank 0's expert MLP,
-    and the combine.  Returns (tokens/s, seconds, threads, description)."""
+def cpu_baseline(cfg, router, bias, weights, budget_tokens: int):
+    """The CPU oracle timed on the same step as the GPU leg, on a bounded sample of the same workload: the simulated
+    world made of the first ``budget_tokens`` tokens of EVERY source shard (the whole workload when the budget covers
+    it).  Untimed, as on the GPU: routing and packing the other shards to assemble rank 0's receive buffer and its
+    real, skewed recv_counts.  Timed: rank 0 as a source (route + count + pack), as a destination (expert-major unpack
+    of what it received, grouped expert MLP over the real per-expert row counts, return pack), as a source again
+    (combine).  Returns (tokens/s, seconds, threads, description)."""
     import numpy as np
+    from iris_testing_amd.configs import gen_shard_tokens
     from oracle import moe_oracle as O
 
-    x, router, bias, weights = world_np
-    Ts = min(budget_tokens, x.shape[0])
-    xs = x[:Ts]
+    W, E, E_l, k = cfg.world, cfg.experts, cfg.e_local, cfg.topk
+    Ts = min(budget_tokens, cfg.tokens)
+    f32 = lambda t: t.float().numpy() if t.dtype != __import__("torch").float32 else t.numpy()  # noqa: E731
+    xs = [f32(gen_shard_tokens(cfg, s)[:Ts]) for s in range(W)]
+
+    def source_side(x):
+        idx, gate, _ = O.route(x, router, k, bias)
+        counts = O.send_counts(idx, W, E)
+        sizes, offs = O.dst_sizes_offsets(counts)
+        pos, row_token = O.payload_positions(idx, E)
+        return idx, gate, counts, sizes, offs, pos, O.send_payload(x, row_token)
+
+    # ---- untimed: what the other ranks send to rank 0
+    others = [source_side(x) for x in xs]
+    M = O.pair_capacity(np.stack([o[3] for o in others]))
+    recv = np.stack([O.pack_fixed_m(o[6], o[4], o[3], M)[0] for o in others])
+    rc = np.stack([o[2][0] for o in others]).astype(np.int32)
+    S = int(rc.sum())
+    rng = np.random.default_rng(cfg.seed + 4242)
+    returned = O.round_to(rng.standard_normal((W, M, cfg.hidden)).astype(np.float32), cfg.dtype)
+    del others
+
+    # ---- timed: one step of rank 0
     t0 = time.perf_counter()
-    idx, gate, _ = O.route(xs, router, cfg.topk, bias)
-    counts = O.send_counts(idx, cfg.world, cfg.experts)
-    sizes, offs = O.dst_sizes_offsets(counts)
-    pos, row_token = O.payload_positions(idx, cfg.experts)
-    payload = O.send_payload(xs, row_token)
-    M = O.pair_capacity(sizes)
+    idx, gate, counts, sizes, offs, pos, payload = source_side(xs[0])
+    assert O.pair_capacity(sizes) <= M
     send = O.pack_fixed_m(payload, offs, sizes, M)
-    # destination side on the same number of routed rows: all rows through the local experts of rank 0,
-    # spread over them in proportion (the sample keeps rows-per-token = k)
-    rows = payload
-    E_l = cfg.e_local
-    cnt = np.full(E_l, rows.shape[0] // E_l, np.int32)
-    cnt[: rows.shape[0] - int(cnt.sum())] += 1
+    rows = O.unpack_expert_major(recv, rc)
+    cnt = O.expert_row_counts(rc.T)
     if cfg.quant == "fp8":
         y = O.expert_mlp_fp8(rows, cnt, *weights)
     elif cfg.act == "swiglu":
         y = O.expert_mlp(rows, cnt, weights[0], weights[2], "swiglu", cfg.dtype, w_up=weights[1])
     else:
         y = O.expert_mlp(rows, cnt, weights[0], weights[1], cfg.act, cfg.dtype)
-    ret = O.pack_fixed_m(y, offs, sizes, M)
-    out = O.combine(ret, idx, pos, gate, offs, E_l, cfg.dtype)
+    ret = O.return_pack(y, rc, M)
+    returned[0] = ret[0]
+    out = O.combine(returned, idx, pos, gate, offs, E_l, cfg.dtype)
     dt = time.perf_counter() - t0
-    assert out.shape == xs.shape and send.shape[1] == M
-    return Ts / dt, dt, blas_threads(), f"first {Ts} tokens of shard 0 ({rows.shape[0]} routed rows), all stages, numpy/C oracle"
+    assert out.shape == xs[0].shape and send.shape == (W, M, cfg.hidden) and rows.shape[0] == S
+    whole = "the whole workload" if Ts == cfg.tokens else f"the first {Ts} of {cfg.tokens} tokens of every source shard"
+    return Ts / dt, dt, blas_threads(), (f"{whole}: rank 0 routes and packs {Ts} tokens, runs its {E_l} local experts on the "
+                                         f"{S} rows it receives (real per-expert counts, {int(cnt.min())}..{int(cnt.max())}), "
+                                         f"returns them and combines; numpy/C oracle")
 
 
 def blas_threads() -> int:
@@ -103,6 +124,140 @@ def profiled_traffic(workload: str, stage: str):
     return None, None
 
 
+def _timed(fn, n, torch):
+    """Average milliseconds of n calls of fn on the current stream (one untimed call first)."""
+    fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(n):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / n
+
+
+def backward_leg(cfg, world, raw, steps):
+    """Forward and backward of rank 0's expert MLP at the workload's shape (the S rows it receives, its real per-expert
+    counts), through the autograd operators of the host layer: gradients with respect to the rows and to every weight
+    matrix.  bf16 / fp32 experts only.  Flops: forward 2 S H F n_mat, backward twice that (one product for the
+    gradient of the input and one for the gradient of the weights per forward product)."""
+    import torch
+    from iris_testing_amd import ops
+    from iris_testing_amd.layers import ExpertWeights, expert_mlp
+    from iris_testing_amd.layers.expert import _packed_weights_t, _part_ws
+    dev = world.recv.device
+    S, H, F = world.S, cfg.hidden, cfg.ffn
+    rows, cnt = ops.unpack_expert_major(world.recv, world.recv_counts, S)
+    rows.requires_grad_(True)
+    ws = [w.to(dev).requires_grad_(True) for w in raw]
+    ew = ExpertWeights.prepare(cfg.act, ws[0], ws[2], ws[1]) if cfg.act == "swiglu" else ExpertWeights.prepare(cfg.act, ws[0], ws[1])
+    gy = torch.randn((S, H), generator=torch.Generator(device="cpu").manual_seed(cfg.seed + 77), dtype=torch.float32).to(cfg.torch_dtype).to(dev)
+
+    def fwd():
+        with torch.no_grad():
+            expert_mlp(rows, ew, cnt)
+
+    def fwd_bwd():
+        rows.grad = None
+        for w in ws:
+            w.grad = None
+        expert_mlp(rows, ew, cnt).backward(gy)
+
+    f_ms = _timed(fwd, steps, torch)
+    fb_ms = _timed(fwd_bwd, steps, torch)
+    # the forward inside fwd_bwd also keeps the pre-activations (one more store per value): time it on its own
+    def fwd_keep():
+        expert_mlp(rows, ew, cnt)
+    fk_ms = _timed(fwd_keep, steps, torch)
+    b_ms = fb_ms - fk_ms
+    fl_f = 2 * S * H * F * cfg.n_mat
+    peak = PEAK["fp32"] if cfg.dtype == "f32" else PEAK["mfma_bf16"]
+    # the pieces of the backward pass one by one (same calls as ExpertMLP.backward makes)
+    pieces = {}
+    if cfg.dtype == "bf16":
+        swiglu = cfg.act == "swiglu"
+        NP = 2 * F if swiglu else F
+        pws = _part_ws(dev)
+        with torch.no_grad():
+            hidden = torch.empty((S, F), dtype=rows.dtype, device=dev)
+            a1 = torch.empty((S, NP), dtype=rows.dtype, device=dev)
+            ops.grouped_gemm_act_keep(rows, ew.w1, cnt, S, F, ew.act, hidden, a1, part_ws=pws)
+            dh = torch.zeros((S, F), dtype=rows.dtype, device=dev)
+            dx = torch.zeros((S, H), dtype=rows.dtype, device=dev)
+            w1r, w2r, wur = ew.raw
+            w2t, w1t = _packed_weights_t(w2r), _packed_weights_t(w1r, wur)
+            da1 = ops.mlp_act_backward(a1, dh, ew.act)
+            pieces["d_hidden = dy @ W2^T"] = (_timed(lambda: ops.grouped_gemm_mapped(gy, None, w2t, cnt, S, F, "none", dh, part_ws=pws), steps, torch), 2 * S * H * F)
+            pieces["d_W2 = hidden^T @ dy (ragged K)"] = (_timed(lambda: ops.grouped_gemm_dw(hidden, gy, cnt), steps, torch), 2 * S * H * F)
+            pieces["activation gradient"] = (_timed(lambda: ops.mlp_act_backward(a1, dh, ew.act), steps, torch), 0)
+            pieces["d_x = d_a1 @ W1^T"] = (_timed(lambda: ops.grouped_gemm_mapped(da1, None, w1t, cnt, S, H, "none", dx, part_ws=pws), steps, torch), 2 * S * H * NP)
+            pieces["d_W1 = x^T @ d_a1 (ragged K)"] = (_timed(lambda: ops.grouped_gemm_dw(rows, da1, cnt, split_F=F if swiglu else 0), steps, torch), 2 * S * H * NP)
+    return {
+        "what": "expert MLP of rank 0 on the rows it receives: forward, then gradients of the rows and of every weight matrix",
+        "rows": S, "forward_ms": round(f_ms, 4), "forward_keeping_preactivations_ms": round(fk_ms, 4),
+        "backward_ms": round(b_ms, 4), "backward_over_forward": round(b_ms / f_ms, 3),
+        "forward_tflops": round(fl_f / f_ms / 1e9, 1), "backward_tflops": round(2 * fl_f / b_ms / 1e9, 1),
+        "backward_frac_of_peak": round(2 * fl_f / b_ms / 1e9 / peak, 4), "peak_tflops": peak,
+        "pieces": {n: {"ms": round(ms, 4), **({"tflops": round(fl / ms / 1e9, 1), "frac": round(fl / ms / 1e9 / peak, 4)} if fl else {})}
+                   for n, (ms, fl) in pieces.items()},
+    }
+
+
+def stream_ceiling_leg(cfg, steps):
+    """What the memory system sustains for the three traffic mixes of the row-moving stages, measured with the product's own
+    kernels on buffers of 1 GiB: a plain row copy (moe_pack_payload with the identity map: one byte read per byte written),
+    a pure write (moe_zero_padding_rows over a buffer that is all padding) and read-mostly sums (moe_combine with unit gates
+    and k rows read per row written).  From the first two, the read rate R and write rate W of the model
+    time = read bytes / R + written bytes / W."""
+    import torch
+    from iris_testing_amd import ops
+    dev = "cuda"
+    H = cfg.hidden
+    B = 2
+    rows = (1 << 30) // (H * B)
+    src = torch.randn((rows, H), device=dev, dtype=torch.float32).to(torch.bfloat16)
+    ident = torch.arange(rows, dtype=torch.int32, device=dev)
+    dst = torch.empty_like(src)
+    L_ = __import__("iris_testing_amd._lib", fromlist=["x"])
+    lib, p, st = L_.lib(), L_.ptr, L_.stream_ptr
+
+    def copy():
+        L_.check(lib.moe_pack_payload(p(src), 1, rows, H, p(ident), rows, p(dst), st()))
+    ms_copy = _timed(copy, steps, torch)
+    zero_counts = torch.zeros((1, 1), dtype=torch.int32, device=dev)
+
+    def write():
+        L_.check(lib.moe_zero_padding_rows(p(dst), 1, 1, rows, H, p(zero_counts), 1, st()))
+    ms_write = _timed(write, steps, torch)
+    n_bytes = rows * H * B
+    copy_rate = 2 * n_bytes / ms_copy / 1e6   # GB/s
+    write_rate = n_bytes / ms_write / 1e6
+    read_rate = n_bytes / (ms_copy - ms_write) / 1e6 if ms_copy > ms_write else float("nan")
+    out = {"buffer_rows": rows, "row_bytes": H * B,
+           "copy": {"kernel": "gather_rows_kernel (moe_pack_payload, identity map)", "ms": round(ms_copy, 4), "GB/s": round(copy_rate, 1)},
+           "write": {"kernel": "zero_padding_rows_kernel (every row padding)", "ms": round(ms_write, 4), "GB/s": round(write_rate, 1)},
+           "model": {"read_GB/s": round(read_rate, 1), "write_GB/s": round(write_rate, 1),
+                     "formula": "time = bytes read / read rate + bytes written / write rate; read rate from copy time - write time"},
+           "combine_unit_gates": {}}
+    for k in (1, 2, 8):
+        T = rows // k
+        idx = torch.zeros((T, k), dtype=torch.int32, device=dev)
+        # slot of (t, kk): rows spread over the whole buffer, every row read exactly once
+        pos = (torch.arange(T, device=dev, dtype=torch.int32)[:, None] + T * torch.arange(k, device=dev, dtype=torch.int32)[None, :]).contiguous()
+        zero = torch.zeros(1, dtype=torch.int32, device=dev)
+        o = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+
+        def comb():
+            L_.check(lib.moe_combine(p(src), 1, 1, rows, H, p(idx), p(pos), None, p(zero), T, k, 1, p(o), None, st()))
+        ms = _timed(comb, steps, torch)
+        rd, wr = T * k * H * B, T * H * B
+        model_ms = (rd / read_rate + wr / write_rate) / 1e6
+        out["combine_unit_gates"][f"k={k}"] = {"ms": round(ms, 4), "GB/s": round((rd + wr) / ms / 1e6, 1), "read_share": round(rd / (rd + wr), 3),
+                                                "model_GB/s": round((rd + wr) / model_ms / 1e6, 1)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -117,6 +272,15 @@ def main():
     ap.add_argument("--unfused", action="store_true",
                     help="run the destination side as unpack + MLP + return pack (the reference's operator split) "
                          "instead of gathering / scattering inside the GEMMs")
+    ap.add_argument("--gated", action="store_true",
+                    help="ship the top-k gates with the rows, weight the result rows in the down projection's epilogue, "
+                         "combine by plain sum (bf16 experts)")
+    ap.add_argument("--padding-free", action="store_true",
+                    help="rows cross as the padding-free payload instead of fixed-M slots: the GEMMs gather from / scatter "
+                         "into flat buffers through a row map over the payload")
+    ap.add_argument("--backward", action="store_true", help="also time forward + backward of rank 0's expert MLP")
+    ap.add_argument("--stream-ceiling", action="store_true",
+                    help="also measure copy / write / read-mostly rates of the row-moving kernels on 1 GiB buffers")
     ap.add_argument("--cpu-sample-tokens", type=int, default=0, help="0 = sized for roughly 10-30 s")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -140,14 +304,18 @@ def main():
     world = harness.build_world(cfg, dev)
     ew, raw, qs = harness.expert_weights(cfg, 0, dev)
     pipe = DispatchPipeline(world, ew, fused=False if args.unfused else None,
-                            fp8_dispatch=False if (args.unfused or args.bf16_dispatch) else None)
+                            fp8_dispatch=False if (args.unfused or args.bf16_dispatch or args.padding_free) else None,
+                            gated=args.gated, padding_free=args.padding_free,
+                            recv_gate=harness.recv_gates(world) if args.gated else None,
+                            recv_flat=harness.recv_flat(world) if args.padding_free else None)
     # the returned buffer: slot 0 is rank 0's own return slot; the other slots stand in for what the
     # other ranks' experts would send back (same shape and dtype, arbitrary finite contents)
     pipe.step()
     torch.cuda.synchronize()
     g = torch.Generator(device="cpu").manual_seed(cfg.seed + 4242)
     pipe.returned.copy_(torch.randn(pipe.returned.shape, generator=g, dtype=torch.float32).to(cfg.torch_dtype))
-    pipe.returned[0].copy_(pipe.ret[0])
+    if not args.padding_free:
+        pipe.returned[0].copy_(pipe.ret[0])
     assert int(pipe.status.item()) == 0
 
     for _ in range(args.warmup):
@@ -201,14 +369,19 @@ def main():
             # a few KB or a few rows: no roofline applies, the time is launch + dependency latency
             stages[n] = {"ms": round(ms, 4), "bound": "latency", "bytes": wk["amount"]}
             continue
-        if wk["bound"] == "hbm":
+        bound = wk["bound"]
+        if bound == "hbm" and wk.get("flops", 0) / (PEAK["fp32"] * 1e12) > wk["amount"] / (PEAK["hbm"] * 1e9):
+            # more fp32 matrix work than memory traffic (the router logits of a workload with many experts): the fp32 rate binds
+            bound = "fp32"
+            ach, peak, unit = wk["flops"] / (ms * 1e-3) / 1e12, PEAK["fp32"], "TFLOP/s"
+        elif bound == "hbm":
             ach, peak, unit = wk["amount"] / (ms * 1e-3) / 1e9, PEAK["hbm"], "GB/s"
         else:
             ach = wk["amount"] / (ms * 1e-3) / 1e12
             peak = PEAK["mfma_fp8"] if cfg.quant == "fp8" else (PEAK["fp32"] if cfg.dtype == "f32" else PEAK["mfma_bf16"])
             unit = "TFLOP/s"
         stages[n] = {"ms": round(ms, 4), "ms_min": round(stage_spread[n][0], 4), "ms_median": round(stage_spread[n][1], 4),
-                     "bound": wk["bound"], "achieved": round(ach, 2), "peak": peak, "unit": unit, "frac": round(ach / peak, 4)}
+                     "bound": bound, "achieved": round(ach, 2), "peak": peak, "unit": unit, "frac": round(ach / peak, 4)}
     dom = "mlp_up"  # the gate/up grouped GEMM: most of the flops of a step
     traffic, traffic_source = profiled_traffic(cfg.name, dom + "_fp8_dispatch" if pipe.fp8_dispatch else dom)
     if cfg.quant == "fp8":
@@ -239,7 +412,9 @@ def main():
         "routed_rows_per_s": round(cfg.tokens * cfg.topk / (ms_per_step * 1e-3), 1),
         "host_wall_ms_per_step": round(wall * 1e3 / args.steps, 4),
         "launch": launch,
-        "destination_side": "gather/scatter inside the GEMMs" if pipe.fused else "unpack + MLP + return pack",
+        "destination_side": ("gather/scatter inside the GEMMs over the padding-free payload" if pipe.padding_free else
+                             "gather/scatter inside the GEMMs, result rows weighted by their gates, combine by plain sum" if pipe.gated
+                             else "gather/scatter inside the GEMMs" if pipe.fused else "unpack + MLP + return pack"),
         "dispatch": "fp8 codes + row scales (quantised while packing)" if pipe.fp8_dispatch else cfg.dtype,
         "ms_per_step_stream": round(stream_ms_per_step, 4),
         "ms_per_step_graph": None if ms_graph is None else round(ms_graph, 4),
@@ -247,12 +422,19 @@ def main():
         "stages": stages,
     }
 
+    if args.backward:
+        if cfg.quant == "fp8":
+            out["backward"] = {"skipped": "the fp8 expert has no backward pass"}
+        else:
+            out["backward"] = backward_leg(cfg, world, raw, max(args.steps // 4, 2))
+    if args.stream_ceiling:
+        out["stream_ceiling"] = stream_ceiling_leg(cfg, max(args.steps // 2, 3))
+
     if not args.no_cpu_baseline:
         def to_np(t):
             t = t.detach().cpu()
             return t.float().numpy() if t.dtype == torch.bfloat16 else t.numpy()
 
-        x_np = to_np(world.x0)
         router_np = to_np(world.router)
         bias_np = None if world.bias is None else to_np(world.bias)
         if qs is not None:
@@ -261,7 +443,7 @@ def main():
             w_np = tuple(to_np(t) for t in raw)
         flops_per_token = 2 * cfg.hidden * cfg.ffn * cfg.n_mat * cfg.topk
         sample = args.cpu_sample_tokens or max(64, min(cfg.tokens, int(1.2e13 / flops_per_token)))
-        v, secs, threads, desc = cpu_baseline(cfg, (x_np, router_np, bias_np, w_np), sample)
+        v, secs, threads, desc = cpu_baseline(cfg, router_np, bias_np, w_np, sample)
         out["cpu_baseline"] = {"value": round(v, 1), "unit": "tokens/s", "cores": threads, "kind": "port",
                                "sample": desc, "seconds": round(secs, 2), "host_cpus": os.cpu_count(),
                                "per_element_loop_plumbing": per_element_loop_baseline()}

@@ -118,6 +118,15 @@ int moe_pack_tokens(const void* x, int dtype, int T, int H, const int32_t* topk_
                     int E_l, const int32_t* dst_sizes, const int32_t* dst_offsets, int W, int M, void* send_buf,
                     int32_t* status, moe_stream_t stream);
 
+/* moe_pack_tokens that also ships each slot's top-k gate: send_gate[dst,m] = gate[t,kk] (fp32 [W,M], zero in the padding
+ * slots), for a destination that multiplies the expert's result rows by their gates before it returns them
+ * (moe_recv_row_map_gated, moe_grouped_gemm_mapped_gated) so that the source only adds (moe_combine with gate == NULL).
+ * gate [T,k] as moe_route_topk returns it.  The reference drops the gates (utils.py:202) and has no return path: this
+ * carries the same README.md:5-7 layout one column further. */
+int moe_pack_tokens_gated(const void* x, int dtype, int T, int H, const int32_t* topk_idx, const int32_t* pos,
+                          const float* gate, int k, int E_l, const int32_t* dst_sizes, const int32_t* dst_offsets, int W, int M,
+                          void* send_buf, float* send_gate, int32_t* status, moe_stream_t stream);
+
 /* The fp8 form of the same send buffer (BASELINE workload "quantized skew sweep": activations quantised per token to
  * e4m3 for the fp8 grouped GEMM).  Per-row quantisation commutes with moving rows, so the tokens can be quantised where
  * they are packed: send_q [W,M,H] codes and send_scale [W,M] hold, slot for slot, what moe_quantize_rows_fp8 would make
@@ -126,6 +135,11 @@ int moe_pack_tokens(const void* x, int dtype, int T, int H, const int32_t* topk_
 int moe_pack_tokens_fp8(const void* x_bf16, int T, int H, const int32_t* topk_idx, const int32_t* pos, int k, int E_l,
                         const int32_t* dst_sizes, const int32_t* dst_offsets, int W, int M, uint8_t* send_q,
                         float* send_scale, int32_t* status, moe_stream_t stream);
+
+/* moe_pack_tokens_fp8 that also ships the gates (send_gate [W,M], as moe_pack_tokens_gated). */
+int moe_pack_tokens_fp8_gated(const void* x_bf16, int T, int H, const int32_t* topk_idx, const int32_t* pos, const float* gate,
+                              int k, int E_l, const int32_t* dst_sizes, const int32_t* dst_offsets, int W, int M, uint8_t* send_q,
+                              float* send_scale, float* send_gate, int32_t* status, moe_stream_t stream);
 
 /* ---- a9: receive layout (reference baseline.py:178-222; kernels.py:93-102,124-125) ------------
  * recv [W,M,H]: slot s holds what source s sent to this rank ((el, token) order, zero padded);
@@ -235,6 +249,26 @@ int moe_grouped_gemm_mapped(const void* a_base, int a_rows, const int32_t* a_row
                             const int32_t* expert_cnt, int S_rows, int K, int N, int E_l, int act, void* out,
                             int out_rows, const int32_t* c_row_map, void* part_ws, size_t part_ws_bytes,
                             moe_stream_t stream);
+/* Two more forms of the row map, for the two ways the fused destination side is widened:
+ *   moe_recv_row_map_flat   the receive buffer is a padding-free flat payload [sum recv_counts, H] instead of [W,M,H]:
+ *                           source-major, expert-minor blocks, what each source's send_payload[dst_offsets[dst] ..] holds
+ *                           (reference utils.py:235-246) and reorder_flat_to_token_buf reads (baseline.py:204-218);
+ *                           row_map[r] = start of block (s,e) + j.  No row can have been dropped, nothing is padding; the
+ *                           same map places result row r in a flat returned buffer.
+ *   moe_recv_row_map_gated  M >= 1: moe_recv_row_map; M == 0: moe_recv_row_map_flat; with recv_gate (fp32, one per row of
+ *                           the receive buffer, as moe_pack_tokens_gated ships them) also row_gate[r] = recv_gate[row_map[r]]
+ *                           (0 for rows without a source), the row gates in the GEMM's row order.  Both or neither.
+ *   moe_grouped_gemm_mapped_gated  moe_grouped_gemm_mapped without activation whose result row r is multiplied by
+ *                           row_gate[r] in fp32 before the one rounding to bf16: the down projection of an expert MLP whose
+ *                           rows return already weighted (the combine then only adds: moe_combine with gate == NULL). */
+int moe_recv_row_map_flat(const int32_t* recv_counts, int W, int E_l, int n_rows, int32_t* row_map, int32_t* expert_cnt,
+                          moe_stream_t stream);
+int moe_recv_row_map_gated(const int32_t* recv_counts, int W, int E_l, int M, int n_rows, const float* recv_gate,
+                           int32_t* row_map, float* row_gate, int32_t* expert_cnt, moe_stream_t stream);
+int moe_grouped_gemm_mapped_gated(const void* a_base, int a_rows, const int32_t* a_row_map, const void* packed,
+                                  const int32_t* expert_cnt, int S_rows, int K, int N, int E_l, const float* row_gate, void* out,
+                                  int out_rows, const int32_t* c_row_map, void* part_ws, size_t part_ws_bytes,
+                                  moe_stream_t stream);
 size_t moe_gemm_part_workspace_bytes(void);
 /* How a launch with total_tiles output tiles, a persistent grid of `grid` workgroups, k_stages 64-byte stages of K
  * (even) and room for max_units part tiles in the workspace is walked: out[0] = tiles taken whole, out[1] = parts
@@ -314,7 +348,9 @@ int moe_return_pack(const void* y, int dtype, int S_rows, int H, const int32_t* 
                     int M, void* ret, int32_t* map_ws, moe_stream_t stream);
 
 /* out[t,:] = sum_kk gate[t,kk] * ret[dst, pos[t,kk]-dst_offsets[dst], :], dst = idx[t,kk]/E_l;
- * fp32 multiply then add in ascending kk (no fma), one rounding to `dtype`.  A slot whose dst lies
+ * fp32 multiply then add in ascending kk (no fma), one rounding to `dtype`.  gate == NULL: the rows arrive weighted
+ * (moe_grouped_gemm_mapped_gated) and are only added, in the same order.  A flat returned payload [R,H] in payload order
+ * (row = pos[t,kk]) is the case W = 1, M = R, E_l = number of experts, dst_offsets = {0}.  A slot whose dst lies
  * outside [0,W) or whose row lies outside [0,M) -- a row the pack dropped because the pair capacity
  * was exceeded -- has no returned row: it is skipped and *status (nullable) is set to 1. */
 int moe_combine(const void* ret, int dtype, int W, int M, int H, const int32_t* topk_idx, const int32_t* pos,

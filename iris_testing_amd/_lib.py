@@ -43,6 +43,11 @@ _SIGNATURES = {
     "moe_pack_payload": (c_int, [P, c_int, c_int, c_int, P, c_int, P, P]),
     "moe_pack": (c_int, [P, c_int, c_int, c_int, P, P, P, c_int, c_int, P, P, P, P]),
     "moe_pack_tokens": (c_int, [P, c_int, c_int, c_int, P, P, c_int, c_int, P, P, c_int, c_int, P, P, P]),
+    "moe_pack_tokens_gated": (c_int, [P, c_int, c_int, c_int, P, P, P, c_int, c_int, P, P, c_int, c_int, P, P, P, P]),
+    "moe_pack_tokens_fp8_gated": (c_int, [P, c_int, c_int, P, P, P, c_int, c_int, P, P, c_int, c_int, P, P, P, P, P]),
+    "moe_recv_row_map_flat": (c_int, [P, c_int, c_int, c_int, P, P, P]),
+    "moe_recv_row_map_gated": (c_int, [P, c_int, c_int, c_int, c_int, P, P, P, P, P]),
+    "moe_grouped_gemm_mapped_gated": (c_int, [P, c_int, P, P, P, c_int, c_int, c_int, c_int, P, P, c_int, P, P, c_size_t, P]),
     "moe_recv_map_ints": (c_size_t, [c_int, c_int, c_int]),
     "moe_unpack_token_buf": (c_int, [P, c_int, c_int, c_int, c_int, P, c_int, c_int, P, P, P, P, P]),
     "moe_reorder_flat_to_token_buf": (c_int, [P, c_int, c_int, c_int, P, c_int, c_int, c_int, P, P, P, P]),

@@ -432,7 +432,10 @@ __global__ __launch_bounds__(WPB * WAVE) void pack_tokens_kernel(const u32x4* __
                                                                   const int32_t* __restrict__ idx, const int32_t* __restrict__ pos,
                                                                   const int32_t* __restrict__ dst_sizes,
                                                                   const int32_t* __restrict__ dst_offsets, int T, int k, int E_l,
-                                                                  int W, int M, int row_vec, int32_t* __restrict__ status) {
+                                                                  int W, int M, int row_vec, int32_t* __restrict__ status,
+                                                                  const float* __restrict__ gate, float* __restrict__ send_gate) {
+    // gate / send_gate (both or neither): the slot's top-k gate travels with its row, send_gate[d,m] = gate[t,kk], zero
+    // in the padding slots -- for a destination that applies the gate to the expert's result before sending it back
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const int n_slots = W * M;
     const int n_units = T + (n_slots + PACK_ZR - 1) / PACK_ZR;
@@ -448,6 +451,7 @@ __global__ __launch_bounds__(WPB * WAVE) void pack_tokens_kernel(const u32x4* __
                     u32x4* o = send + (size_t)sl * row_vec;
                     // (ordinary stores: measured 4 to 10 % faster here than non-temporal ones, which win for the copies below)
                     for (int c = lane; c < row_vec; c += WAVE) o[c] = z;
+                    if (send_gate && lane == 0) send_gate[sl] = 0.f;
                 }
                 if (++m == M && sl + 1 < s1) { m = 0; cnt = dst_sizes[++d]; }
             }
@@ -463,6 +467,7 @@ __global__ __launch_bounds__(WPB * WAVE) void pack_tokens_kernel(const u32x4* __
                 const bool d_ok = (unsigned)d < (unsigned)W;  // (an expert id outside [0, W E_l): no slot, and no read of its offset)
                 const int m = pos[(size_t)r * k + j] - dst_offsets[d_ok ? d : 0];
                 if (d_ok && (unsigned)m < (unsigned)M) drow[j] = d * M + m;
+                if (send_gate && drow[j] >= 0 && lane == 0) send_gate[drow[j]] = gate[(size_t)r * k + j];
             }
         }
         const u32x4* src = x + (size_t)r * row_vec;
@@ -541,7 +546,7 @@ __global__ __launch_bounds__(WPB * WAVE) void combine_kernel(const uint4* __rest
                 const int m = pos[(size_t)t * k + j] - dst_offsets[d_ok ? d : 0];
                 have[j] = d_ok && (unsigned)m < (unsigned)M;
                 rows[j] = have[j] ? ((size_t)d * M + m) * row_vec : 0;
-                g[j] = gate[(size_t)t * k + j];
+                g[j] = gate ? gate[(size_t)t * k + j] : 1.f;  // (no gates: the rows arrive weighted, 1 * x is x exactly)
                 if (!have[j] && status && lane == 0) *status = 1;
             }
         }
@@ -669,11 +674,18 @@ int gather_rows(const void* src, void* dst, const RowSource& a, int n_rows, int 
 // the pair capacity M) map to -1: the GEMMs read row 0 for them and store nothing.
 // One launch: every block derives the two prefix tables it needs from recv_counts in LDS (at most
 // MOE_MAX_EXPERTS entries: a wave's scan) instead of waiting for a table kernel; block 0 also leaves the per-expert totals.
+// M = 0: the receive buffer is a padding-free flat payload instead (source-major, expert-minor blocks, the layout
+// reorder_flat_to_token_buf of the reference reads, baseline.py:204-218): the row of (e, s, j) is the exclusive prefix of the
+// counts over flattened (s, e) plus j, and no row can have been dropped.
+// recv_gate / row_gate (both or neither): the gates that arrived with the rows, [rows of the receive buffer], gathered
+// into expert-major order for the GEMM that applies them (0 for rows without a source).
 __global__ __launch_bounds__(256) void row_map_from_counts_kernel(const int32_t* __restrict__ rc, int W, int E_l, int M, int n_rows,
-                                                                   int32_t* __restrict__ map, int32_t* __restrict__ expert_cnt) {
+                                                                   int32_t* __restrict__ map, int32_t* __restrict__ expert_cnt,
+                                                                   const float* __restrict__ recv_gate, float* __restrict__ row_gate) {
     __shared__ int32_t s_row_off[MOE_MAX_EXPERTS + 1];
     __shared__ int32_t s_src_off[MOE_MAX_EXPERTS];
     const int n = W * E_l;
+    const bool flat = M == 0;
     if (threadIdx.x < WAVE) {
         const int lane = lane_id();
         const int per = (n + WAVE - 1) / WAVE;
@@ -684,9 +696,17 @@ __global__ __launch_bounds__(256) void row_map_from_counts_kernel(const int32_t*
         int run = incl - sum;
         for (int i = lo; i < hi; ++i) { s_row_off[i] = run; run += rc[(i % W) * E_l + (i / W)]; }
         if (lane == WAVE - 1) s_row_off[n] = incl;
-        for (int sr = lane; sr < W; sr += WAVE) {
-            int r = 0;
-            for (int e = 0; e < E_l; ++e) { s_src_off[sr * E_l + e] = r; r += rc[sr * E_l + e]; }
+        if (flat) {  // exclusive prefix over flattened (s, e): where the block of (s, e) starts in the flat payload
+            int fsum = 0;
+            for (int i = lo; i < hi; ++i) fsum += rc[i];
+            const int fincl = wave_incl_scan(fsum);
+            int frun = fincl - fsum;
+            for (int i = lo; i < hi; ++i) { s_src_off[i] = frun; frun += rc[i]; }
+        } else {
+            for (int sr = lane; sr < W; sr += WAVE) {
+                int r = 0;
+                for (int e = 0; e < E_l; ++e) { s_src_off[sr * E_l + e] = r; r += rc[sr * E_l + e]; }
+            }
         }
         if (blockIdx.x == 0 && expert_cnt)
             for (int e = lane; e < E_l; e += WAVE) {
@@ -698,7 +718,11 @@ __global__ __launch_bounds__(256) void row_map_from_counts_kernel(const int32_t*
     __syncthreads();
     const int r = blockIdx.x * blockDim.x + threadIdx.x;
     if (r >= n_rows) return;
-    if (r >= s_row_off[n]) { map[r] = 0; return; }
+    if (r >= s_row_off[n]) {
+        map[r] = 0;
+        if (row_gate) row_gate[r] = 0.f;
+        return;
+    }
     int lo = 0, hi = n;  // s_row_off[0] = 0 <= r; the last of a run of equal offsets owns the row
     while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;
@@ -706,7 +730,9 @@ __global__ __launch_bounds__(256) void row_map_from_counts_kernel(const int32_t*
     }
     const int e = lo / W, sr = lo % W;
     const int m = s_src_off[sr * E_l + e] + (r - s_row_off[lo]);
-    map[r] = m < M ? sr * M + m : -1;
+    const int row = flat ? m : (m < M ? sr * M + m : -1);
+    map[r] = row;
+    if (row_gate) row_gate[r] = row >= 0 ? recv_gate[row] : 0.f;
 }
 
 // rows [size_s, M) of every slot s of a [W,M,row] buffer <- 0, size_s = sum over e of rc[s,e]; one wave per run of
@@ -881,10 +907,11 @@ extern "C" int moe_pack(const void* x, int dtype, int T, int H, const int32_t* r
     return gather_rows(x, send_buf, a, W * M, H * dtype_size(dtype), s);
 }
 
-extern "C" int moe_pack_tokens(const void* x, int dtype, int T, int H, const int32_t* topk_idx, const int32_t* pos, int k,
-                               int E_l, const int32_t* dst_sizes, const int32_t* dst_offsets, int W, int M, void* send_buf,
-                               int32_t* status, moe_stream_t stream) {
+extern "C" int moe_pack_tokens_gated(const void* x, int dtype, int T, int H, const int32_t* topk_idx, const int32_t* pos,
+                                     const float* gate, int k, int E_l, const int32_t* dst_sizes, const int32_t* dst_offsets, int W,
+                                     int M, void* send_buf, float* send_gate, int32_t* status, moe_stream_t stream) {
     int rc = check_rows("pack_tokens", dtype, H);
+    MOE_REQUIRE((gate == nullptr) == (send_gate == nullptr), MOE_ERR_INVALID, "pack_tokens: gate and send_gate go together");
     if (rc) return rc;
     MOE_REQUIRE(W > 0 && M >= 1 && T >= 0 && E_l > 0, MOE_ERR_INVALID, "pack_tokens: bad shape W=%d M=%d E_l=%d", W, M, E_l);
     MOE_REQUIRE(k >= 1 && k <= MOE_MAX_TOPK, MOE_ERR_UNSUPPORTED, "pack_tokens: topk=%d outside [1,%d]", k, MOE_MAX_TOPK);
@@ -895,8 +922,15 @@ extern "C" int moe_pack_tokens(const void* x, int dtype, int T, int H, const int
     const int blocks = min(ceil_div(n_units, 4), 65535 * 8);
     pack_tokens_kernel<4><<<blocks, 4 * WAVE, 0, (hipStream_t)stream>>>((const u32x4*)x, (u32x4*)send_buf, topk_idx, pos, dst_sizes,
                                                                         dst_offsets, T, k, E_l, W, M,
-                                                                        H * dtype_size(dtype) / 16, status);
+                                                                        H * dtype_size(dtype) / 16, status, gate, send_gate);
     return moe_check_launch("pack_tokens");
+}
+
+extern "C" int moe_pack_tokens(const void* x, int dtype, int T, int H, const int32_t* topk_idx, const int32_t* pos, int k,
+                               int E_l, const int32_t* dst_sizes, const int32_t* dst_offsets, int W, int M, void* send_buf,
+                               int32_t* status, moe_stream_t stream) {
+    return moe_pack_tokens_gated(x, dtype, T, H, topk_idx, pos, nullptr, k, E_l, dst_sizes, dst_offsets, W, M, send_buf, nullptr,
+                                 status, stream);
 }
 
 static int recv_driven(const char* who, int mode, const void* src, void* dst, int dtype, int H, const int32_t* rc_dev,
@@ -963,8 +997,25 @@ extern "C" int moe_recv_row_map(const int32_t* recv_counts, int W, int E_l, int 
     (void)map_ws;  // (the tables of earlier versions live in LDS now)
     MOE_REQUIRE(n_rows == 0 || row_map, MOE_ERR_INVALID, "recv_row_map: null pointer");
     // (one launch: every block rebuilds the prefix tables in LDS; at least one block, for the per-expert totals)
-    row_map_from_counts_kernel<<<max(ceil_div(n_rows, 256), 1), 256, 0, s>>>(recv_counts, W, E_l, M, n_rows, row_map, expert_cnt);
+    row_map_from_counts_kernel<<<max(ceil_div(n_rows, 256), 1), 256, 0, s>>>(recv_counts, W, E_l, M, n_rows, row_map, expert_cnt,
+                                                                             nullptr, nullptr);
     return moe_check_launch("recv_row_map");
+}
+
+extern "C" int moe_recv_row_map_gated(const int32_t* recv_counts, int W, int E_l, int M, int n_rows, const float* recv_gate,
+                                      int32_t* row_map, float* row_gate, int32_t* expert_cnt, moe_stream_t stream) {
+    MOE_REQUIRE(W > 0 && E_l > 0 && W * E_l <= MOE_MAX_EXPERTS, MOE_ERR_INVALID, "recv_row_map_gated: bad W=%d E_l=%d", W, E_l);
+    MOE_REQUIRE(M >= 0 && n_rows >= 0 && recv_counts, MOE_ERR_INVALID, "recv_row_map_gated: bad arguments");
+    MOE_REQUIRE((recv_gate == nullptr) == (row_gate == nullptr), MOE_ERR_INVALID, "recv_row_map_gated: recv_gate and row_gate go together");
+    MOE_REQUIRE(n_rows == 0 || row_map, MOE_ERR_INVALID, "recv_row_map_gated: null pointer");
+    row_map_from_counts_kernel<<<max(ceil_div(n_rows, 256), 1), 256, 0, (hipStream_t)stream>>>(recv_counts, W, E_l, M, n_rows, row_map,
+                                                                                               expert_cnt, recv_gate, row_gate);
+    return moe_check_launch("recv_row_map_gated");
+}
+
+extern "C" int moe_recv_row_map_flat(const int32_t* recv_counts, int W, int E_l, int n_rows, int32_t* row_map, int32_t* expert_cnt,
+                                     moe_stream_t stream) {
+    return moe_recv_row_map_gated(recv_counts, W, E_l, 0, n_rows, nullptr, row_map, nullptr, expert_cnt, stream);
 }
 
 extern "C" int moe_zero_padding_rows(void* buf, int dtype, int W, int M, int H, const int32_t* recv_counts, int E_l,
@@ -1050,7 +1101,7 @@ extern "C" int moe_combine(const void* ret, int dtype, int W, int M, int H, cons
     MOE_REQUIRE(W > 0 && M >= 1 && T >= 0 && E_l > 0, MOE_ERR_INVALID, "combine: bad shape");
     MOE_REQUIRE(k >= 1 && k <= MOE_MAX_TOPK, MOE_ERR_UNSUPPORTED, "combine: topk=%d outside [1,%d]", k, MOE_MAX_TOPK);
     if (T == 0) return MOE_OK;
-    MOE_REQUIRE(ret && topk_idx && pos && gate && dst_offsets && out, MOE_ERR_INVALID, "combine: null pointer");
+    MOE_REQUIRE(ret && topk_idx && pos && dst_offsets && out, MOE_ERR_INVALID, "combine: null pointer");  // (gate may be NULL)
     const int row_vec = H * dtype_size(dtype) / 16;
     if (dtype == MOE_F32) return launch_combine<float>(ret, topk_idx, pos, gate, dst_offsets, T, k, E_l, W, M, row_vec, out, status, s);
     return launch_combine<bf16_t>(ret, topk_idx, pos, gate, dst_offsets, T, k, E_l, W, M, row_vec, out, status, s);

@@ -49,7 +49,7 @@ struct GemmParams {
     void* C2;                 // optional (bf16 kernels with an activation): the values BEFORE the activation, bf16, row pitch ldc
                               // (SwiGLU: 2 ldc, in the packed gate / up column order), kept for the backward pass
     const int32_t* cnt;       // [E_l] rows per group
-    const float* row_scale;   // fp8: [S_rows] per-row activation scale
+    const float* row_scale;   // fp8: [S_rows] per-row activation scale; bf16 with EPI_GATE: [S_rows] per-row gate
     const float* col_scale;   // fp8: [E_l, ncs] per-output-channel scale (gate for SwiGLU)
     const float* col_scale2;  // fp8 SwiGLU: [E_l, ncs] up scales
     const int32_t* a_map;     // optional: logical row -> row of A (gather while loading), else A is row r itself
@@ -169,7 +169,10 @@ __device__ __forceinline__ int seg_of(const int* off, int n, int r) {
     return lo;
 }
 
-enum { EPI_NONE = 0, EPI_GELU = 1, EPI_SILU = 2, EPI_SWIGLU = 3 };
+// EPI_GATE: no activation, and every result row is multiplied by its row's gate (GemmParams::row_scale, one fp32
+// multiplication before the rounding to bf16): the down projection of an expert whose rows return already weighted.
+// (The fp8 kernels have a row scale as it is: a gate is folded into it by the caller.)
+enum { EPI_NONE = 0, EPI_GELU = 1, EPI_SILU = 2, EPI_SWIGLU = 3, EPI_GATE = 4 };
 
 // One output tile of the walk: group g, n tile nt, first row row0, rv valid rows (rv <= 0: none).
 struct GgTile {
@@ -625,7 +628,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                 const int lane_t = gg_lane_now(), tid_t = wave_s * WAVE + lane_t;  // (a fresh lane id: nothing kept live for this)
                 const uint32_t t4 = (uint32_t)min(tid_t, rv - 1) * 4u;
                 if (wave_s * WAVE < BM) {
-                    if constexpr (FP8)
+                    if constexpr (FP8 || EPI == EPI_GATE)
                         gg_dma4(gg_uniform((const uint8_t*)(p.row_scale + row0)), t4,
                                 __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(s_row_scale[tpar] + wave_s * WAVE)));
                     if (p.c_map)
@@ -762,7 +765,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         const int lsub = FP8 ? (lane_e >> 5) : (lane_e >> 4);  // which of the lanes that share a tile row this one is
         // What the tile's top requested into LDS (scales, row map) is behind two block ends of the K loop at least -- the
         // second one has waited for it in every wave -- unless the tile has only two stages:
-        if (nks < 4 && (FP8 || p.c_map)) {
+        if (nks < 4 && (FP8 || EPI == EPI_GATE || p.c_map)) {
             gg_wait<0, 15>();
             __syncthreads();
         }
@@ -774,7 +777,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             rs[i] = 1.f;
-            if constexpr (FP8) rs[i] = s_row_scale[tpar][rbase_e + i * MT + (lane_e & (MT - 1))];  // (of the row it computed)
+            if constexpr (FP8 || EPI == EPI_GATE) rs[i] = s_row_scale[tpar][rbase_e + i * MT + (lane_e & (MT - 1))];  // (of the row it computed)
 #pragma unroll
             for (int h = 0; h < NR; ++h) {
                 const int r = rbase_e + i * MT + (FP8 ? (lane_e & 15) + 16 * h : (lane_e & (MT - 1)));
@@ -824,7 +827,8 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                     for (int e = 0; e < 4; ++e) {
                         float v = acc[i][j][4 * qd + e];
                         if constexpr (FP8) v *= cg[e] * rs[i];
-                        if constexpr (!FP8 && EPI != EPI_NONE) pre_g[4 * t + e] = v;
+                        if constexpr (!FP8 && EPI == EPI_GATE) v *= rs[i];
+                        if constexpr (!FP8 && EPI != EPI_NONE && EPI != EPI_GATE) pre_g[4 * t + e] = v;
                         if constexpr (EPI == EPI_SWIGLU) {
                             float uv = acc[i][ju % TN][4 * qd + e];
                             if constexpr (FP8) uv *= cu[e] * rs[i];
@@ -845,7 +849,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                     pk[u] = o4;
                 } else if (ok[i][0] && col < p.N) {
                     *(uint4*)(crow[i][0] + col) = o4;
-                    if constexpr (EPI != EPI_NONE) {
+                    if constexpr (EPI != EPI_NONE && EPI != EPI_GATE) {
                         if (p.C2) {
                             // same row, in a matrix whose rows are as long (SwiGLU: twice as long, packed column order)
                             constexpr int W2 = EPI == EPI_SWIGLU ? 2 : 1;
@@ -967,9 +971,9 @@ __global__ __launch_bounds__(256) void gg_reduce_parts_kernel(const GemmParams p
         }
         const size_t grow = (size_t)(t.row0 + r);
         float rs = 1.f;
-        if constexpr (FP8) rs = p.row_scale[grow];
+        if constexpr (FP8 || EPI == EPI_GATE) rs = p.row_scale[grow];
         float av[4] = {a.x, a.y, a.z, a.w}, bv[4] = {b.x, b.y, b.z, b.w};
-        if constexpr (!FP8 && EPI != EPI_NONE) {
+        if constexpr (!FP8 && EPI != EPI_NONE && EPI != EPI_GATE) {
             if (p.C2 && col < p.N) {  // the values before the activation, kept for the backward pass (rows are never remapped there)
                 constexpr int W2 = EPI == EPI_SWIGLU ? 2 : 1;
                 bf16_t* r2 = (bf16_t*)p.C2 + grow * (size_t)p.ldc * W2 + (EPI == EPI_SWIGLU ? gp : col);
@@ -993,6 +997,7 @@ __global__ __launch_bounds__(256) void gg_reduce_parts_kernel(const GemmParams p
             } else {
                 float v = av[e];
                 if constexpr (FP8) v *= c0[e] * rs;
+                if constexpr (!FP8 && EPI == EPI_GATE) v *= rs;
                 if constexpr (EPI == EPI_GELU) v = act_gelu(v);
                 if constexpr (EPI == EPI_SILU) v = act_silu_fast(v);
                 x[e] = v;
@@ -1238,7 +1243,9 @@ __global__ __launch_bounds__(256) void pack_tokens_fp8_kernel(const bf16_t* __re
                                                                const int32_t* __restrict__ dst_sizes,
                                                                const int32_t* __restrict__ dst_offsets, int k, int E_l, int W, int M,
                                                                uint8_t* __restrict__ send_q, float* __restrict__ send_scale,
-                                                               int32_t* __restrict__ status) {
+                                                               int32_t* __restrict__ status, const float* __restrict__ gate,
+                                                               float* __restrict__ send_gate) {
+    // (gate / send_gate, both or neither: the slot's top-k gate travels with its row, zero in the padding slots)
     const int wave = threadIdx.x / WAVE, lane = lane_id();
     const int nv = cols / 8;  // 16-byte vectors of bf16 per row = 8-byte vectors of codes
     const int n_slots = W * M;
@@ -1254,6 +1261,7 @@ __global__ __launch_bounds__(256) void pack_tokens_fp8_kernel(const bf16_t* __re
                     uint2* o = (uint2*)(send_q + (size_t)sl * cols);
                     for (int c = lane; c < nv; c += WAVE) o[c] = make_uint2(0u, 0u);
                     if (lane == 0) send_scale[sl] = 1.f;
+                    if (send_gate && lane == 0) send_gate[sl] = 0.f;
                 }
                 if (++m == M && sl + 1 < s1) { m = 0; cnt = dst_sizes[++d]; }
             }
@@ -1268,6 +1276,7 @@ __global__ __launch_bounds__(256) void pack_tokens_fp8_kernel(const bf16_t* __re
                 const bool d_ok = (unsigned)d < (unsigned)W;
                 const int m = pos[(size_t)r * k + j] - dst_offsets[d_ok ? d : 0];
                 if (d_ok && (unsigned)m < (unsigned)M) drow[j] = d * M + m;
+                if (send_gate && drow[j] >= 0 && lane == 0) send_gate[drow[j]] = gate[(size_t)r * k + j];
             }
         }
         const uint4* src = (const uint4*)(x + (size_t)r * cols);
@@ -1566,7 +1575,8 @@ int launch_gemm(const GemmParams& p_in, int epi, hipStream_t s, void* part_ws = 
     do {                                                                                                  \
         if (!all_split) grouped_gemm_kernel<BMv, NWMv, EPIv, FP8, false><<<grid, NWMv * 2 * WAVE, 0, s>>>(p); \
         if (p.part_ws && red_blocks > 0) {                                                                \
-            grouped_gemm_kernel<BMv, NWMv, EPIv, FP8, true><<<grid, NWMv * 2 * WAVE, 0, s>>>(p);           \
+            /* (the launch that takes parts stores raw partial sums: one instantiation whatever the epilogue) */ \
+            grouped_gemm_kernel<BMv, NWMv, EPI_NONE, FP8, true><<<grid, NWMv * 2 * WAVE, 0, s>>>(p);       \
             gg_reduce_parts_kernel<BMv, EPIv, FP8><<<red_blocks, 256, 0, s>>>(p, grid);                    \
         }                                                                                                 \
     } while (0)
@@ -1581,6 +1591,7 @@ int launch_gemm(const GemmParams& p_in, int epi, hipStream_t s, void* part_ws = 
         case EPI_GELU: if constexpr (FP8) return moe_fail(MOE_ERR_UNSUPPORTED, "grouped_gemm: fp8 with activation %d", epi); else GG_EPI(EPI_GELU); break;
         case EPI_SILU: if constexpr (FP8) return moe_fail(MOE_ERR_UNSUPPORTED, "grouped_gemm: fp8 with activation %d", epi); else GG_EPI(EPI_SILU); break;
         case EPI_SWIGLU: GG_EPI(EPI_SWIGLU); break;
+        case EPI_GATE: if constexpr (FP8) return moe_fail(MOE_ERR_UNSUPPORTED, "grouped_gemm: fp8 folds a gate into its row scale"); else GG_EPI(EPI_GATE); break;
         default: return moe_fail(MOE_ERR_INVALID, "grouped_gemm: activation %d", epi);
     }
 #undef GG_EPI
@@ -1703,6 +1714,25 @@ extern "C" int moe_grouped_gemm_mapped(const void* a_base, int a_rows, const int
     return launch_gemm<false>(p, act, (hipStream_t)stream, part_ws, part_ws_bytes);
 }
 
+extern "C" int moe_grouped_gemm_mapped_gated(const void* a_base, int a_rows, const int32_t* a_row_map, const void* packed,
+                                             const int32_t* expert_cnt, int S_rows, int K, int N, int E_l, const float* row_gate,
+                                             void* out, int out_rows, const int32_t* c_row_map, void* part_ws, size_t part_ws_bytes,
+                                             moe_stream_t stream) {
+    MOE_REQUIRE(S_rows >= 0 && K > 0 && N > 0 && E_l > 0 && E_l <= GG_MAXG, MOE_ERR_INVALID, "grouped_gemm_mapped_gated: bad shape");
+    MOE_REQUIRE(K % 64 == 0 && N % 8 == 0, MOE_ERR_UNSUPPORTED, "grouped_gemm_mapped_gated: needs K %% 64 == 0 and N %% 8 == 0 (K=%d N=%d)", K, N);
+    MOE_REQUIRE(a_rows >= 0 && out_rows >= 0, MOE_ERR_INVALID, "grouped_gemm_mapped_gated: negative buffer rows");
+    MOE_REQUIRE(!a_row_map || (unsigned long long)a_rows * (unsigned long long)K * 2ull < (1ull << 32), MOE_ERR_UNSUPPORTED,
+                "grouped_gemm_mapped_gated: the gathered buffer must be smaller than 4 GiB (%d rows of %d)", a_rows, K);
+    if (S_rows == 0) return MOE_OK;
+    MOE_REQUIRE(a_base && packed && expert_cnt && out && row_gate, MOE_ERR_INVALID, "grouped_gemm_mapped_gated: null pointer");
+    GemmParams p{};
+    p.A = (const uint8_t*)a_base; p.B = (const uint8_t*)packed; p.C = out; p.cnt = expert_cnt;
+    p.a_map = a_row_map; p.c_map = c_row_map; p.row_scale = row_gate;
+    p.E_l = E_l; p.K = K; p.N = N; p.ldc = N; p.S_rows = S_rows;
+    p.Npad = round_up(N, GG_BN);
+    return launch_gemm<false>(p, EPI_GATE, (hipStream_t)stream, part_ws, part_ws_bytes);
+}
+
 extern "C" int moe_grouped_gemm_act_keep(const void* a_base, int a_rows, const int32_t* a_row_map, const void* packed,
                                          const int32_t* expert_cnt, int S_rows, int K, int N, int E_l, int act, void* out,
                                          void* pre_act, void* part_ws, size_t part_ws_bytes, moe_stream_t stream) {
@@ -1817,6 +1847,15 @@ extern "C" int moe_grouped_mlp_fp8(const void* tokens_bf16, const int32_t* exper
 extern "C" int moe_pack_tokens_fp8(const void* x_bf16, int T, int H, const int32_t* topk_idx, const int32_t* pos, int k, int E_l,
                                    const int32_t* dst_sizes, const int32_t* dst_offsets, int W, int M, uint8_t* send_q,
                                    float* send_scale, int32_t* status, moe_stream_t stream) {
+    return moe_pack_tokens_fp8_gated(x_bf16, T, H, topk_idx, pos, nullptr, k, E_l, dst_sizes, dst_offsets, W, M, send_q, send_scale,
+                                     nullptr, status, stream);
+}
+
+extern "C" int moe_pack_tokens_fp8_gated(const void* x_bf16, int T, int H, const int32_t* topk_idx, const int32_t* pos,
+                                         const float* gate, int k, int E_l, const int32_t* dst_sizes, const int32_t* dst_offsets,
+                                         int W, int M, uint8_t* send_q, float* send_scale, float* send_gate, int32_t* status,
+                                         moe_stream_t stream) {
+    MOE_REQUIRE((gate == nullptr) == (send_gate == nullptr), MOE_ERR_INVALID, "pack_tokens_fp8: gate and send_gate go together");
     MOE_REQUIRE(T >= 0 && H > 0 && H % 8 == 0 && W > 0 && M >= 1 && E_l > 0, MOE_ERR_INVALID, "pack_tokens_fp8: bad shape");
     MOE_REQUIRE(k >= 1 && k <= MOE_MAX_TOPK, MOE_ERR_UNSUPPORTED, "pack_tokens_fp8: topk=%d outside [1,%d]", k, MOE_MAX_TOPK);
     MOE_REQUIRE((long long)W * M + T < (1ll << 31), MOE_ERR_UNSUPPORTED, "pack_tokens_fp8: W*M + T too large");
@@ -1826,7 +1865,7 @@ extern "C" int moe_pack_tokens_fp8(const void* x_bf16, int T, int H, const int32
     const int blocks = min(ceil_div(n_units, 4), 65535 * 8);
     const int nv = ceil_div(H / 8, WAVE);
     hipStream_t s = (hipStream_t)stream;
-#define GG_PQ(NVv) pack_tokens_fp8_kernel<NVv><<<blocks, 256, 0, s>>>((const bf16_t*)x_bf16, T, H, topk_idx, pos, dst_sizes, dst_offsets, k, E_l, W, M, send_q, send_scale, status)
+#define GG_PQ(NVv) pack_tokens_fp8_kernel<NVv><<<blocks, 256, 0, s>>>((const bf16_t*)x_bf16, T, H, topk_idx, pos, dst_sizes, dst_offsets, k, E_l, W, M, send_q, send_scale, status, gate, send_gate)
     if (nv <= 2) GG_PQ(2);
     else if (nv <= 4) GG_PQ(4);
     else if (nv <= 8) GG_PQ(8);

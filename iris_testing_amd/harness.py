@@ -111,3 +111,30 @@ def quantize_weight_fp8(w: torch.Tensor):
     inv = torch.where(zero, torch.ones_like(amax), 448.0 / safe)
     q = (wf * inv[:, None, :]).to(torch.float8_e4m3fn).view(torch.uint8)
     return q.contiguous(), scale.contiguous()
+
+
+def recv_gates(world: World, dst_rank: int = 0) -> torch.Tensor:
+    """[W,M] fp32: the gates that arrive with rank ``dst_rank``'s rows when the sources ship them (ops.pack_tokens with
+    ``gate``): slot s = what source s wrote beside its rows, zero in the padding."""
+    cfg = world.cfg
+    out = torch.empty((cfg.world, world.M), dtype=torch.float32, device=world.recv.device)
+    send = torch.empty((cfg.world, world.M, cfg.hidden), dtype=cfg.torch_dtype, device=world.recv.device)
+    for s, r in enumerate(world.routes):
+        x = world.x0 if s == 0 else gen_shard_tokens(cfg, s).to(world.recv.device)
+        c = r.counts
+        _, g = ops.pack_tokens(x, r.idx, c.pos, c.dst_sizes, c.dst_offsets, cfg.e_local, world.M, out=send, gate=r.gate)
+        out[s] = g[dst_rank]
+    return out
+
+
+def recv_flat(world: World, dst_rank: int = 0) -> torch.Tensor:
+    """[S,H]: what rank ``dst_rank`` receives when the sources send their padding-free payload (reference utils.py:235-246)
+    instead of fixed-M slots: every source's block for this rank, concatenated in source order."""
+    cfg = world.cfg
+    blocks = []
+    for s, r in enumerate(world.routes):
+        x = world.x0 if s == 0 else gen_shard_tokens(cfg, s).to(world.recv.device)
+        c = r.counts
+        o, n = int(c.dst_offsets[dst_rank].item()), int(c.dst_sizes[dst_rank].item())
+        blocks.append(ops.pack_payload(x, c.row_token[o:o + n].contiguous()))
+    return torch.cat(blocks) if blocks else torch.empty((0, cfg.hidden), dtype=cfg.torch_dtype, device=world.recv.device)

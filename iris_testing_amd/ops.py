@@ -120,8 +120,10 @@ def pack_fixed_m(x: torch.Tensor, row_token: torch.Tensor, dst_sizes: torch.Tens
 
 def pack_tokens(x: torch.Tensor, topk_idx: torch.Tensor, pos: torch.Tensor, dst_sizes: torch.Tensor,
                 dst_offsets: torch.Tensor, e_local: int, M: int, out: Optional[torch.Tensor] = None,
-                status: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """The send buffer of pack_fixed_m written token by token (every token row read once, stored k times)."""
+                status: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                out_gate: Optional[torch.Tensor] = None):
+    """The send buffer of pack_fixed_m written token by token (every token row read once, stored k times).
+    With ``gate`` [T,k] the slots' gates travel too: returns (send [W,M,H], send_gate [W,M] fp32, zero in the padding)."""
     _req_cuda(x, "tokens")
     _req_i32(topk_idx, "topk_idx")
     _req_i32(pos, "pos")
@@ -134,6 +136,16 @@ def pack_tokens(x: torch.Tensor, topk_idx: torch.Tensor, pos: torch.Tensor, dst_
     if out is None:
         out = torch.empty((W, M, H), dtype=x.dtype, device=x.device)
     assert out.shape == (W, M, H) and out.dtype == x.dtype and out.is_contiguous()
+    if gate is not None:
+        _req_cuda(gate, "gate")
+        assert gate.dtype == torch.float32 and gate.numel() == T * k and gate.is_contiguous()
+        if out_gate is None:
+            out_gate = torch.empty((W, M), dtype=torch.float32, device=x.device)
+        assert out_gate.shape == (W, M) and out_gate.dtype == torch.float32 and out_gate.is_contiguous()
+        L.check(L.lib().moe_pack_tokens_gated(L.ptr(x), L.dtype_code(x.dtype), T, H, L.ptr(topk_idx), L.ptr(pos), L.ptr(gate), k,
+                                              e_local, L.ptr(dst_sizes), L.ptr(dst_offsets), W, M, L.ptr(out), L.ptr(out_gate),
+                                              L.ptr(status), L.stream_ptr()))
+        return out, out_gate
     L.check(L.lib().moe_pack_tokens(L.ptr(x), L.dtype_code(x.dtype), T, H, L.ptr(topk_idx), L.ptr(pos), k, e_local,
                                     L.ptr(dst_sizes), L.ptr(dst_offsets), W, M, L.ptr(out), L.ptr(status), L.stream_ptr()))
     return out
@@ -141,7 +153,8 @@ def pack_tokens(x: torch.Tensor, topk_idx: torch.Tensor, pos: torch.Tensor, dst_
 
 def pack_tokens_fp8(x: torch.Tensor, topk_idx: torch.Tensor, pos: torch.Tensor, dst_sizes: torch.Tensor,
                     dst_offsets: torch.Tensor, e_local: int, M: int, out_q: Optional[torch.Tensor] = None,
-                    out_scale: Optional[torch.Tensor] = None, status: Optional[torch.Tensor] = None):
+                    out_scale: Optional[torch.Tensor] = None, status: Optional[torch.Tensor] = None,
+                    gate: Optional[torch.Tensor] = None, out_gate: Optional[torch.Tensor] = None):
     """pack_tokens with the per-token fp8 quantisation done on the way: ([W,M,H] uint8 codes, [W,M] fp32 scales) -- slot for
     slot what quantize_rows_fp8 makes of pack_tokens' bf16 buffer."""
     _req_cuda(x, "tokens")
@@ -158,6 +171,16 @@ def pack_tokens_fp8(x: torch.Tensor, topk_idx: torch.Tensor, pos: torch.Tensor, 
         out_scale = torch.empty((W, M), dtype=torch.float32, device=x.device)
     assert out_q.shape == (W, M, H) and out_q.dtype == torch.uint8 and out_q.is_contiguous()
     assert out_scale.shape == (W, M) and out_scale.dtype == torch.float32 and out_scale.is_contiguous()
+    if gate is not None:  # (the slots' gates travel too: a third result, [W,M] fp32, zero in the padding)
+        _req_cuda(gate, "gate")
+        assert gate.dtype == torch.float32 and gate.numel() == T * k and gate.is_contiguous()
+        if out_gate is None:
+            out_gate = torch.empty((W, M), dtype=torch.float32, device=x.device)
+        assert out_gate.shape == (W, M) and out_gate.dtype == torch.float32 and out_gate.is_contiguous()
+        L.check(L.lib().moe_pack_tokens_fp8_gated(L.ptr(x), T, H, L.ptr(topk_idx), L.ptr(pos), L.ptr(gate), k, e_local,
+                                                  L.ptr(dst_sizes), L.ptr(dst_offsets), W, M, L.ptr(out_q), L.ptr(out_scale),
+                                                  L.ptr(out_gate), L.ptr(status), L.stream_ptr()))
+        return out_q, out_scale, out_gate
     L.check(L.lib().moe_pack_tokens_fp8(L.ptr(x), T, H, L.ptr(topk_idx), L.ptr(pos), k, e_local, L.ptr(dst_sizes),
                                         L.ptr(dst_offsets), W, M, L.ptr(out_q), L.ptr(out_scale), L.ptr(status), L.stream_ptr()))
     return out_q, out_scale
@@ -431,6 +454,61 @@ def recv_row_map(recv_counts: torch.Tensor, M: int, n_rows: int, row_map: Option
     return row_map, expert_cnt
 
 
+def recv_row_map_gated(recv_counts: torch.Tensor, M: int, n_rows: int, recv_gate: Optional[torch.Tensor] = None,
+                       row_map: Optional[torch.Tensor] = None, expert_cnt: Optional[torch.Tensor] = None,
+                       row_gate: Optional[torch.Tensor] = None):
+    """recv_row_map that, given the gates that arrived with the rows (recv_gate, one per row of the receive buffer), also
+    returns them in the GEMM's row order; M == 0: the receive buffer is a padding-free flat payload (see recv_row_map_flat).
+    -> (row_map, expert_cnt, row_gate or None)."""
+    _req_i32(recv_counts, "recv_counts")
+    W, E_l = recv_counts.shape
+    dev = recv_counts.device
+    if row_map is None:
+        row_map = _i32((max(n_rows, 1),), dev)
+    if expert_cnt is None:
+        expert_cnt = _i32((E_l,), dev)
+    if recv_gate is not None:
+        _req_cuda(recv_gate, "recv_gate")
+        assert recv_gate.dtype == torch.float32 and recv_gate.is_contiguous()
+        if row_gate is None:
+            row_gate = torch.empty((max(n_rows, 1),), dtype=torch.float32, device=dev)
+    L.check(L.lib().moe_recv_row_map_gated(L.ptr(recv_counts), W, E_l, M, n_rows, L.ptr(recv_gate), L.ptr(row_map), L.ptr(row_gate),
+                                           L.ptr(expert_cnt), L.stream_ptr()))
+    return row_map, expert_cnt, row_gate
+
+
+def recv_row_map_flat(recv_counts: torch.Tensor, n_rows: int, row_map: Optional[torch.Tensor] = None,
+                      expert_cnt: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """row_map[r] = row of a padding-free flat receive payload (source-major, expert-minor blocks: what
+    reorder_flat_to_token_buf reads) holding expert-major row r, and the per-expert row counts."""
+    _req_i32(recv_counts, "recv_counts")
+    W, E_l = recv_counts.shape
+    dev = recv_counts.device
+    if row_map is None:
+        row_map = _i32((max(n_rows, 1),), dev)
+    if expert_cnt is None:
+        expert_cnt = _i32((E_l,), dev)
+    L.check(L.lib().moe_recv_row_map_flat(L.ptr(recv_counts), W, E_l, n_rows, L.ptr(row_map), L.ptr(expert_cnt), L.stream_ptr()))
+    return row_map, expert_cnt
+
+
+def grouped_gemm_mapped_gated(a_base: torch.Tensor, a_row_map: Optional[torch.Tensor], packed: torch.Tensor,
+                              expert_cnt: torch.Tensor, S_rows: int, N: int, row_gate: torch.Tensor, out: torch.Tensor,
+                              c_row_map: Optional[torch.Tensor] = None, part_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """grouped_gemm_mapped without activation whose result row r is multiplied by row_gate[r] (fp32, before the rounding)."""
+    assert a_base.dim() == 2 and out.dim() == 2 and a_base.is_contiguous() and out.is_contiguous()
+    assert a_base.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and out.shape[1] == N
+    assert row_gate.dtype == torch.float32 and row_gate.numel() >= S_rows and row_gate.is_contiguous()
+    _req_i32(expert_cnt, "expert_cnt")
+    K = a_base.shape[1]
+    L.check(L.lib().moe_grouped_gemm_mapped_gated(L.ptr(a_base), a_base.shape[0], L.ptr(a_row_map), L.ptr(packed), L.ptr(expert_cnt),
+                                                  S_rows, K, N, expert_cnt.numel(), L.ptr(row_gate), L.ptr(out), out.shape[0],
+                                                  L.ptr(c_row_map), L.ptr(part_ws),
+                                                  0 if part_ws is None else part_ws.numel() * part_ws.element_size(),
+                                                  L.stream_ptr()))
+    return out
+
+
 def grouped_gemm_mapped(a_base: torch.Tensor, a_row_map: Optional[torch.Tensor], packed: torch.Tensor,
                         expert_cnt: torch.Tensor, S_rows: int, N: int, act: str, out: torch.Tensor,
                         c_row_map: Optional[torch.Tensor] = None, part_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -488,17 +566,18 @@ def zero_padding_rows(buf: torch.Tensor, recv_counts: torch.Tensor) -> torch.Ten
     return buf
 
 
-def combine(ret: torch.Tensor, topk_idx: torch.Tensor, pos: torch.Tensor, gate: torch.Tensor,
+def combine(ret: torch.Tensor, topk_idx: torch.Tensor, pos: torch.Tensor, gate: Optional[torch.Tensor],
             dst_offsets: torch.Tensor, e_local: int, out: Optional[torch.Tensor] = None,
             status: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[t] = sum_kk gate[t,kk] * ret[slot of (t,kk)].  Slots the pack dropped (row at or past M) are skipped
-    and raise ``status`` (int32 [1], optional)."""
+    and raise ``status`` (int32 [1], optional).  gate None: the rows arrive weighted and are only added."""
     _req_cuda(ret, "ret")
     _req_i32(topk_idx, "topk_idx")
     _req_i32(pos, "pos")
     _req_i32(dst_offsets, "dst_offsets")
-    _req_cuda(gate, "gate")
-    assert gate.dtype == torch.float32
+    if gate is not None:
+        _req_cuda(gate, "gate")
+        assert gate.dtype == torch.float32
     W, M, H = ret.shape
     T, k = topk_idx.shape
     if out is None:

@@ -486,9 +486,12 @@ def expert_row_counts(pca: np.ndarray) -> np.ndarray:
 # --------------------------------------------------------------------------------------
 # a11: grouped GEMM  (reference layers/expert.py:20-43; kernels.py:240-289)
 # --------------------------------------------------------------------------------------
-def grouped_gemm(tokens: np.ndarray, weights: np.ndarray, cnt: np.ndarray, dtype: str = "f32") -> np.ndarray:
+def grouped_gemm(tokens: np.ndarray, weights: np.ndarray, cnt: np.ndarray, dtype: str = "f32",
+                 row_gate: Optional[np.ndarray] = None) -> np.ndarray:
     """out[rows of e] = tokens[rows of e] @ weights[e]; fp32 accumulate (kernels.py:265),
-    cast to the token dtype (kernels.py:276); rows of e = [sum cnt[:e], + cnt[e])."""
+    cast to the token dtype (kernels.py:276); rows of e = [sum cnt[:e], + cnt[e]).
+    row_gate [S] (not in the reference, which has no return path): every fp32 result row is multiplied by its
+    gate -- one fp32 multiplication -- before the one rounding to ``dtype``."""
     S, K = tokens.shape
     E_l, K2, N = weights.shape
     assert K == K2 and len(cnt) == E_l
@@ -500,6 +503,8 @@ def grouped_gemm(tokens: np.ndarray, weights: np.ndarray, cnt: np.ndarray, dtype
             out[r:r + c] = tokens[r:r + c].astype(np.float32) @ weights[e].astype(np.float32)
         r += c
     assert r <= S
+    if row_gate is not None:
+        out = (out * np.asarray(row_gate, dtype=np.float32)[:S, None]).astype(np.float32)
     return round_to(out, dtype)
 
 
@@ -526,8 +531,10 @@ def act_silu(x: np.ndarray) -> np.ndarray:
     return (x64 / (1.0 + np.exp(-x64))).astype(np.float32)
 
 
-def expert_mlp(tokens, cnt, w1, w2, act: str, dtype: str = "bf16", w_up=None):
+def expert_mlp(tokens, cnt, w1, w2, act: str, dtype: str = "bf16", w_up=None, row_gate=None):
     """Per-expert MLP on expert-major rows.
+
+    row_gate [S] (optional): the result rows leave weighted, round(fp32 result * gate) -- see grouped_gemm.
 
     act in {"gelu","silu"}:  y = act(x W1_e) W2_e              (w1 [E_l,H,F], w2 [E_l,F,H])
     act == "swiglu":         y = (silu(x Wg_e) * (x Wu_e)) Wd_e (w1 = Wg, w_up = Wu, w2 = Wd)
@@ -557,6 +564,8 @@ def expert_mlp(tokens, cnt, w1, w2, act: str, dtype: str = "bf16", w_up=None):
             h = round_to(h, dtype)
             y[r:r + c] = h @ w2[e].astype(np.float32)
         r += c
+    if row_gate is not None:
+        y = (y * np.asarray(row_gate, dtype=np.float32)[:S, None]).astype(np.float32)
     return round_to(y, dtype)
 
 
@@ -626,9 +635,44 @@ def return_pack(y: np.ndarray, recv_counts: np.ndarray, M: int) -> np.ndarray:
     return ret
 
 
+def pack_gates(gate: np.ndarray, idx: np.ndarray, pos: np.ndarray, dst_offsets: np.ndarray, e_local: int,
+               W: int, M: int) -> np.ndarray:
+    """send_gate[dst, m] = gate[t,kk] for the slot (dst, m) of (t,kk), zero in the padding: the gates shipped with the
+    rows of the fixed [W,M,H] layout (README.md:5-7) when the destination is to apply them.  Slots past M are dropped
+    like their rows."""
+    T, k = idx.shape
+    out = np.zeros((W, M), dtype=np.float32)
+    for t in range(T):
+        for kk in range(k):
+            d = int(idx[t, kk]) // e_local
+            if 0 <= d < W:
+                m = int(pos[t, kk]) - int(dst_offsets[d])
+                if 0 <= m < M:
+                    out[d, m] = gate[t, kk]
+    return out
+
+
+def flat_recv_row_map(recv_counts: np.ndarray) -> np.ndarray:
+    """Expert-major row r = (e, s, j) -> row of a padding-free flat receive payload laid out in source-major,
+    expert-minor blocks (what every source's send_payload holds for this rank, utils.py:235-246, concatenated in source
+    order; the layout reorder_flat_to_token_buf reads, baseline.py:204-218)."""
+    W, e_local = recv_counts.shape
+    flat_off = np.concatenate([[0], np.cumsum(recv_counts.reshape(-1).astype(np.int64))])
+    rows = []
+    for e in range(e_local):
+        for s in range(W):
+            c = int(recv_counts[s, e])
+            rows.append(flat_off[s * e_local + e] + np.arange(c, dtype=np.int64))
+    return np.concatenate(rows).astype(np.int32) if rows else np.zeros(0, np.int32)
+
+
 def combine(ret: np.ndarray, idx: np.ndarray, pos: np.ndarray, gate: np.ndarray,
-            dst_offsets: np.ndarray, e_local: int, dtype: str = "bf16") -> np.ndarray:
+            dst_offsets: np.ndarray, e_local: int, dtype: str = "bf16", pre_weighted: bool = False) -> np.ndarray:
     """out[t] = sum_kk gate[t,kk] * ret[dst, pos[t,kk] - dst_offsets[dst]],  dst = idx[t,kk] // E_l.
+
+    pre_weighted: the returned rows were multiplied by their gates where they were computed (grouped_gemm /
+    expert_mlp with row_gate: the multiplication happens in fp32 BEFORE the expert output is rounded to ``dtype``,
+    instead of after it); the combine then only adds them, fp32, ascending kk, one rounding.  ``gate`` is ignored.
 
     ret [W,M,H] is the returned buffer in the same slots the send buffer used.  fp32
     accumulate in ascending kk, one fp32 multiply and one fp32 add per term (no fused
@@ -644,6 +688,7 @@ def combine(ret: np.ndarray, idx: np.ndarray, pos: np.ndarray, gate: np.ndarray,
         m = pos[:, kk].astype(np.int64) - dst_offsets.astype(np.int64)[np.where(d_ok, d, 0)]
         have = d_ok & (m >= 0) & (m < M)
         rows = ret[np.where(have, d, 0), np.where(have, m, 0)].astype(np.float32)
-        term = (out + (gate[:, kk:kk + 1].astype(np.float32) * rows).astype(np.float32)).astype(np.float32)
+        weighted = rows if pre_weighted else (gate[:, kk:kk + 1].astype(np.float32) * rows).astype(np.float32)
+        term = (out + weighted).astype(np.float32)
         out = np.where(have[:, None], term, out)
     return round_to(out, dtype)

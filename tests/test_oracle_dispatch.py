@@ -308,3 +308,108 @@ def test_quantising_rows_commutes_with_packing_them():
             want_q[d, m], want_s[d, m] = codes_t[t], scale_t[t]
     assert np.array_equal(q, want_q) and np.array_equal(sc, want_s)
     assert (sc[0, sizes[0]:] == 1.0).all() and (q[0, sizes[0]:] == 0).all()
+
+
+def _routed(rng, T, H, E, k, W):
+    x = (rng.standard_normal((T, H)) * 4).round().astype(np.float32)
+    idx = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.int32)
+    counts = O.send_counts(idx, W, E)
+    sizes, offs = O.dst_sizes_offsets(counts)
+    pos, row_token = O.payload_positions(idx, E)
+    return x, idx, counts, sizes, offs, pos, row_token
+
+
+def test_flat_receive_row_map_against_the_reference_reorder():
+    """A padding-free receive payload (every source's send_payload block for this rank, concatenated in source order,
+    utils.py:235-246) read through flat_recv_row_map gives the expert-major rows that the reference's own route gives:
+    reorder_flat_to_token_buf (baseline.py:204-218) followed by the token shuffle; and the same rows as the fixed-M
+    route (unpack_expert_major of the [W,M,H] buffer)."""
+    rng = np.random.default_rng(21)
+    T, H, E, k, W = 60, 8, 12, 3, 4
+    E_l, dst = E // W, 1
+    flats, slots, rcs = [], [], []
+    parts = [_routed(rng, T, H, E, k, W) for _ in range(W)]
+    M = O.pair_capacity(np.stack([p[3] for p in parts]))
+    for s, (x, idx, counts, sizes, offs, pos, row_token) in enumerate(parts):
+        x += 1000.0 * s  # rows of different sources differ
+        payload = O.send_payload(x, row_token)
+        flats.append(payload[offs[dst]:offs[dst] + sizes[dst]])
+        slots.append(O.pack_fixed_m(payload, offs, sizes, M)[dst])
+        rcs.append(counts[dst])
+    flat, recv, rc = np.concatenate(flats), np.stack(slots), np.stack(rcs).astype(np.int32)
+    rm = O.flat_recv_row_map(rc)
+    assert rm.shape == (int(rc.sum()),) and sorted(rm.tolist()) == list(range(int(rc.sum())))  # a permutation
+    CAP = int(rc.max())
+    tb = O.reorder_flat_to_token_buf(flat, rc, CAP, np.empty((E_l, W, CAP, H), np.float32))
+    assert np.array_equal(flat[rm], O.shuffle(tb, rc.T))
+    assert np.array_equal(flat[rm], O.unpack_expert_major(recv, rc))
+    # brute force: row (e, s, j) of the expert-major order sits at (rows of earlier sources) + (rows of s for earlier experts) + j
+    r = 0
+    for e in range(E_l):
+        for s in range(W):
+            for j in range(rc[s, e]):
+                assert rm[r] == rc[:s].sum() + rc[s, :e].sum() + j
+                r += 1
+
+
+def test_gates_shipped_with_the_rows():
+    """pack_gates puts a slot's gate where pack_fixed_m puts its row: packing a one-column payload of gates (in payload
+    order) gives the same [W,M] array; padding slots hold zero; slots past an undersized M are dropped with their rows."""
+    rng = np.random.default_rng(22)
+    T, H, E, k, W = 50, 4, 8, 2, 4
+    x, idx, counts, sizes, offs, pos, row_token = _routed(rng, T, H, E, k, W)
+    gate = rng.random((T, k)).astype(np.float32) + 0.25
+    g_payload = np.zeros((T * k, 1), np.float32)
+    g_payload[pos.reshape(-1), 0] = gate.reshape(-1)
+    for M in (O.pair_capacity(sizes) + 2, O.pair_capacity(sizes) - 3):
+        sg = O.pack_gates(gate, idx, pos, offs, E // W, W, M)
+        assert np.array_equal(sg, O.pack_fixed_m(g_payload, offs, sizes, M, drop=True)[:, :, 0])
+        for d in range(W):
+            assert (sg[d, min(sizes[d], M):] == 0).all() and (sg[d, :min(sizes[d], M)] > 0).all()
+
+
+def test_pre_weighted_combine():
+    """Gates applied at the destination instead of the source.  In fp32 nothing is rounded between the expert output and
+    the combine, so both orders give the same bits: combine(pre_weighted) of rows multiplied by their gates ==
+    combine(gate) of the plain rows.  In bf16 the weighted rows are rounded once (round(fp32 * gate), pinned against
+    torch's bf16 cast) and the combine only adds: against a per-token evaluation."""
+    import torch
+    rng = np.random.default_rng(23)
+    T, H, E, k, W = 40, 16, 8, 3, 4
+    E_l = E // W
+    x, idx, counts, sizes, offs, pos, row_token = _routed(rng, T, H, E, k, W)
+    x = rng.standard_normal((T, H)).astype(np.float32)
+    gate = rng.random((T, k)).astype(np.float32)
+    M = O.pair_capacity(sizes) + 1
+    send = O.pack_fixed_m(O.send_payload(x, row_token), offs, sizes, M)
+    sg = O.pack_gates(gate, idx, pos, offs, E_l, W, M)
+    # identity experts: the destination returns round(row * gate)
+    cnt_all = np.array([W * M], np.int32)
+    eye = np.eye(H, dtype=np.float32)[None]
+    w32 = O.grouped_gemm(send.reshape(W * M, H), eye, cnt_all, "f32", row_gate=sg.reshape(-1)).reshape(W, M, H)
+    assert np.array_equal(w32, (send * sg[:, :, None]).astype(np.float32))
+    a = O.combine(w32, idx, pos, gate, offs, E_l, "f32", pre_weighted=True)
+    b = O.combine(send, idx, pos, gate, offs, E_l, "f32")
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    # bf16
+    xb = O.bf16_round(x)
+    sendb = O.pack_fixed_m(O.send_payload(xb, row_token), offs, sizes, M)
+    wb = O.grouped_gemm(sendb.reshape(W * M, H), eye, cnt_all, "bf16", row_gate=sg.reshape(-1)).reshape(W, M, H)
+    want_rows = torch.from_numpy((sendb * sg[:, :, None]).astype(np.float32)).bfloat16().float().numpy()
+    assert np.array_equal(wb, want_rows)
+    out = O.combine(wb, idx, pos, None, offs, E_l, "bf16", pre_weighted=True)
+    for t in range(T):
+        acc = np.zeros(H, np.float32)
+        for kk in range(k):
+            acc = (acc + torch.from_numpy((gate[t, kk] * xb[t]).astype(np.float32)).bfloat16().float().numpy()).astype(np.float32)
+        assert np.array_equal(out[t], torch.from_numpy(acc).bfloat16().float().numpy())
+    # the MLP form: expert_mlp(row_gate) is round(fp32 result * gate), i.e. within one bf16 step of gate * round(result)
+    cnt = np.array([30, 10], np.int32)
+    rows = O.bf16_round(rng.standard_normal((40, H)).astype(np.float32))
+    w1 = O.bf16_round(rng.standard_normal((2, H, 32)).astype(np.float32) * 0.25)
+    w2 = O.bf16_round(rng.standard_normal((2, 32, H)).astype(np.float32) * 0.2)
+    g = rng.random(40).astype(np.float32)
+    yw = O.expert_mlp(rows, cnt, w1, w2, "silu", "bf16", row_gate=g)
+    y = O.expert_mlp(rows, cnt, w1, w2, "silu", "bf16")
+    assert np.abs(yw - g[:, None] * y).max() <= 2.0 ** -7 * np.abs(y).max()
+    assert not np.array_equal(yw, O.bf16_round(g[:, None] * y))  # (the rounding order is a different one)
