@@ -385,9 +385,10 @@ def main():
     dom = "mlp_up"  # the gate/up grouped GEMM: most of the flops of a step
     traffic, traffic_source = profiled_traffic(cfg.name, dom + "_fp8_dispatch" if pipe.fp8_dispatch else dom)
     if cfg.quant == "fp8":
-        kname = ("moe_grouped_mlp_fp8_q (gate/up GEMM + SwiGLU + re-quantisation + down GEMM; the tokens arrive quantised)"
-                 if pipe.fp8_dispatch else
-                 "moe_grouped_mlp_fp8 (row quantisation + gate/up GEMM + SwiGLU + re-quantisation + down GEMM)")
+        kname = ("moe_grouped_mlp_fp8_q (gate/up GEMM + SwiGLU + block quantisation in its epilogue, down GEMM on block-scaled "
+                 "MFMAs; the tokens arrive quantised)" if pipe.fp8_dispatch else
+                 "moe_grouped_mlp_fp8 (row quantisation + gate/up GEMM + SwiGLU + block quantisation in its epilogue, down GEMM "
+                 "on block-scaled MFMAs)")
     elif cfg.dtype == "f32":
         kname = "moe_grouped_mlp fp32 (both GEMMs)"
     else:

@@ -210,17 +210,21 @@ int moe_grouped_mlp(const void* tokens, const int32_t* expert_cnt, int dtype, in
                     void* out, moe_stream_t stream);
 
 /* fp8 (OCP e4m3) SwiGLU expert.  Weights: e4m3 codes pre-packed like the bf16 ones (1 byte per
- * element) with per-output-channel fp32 scales (sg, su [E_l,F]; sd [E_l,H]).  Activations
- * (bf16) are quantised per row inside: xq_ws [S_rows,H] u8, xs_ws [S_rows] f32, h_ws [S_rows,F]
- * bf16, hq_ws [S_rows,F] u8, hs_ws [S_rows] f32. */
+ * element) with per-output-channel fp32 scales (sg, su [E_l,F]; sd [E_l,H]).  The input rows (bf16) are quantised per
+ * row inside (scale amax/448): xq_ws [S_rows,H] u8, xs_ws [S_rows] f32.  The hidden activation silu(g) * u is
+ * quantised by the first GEMM's epilogue, from its fp32 values, in blocks of one row x 32 columns: scale 2^(b-127), the
+ * smallest power of two under which the block's largest magnitude is at most 448, codes = e4m3(value / scale):
+ * hq_ws [S_rows,F] u8 and hscale_ws [S_rows, F/32] u8 (the bytes b).  The down projection multiplies the codes with
+ * the scales applied inside the matrix instruction; epilogue acc * s_ch[n] (* row_gate[m] where given).  H and F
+ * multiples of 128. */
 int moe_prepack_weights_fp8(const uint8_t* w, const uint8_t* w_up, int E_l, int K, int N, uint8_t* packed,
                             moe_stream_t stream);
 int moe_quantize_rows_fp8(const void* x_bf16, int rows, int cols, uint8_t* q, float* scale,
                           const int32_t* n_rows_dev, moe_stream_t stream);
 int moe_grouped_mlp_fp8(const void* tokens_bf16, const int32_t* expert_cnt, int S_rows, int H, int F, int E_l,
                         const uint8_t* wgu_packed, const float* sg, const float* su, const uint8_t* wd_packed,
-                        const float* sd, uint8_t* xq_ws, float* xs_ws, void* h_ws, uint8_t* hq_ws, float* hs_ws,
-                        void* out, moe_stream_t stream);
+                        const float* sd, uint8_t* xq_ws, float* xs_ws, uint8_t* hq_ws, uint8_t* hscale_ws, void* out,
+                        moe_stream_t stream);
 
 /* ---- a10 + a11/a12 + a13 without the two row copies ------------------------------------------------
  * The expert-major unpack (token_shuffle.py:31-56) and the return pack only move rows; the grouped GEMM
@@ -284,14 +288,15 @@ int moe_shuffle_backward(const void* grad_rows, int dtype, int E_l, int W, int C
                          void* grad_token_buf, int32_t* map_ws, moe_stream_t stream);
 /* moe_grouped_mlp_fp8 with the same row indirection: the row quantisation reads input row r from row
  * a_row_map[r] of a_base_bf16 (a_rows rows of H), the down GEMM writes result row r to row c_row_map[r]
- * of out (out_rows rows of H); either map may be NULL.  part_ws (nullable): the K-split scratch of
- * moe_grouped_gemm_mapped, used by both GEMMs in turn. */
+ * of out (out_rows rows of H); either map may be NULL.  row_gate (nullable, fp32 [S_rows], as moe_recv_row_map_gated
+ * returns it): result row r is multiplied by row_gate[r] before the one rounding (the gated return).  part_ws
+ * (nullable): the K-split scratch of moe_grouped_gemm_mapped, used by both GEMMs in turn. */
 int moe_grouped_mlp_fp8_mapped(const void* a_base_bf16, int a_rows, const int32_t* a_row_map,
                                const int32_t* expert_cnt, int S_rows, int H, int F, int E_l,
                                const uint8_t* wgu_packed, const float* sg, const float* su, const uint8_t* wd_packed,
-                               const float* sd, uint8_t* xq_ws, float* xs_ws, void* h_ws, uint8_t* hq_ws, float* hs_ws,
-                               void* out, int out_rows, const int32_t* c_row_map, void* part_ws, size_t part_ws_bytes,
-                               moe_stream_t stream);
+                               const float* sd, uint8_t* xq_ws, float* xs_ws, uint8_t* hq_ws, uint8_t* hscale_ws,
+                               const float* row_gate, void* out, int out_rows, const int32_t* c_row_map, void* part_ws,
+                               size_t part_ws_bytes, moe_stream_t stream);
 
 /* moe_grouped_mlp_fp8_mapped for rows that arrive quantised (moe_pack_tokens_fp8): a_q [a_rows,H] codes and a_scale
  * [a_rows] scales, gathered through a_row_map (nullable) by the first GEMM as it loads them; xs_ws [S_rows] receives the
@@ -300,7 +305,7 @@ int moe_grouped_mlp_fp8_mapped(const void* a_base_bf16, int a_rows, const int32_
 int moe_grouped_mlp_fp8_q_mapped(const uint8_t* a_q, const float* a_scale, int a_rows, const int32_t* a_row_map,
                                  const int32_t* expert_cnt, int S_rows, int H, int F, int E_l, const uint8_t* wgu_packed,
                                  const float* sg, const float* su, const uint8_t* wd_packed, const float* sd, float* xs_ws,
-                                 void* h_ws, uint8_t* hq_ws, float* hs_ws, void* out, int out_rows,
+                                 uint8_t* hq_ws, uint8_t* hscale_ws, const float* row_gate, void* out, int out_rows,
                                  const int32_t* c_row_map, void* part_ws, size_t part_ws_bytes, moe_stream_t stream);
 
 /* ---- gradients (every backward of the reference is an empty stub: layers/expert.py:62-64,

@@ -61,13 +61,13 @@ _SIGNATURES = {
     "moe_grouped_mlp": (c_int, [P, P, c_int, c_int, c_int, c_int, c_int, c_int, P, P, P, P, P, P]),
     "moe_prepack_weights_fp8": (c_int, [P, P, c_int, c_int, c_int, P, P]),
     "moe_quantize_rows_fp8": (c_int, [P, c_int, c_int, P, P, P, P]),
-    "moe_grouped_mlp_fp8": (c_int, [P, P, c_int, c_int, c_int, c_int, P, P, P, P, P, P, P, P, P, P, P, P]),
+    "moe_grouped_mlp_fp8": (c_int, [P, P, c_int, c_int, c_int, c_int, P, P, P, P, P, P, P, P, P, P, P]),
     "moe_return_pack": (c_int, [P, c_int, c_int, c_int, P, c_int, c_int, c_int, P, P, P]),
     "moe_recv_row_map": (c_int, [P, c_int, c_int, c_int, c_int, P, P, P, P]),
     "moe_grouped_gemm_mapped": (c_int, [P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P, c_int, P, P, c_size_t, P]),
     "moe_pack_tokens_fp8": (c_int, [P, c_int, c_int, P, P, c_int, c_int, P, P, c_int, c_int, P, P, P, P]),
     "moe_grouped_mlp_fp8_q_mapped": (c_int, [P, P, c_int, P, P, c_int, c_int, c_int, c_int, P, P, P, P, P, P, P, P, P, P, c_int,
-                                             P, P, c_size_t, P]),
+                                             P, P, c_size_t, P]),  # (.., xs_ws, hq_ws, hscale_ws, row_gate, out, out_rows, ..)
     "moe_grouped_gemm_act_keep": (c_int, [P, c_int, P, P, P, c_int, c_int, c_int, c_int, c_int, P, P, P, c_size_t, P]),
     "moe_gemm_part_workspace_bytes": (c_size_t, []),
     "moe_prepack_weights_transposed": (c_int, [P, P, c_int, c_int, c_int, c_int, P, P]),
@@ -79,7 +79,7 @@ _SIGNATURES = {
     "moe_gemm_split_plan": (c_int, [c_int, c_int, c_int, c_int, P]),
     "moe_zero_padding_rows": (c_int, [P, c_int, c_int, c_int, c_int, P, c_int, P]),
     "moe_grouped_mlp_fp8_mapped": (c_int, [P, c_int, P, P, c_int, c_int, c_int, c_int, P, P, P, P, P, P, P, P, P, P, P, c_int, P, P,
-                                           c_size_t, P]),
+                                           c_size_t, P]),  # (.., xq_ws, xs_ws, hq_ws, hscale_ws, row_gate, out, out_rows, ..)
     "moe_combine": (c_int, [P, c_int, c_int, c_int, c_int, P, P, P, P, c_int, c_int, c_int, P, P, P]),
 }
 

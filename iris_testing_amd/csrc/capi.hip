@@ -19,6 +19,6 @@ int moe_check_launch(const char* what) {
     return MOE_OK;
 }
 
-extern "C" int moe_abi_version(void) { return 2; }
+extern "C" int moe_abi_version(void) { return 3; }
 
 extern "C" const char* moe_last_error(void) { return g_err; }

@@ -42,6 +42,10 @@ constexpr int GG_BN = 256;
                       // waves of 128 x 128; the same shape costs bf16 5 %)
 #endif
 
+#ifndef GG_FP8_BSA_NWM
+#define GG_FP8_BSA_NWM 4  // the fp8 down projection (block-scaled activations): waves along M, as for the other fp8 GEMM
+#endif
+
 struct GemmParams {
     const uint8_t* A;         // [S_rows, K] activations (bf16 or fp8)
     const uint8_t* B;         // packed weights [E_l, Npad, K]
@@ -52,6 +56,12 @@ struct GemmParams {
     const float* row_scale;   // fp8: [S_rows] per-row activation scale; bf16 with EPI_GATE: [S_rows] per-row gate
     const float* col_scale;   // fp8: [E_l, ncs] per-output-channel scale (gate for SwiGLU)
     const float* col_scale2;  // fp8 SwiGLU: [E_l, ncs] up scales
+    // fp8, block-scaled hidden activation (one power-of-two scale, an E8M0 exponent byte, per row and 32 columns; bs_pitch
+    // bytes per row): written beside the codes by the gate/up kernel's epilogue (c_bscale, rows as C's), read by the down
+    // kernel as the scale operand of its MFMAs (a_bscale, rows as A's).
+    uint8_t* c_bscale;
+    const uint8_t* a_bscale;
+    int bs_pitch;
     const int32_t* a_map;     // optional: logical row -> row of A (gather while loading), else A is row r itself
     const int32_t* c_map;     // optional: logical row -> row of C (scatter while storing)
     int E_l, K, N, Npad, ldc, S_rows, ncs;
@@ -159,6 +169,52 @@ __device__ __forceinline__ void mma_fp8_k64(floatx16& acc, const uint4& a_lo, co
         acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc, 0, 0, 0, 0, 0, 0);
     }
 }
+
+// The same MFMA with block scales on the activation operand (the instruction's B: the kernels multiply transposed, weights
+// as A).  For row r of the operand and block b of 32 k (b = 0: the first four registers of the lanes 0-31 and 32-63, i.e. k
+// 0-15 and 16-31 of the step; b = 1: the other four registers), the scale is the E8M0 byte OPSEL of the scale register of
+// lane 32 b + r (established with a one-wave probe on the chip); the weight operand takes 2^0 everywhere.
+constexpr int GG_WSCALE = 64;
+// ASMV: the instruction written out, accumulator in ordinary vector registers (the layout of eight waves per workgroup,
+// where a wave's 256 registers hold accumulators and fragments alike).  Through the builtin, the compiler moves the scaled
+// MFMAs of that layout across the scheduling fences that pin the K loop, bunches them, and spills accumulators and
+// fragments inside the loop; a volatile asm statement stays where it is written.  The compiler does not know that the
+// statement is an MFMA: what it would insert between such an instruction and a dependent one is added by hand where the
+// accumulators are next read (GG_MFMA_SETTLE).
+template <bool Z, int OPSEL, bool ASMV = false>
+__device__ __forceinline__ void mma_fp8_k64_bs(floatx16& acc, const uint4& a_lo, const uint4& a_hi, const uint4& b_lo, const uint4& b_hi,
+                                               int scale_b) {
+    const gg_i32x8 a = {(int)a_lo.x, (int)a_lo.y, (int)a_lo.z, (int)a_lo.w, (int)a_hi.x, (int)a_hi.y, (int)a_hi.z, (int)a_hi.w};
+    const gg_i32x8 b = {(int)b_lo.x, (int)b_lo.y, (int)b_lo.z, (int)b_lo.w, (int)b_hi.x, (int)b_hi.y, (int)b_hi.z, (int)b_hi.w};
+    if constexpr (ASMV) {
+        static_assert(!Z, "the written-out form accumulates");
+        const int wsc = GG_WSCALE;
+        if constexpr (OPSEL == 0)
+            asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0]" : "+v"(acc) : "v"(a), "v"(b), "v"(wsc), "v"(scale_b));
+        else
+            asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,1,0]" : "+v"(acc) : "v"(a), "v"(b), "v"(wsc), "v"(scale_b));
+        return;
+    }
+    // (the weight operand's scale byte is GG_WSCALE = 64, a constant the instruction can take without a register; the
+    // activation side adds the 63 that are missing to 2^0 to its own bytes: the product of the two scales is what counts)
+    if constexpr (Z) {
+        const floatx16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, z, 0, 0, 0, GG_WSCALE, OPSEL, scale_b);
+    } else {
+        acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc, 0, 0, 0, GG_WSCALE, OPSEL, scale_b);
+    }
+}
+
+// Block scale of the fp8 hidden activation: the smallest power of two X = 2^(byte - 127) with amax / X <= 448 (the largest
+// e4m3 value), from the bits of amax >= 0: amax = m 2^p, 1 <= m < 2, fits when p - e < 8, or p - e = 8 and m <= 1.75 -- so
+// byte = p + 127 - 8, one more when the mantissa exceeds that of 1.75; never below 0 (amax = 0, or tiny).  Integer work:
+// the CPU checker computes the same byte from the same bits.
+__host__ __device__ inline int gg_block_scale_byte(uint32_t amax_bits) {
+    const int b = (int)((amax_bits + 0x1fffffu) >> 23) - 8;
+    return b < 0 ? 0 : b;
+}
+// 1 / X as a float: 2^(127 - byte), exact (byte <= 247 for finite amax)
+__host__ __device__ inline uint32_t gg_block_inv_bits(int byte) { return (uint32_t)(254 - byte) << 23; }
 
 __device__ __forceinline__ int seg_of(const int* off, int n, int r) {
     int lo = 0, hi = n;
@@ -339,10 +395,14 @@ __device__ __forceinline__ void gg_wait() {
 // blocks of MFMA work to land.
 // SPLIT = false: the launch that takes whole tiles.  SPLIT = true: the launch that takes the tiles of an
 // under-filled last round in parts of the K range and leaves fp32 partial sums in the workspace (GemmParams).
-template <int BM, int NWM, int EPI, bool FP8, bool SPLIT, bool DW = false>
+// BSA: the activation operand carries block scales (fp8 down projection: GemmParams::a_bscale), applied by the MFMAs.
+template <int BM, int NWM, int EPI, bool FP8, bool SPLIT, bool DW = false, bool BSA = false>
 __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const GemmParams p) {
     static_assert(!DW || (!SPLIT && !FP8 && EPI == EPI_NONE), "the weight-gradient mode is a plain bf16 GEMM");
+    static_assert(!BSA || FP8, "block scales belong to the fp8 MFMA");
     constexpr bool VARK = SPLIT || DW;  // the K range differs from tile to tile
+    constexpr bool PEEL = !VARK && !BSA;  // the tile's first two blocks written out apart (see below)
+    constexpr bool QOUT = FP8 && EPI == EPI_SWIGLU && !SPLIT;  // the epilogue stores e4m3 codes and block scales
     constexpr int BN = GG_BN;
     constexpr int ES = FP8 ? 1 : 2;
     constexpr int NW = NWM * 2;                        // waves per workgroup
@@ -381,6 +441,9 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     __shared__ __align__(16) float s_col_scale[2][BN];
     __shared__ int s_crow[2][BM];
     __shared__ int s_amap[BM];              // the NEXT tile's input rows (a_map), fetched while this one is multiplied
+    // BSA: the block-scale bytes of the tile's rows for a PAIR of K stages (4 blocks of 32 k = one dword per row), two
+    // copies: pairs alternate like the ring slots they travel with
+    __shared__ uint32_t s_hsc[BSA ? 2 : 1][BSA ? BM : 1];
     __shared__ __align__(16) int4 s_tiles[GG_TT];
     static_assert(BM <= NWM * 2 * WAVE && BN <= NWM * 2 * WAVE, "one thread per tile row and per tile column");
 
@@ -432,8 +495,11 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     const int lchunk = (lane & 3) ^ ((lane >> 4) & 3);   // global 16-byte chunk this lane fetches
     const int fswz = (lane >> 2) & 3;                    // swizzle of the fragment row (tile rows start at multiples of 16)
     // first 16-byte chunk of the lane's fragment: bf16 lanes 16q .. 16q+15 take chunk q of rows 0 .. 15;
-    // fp8 lanes 32h .. 32h+31 take chunks 2h, 2h+1 of rows 0 .. 31
-    const int fpos = (FP8 ? 2 * (lane >> 5) : (lane >> 4)) ^ fswz;
+    // fp8 lanes 32h .. 32h+31 take chunks h and h + 2 of rows 0 .. 31 (both operands alike, so every k meets its partner):
+    // the MFMA's first four operand registers of the two lane halves are then bytes 0-31 of the stage and the other four
+    // bytes 32-63 -- the two blocks of 32 k that the scaled form of the instruction scales separately
+    constexpr int FSTEP = FP8 ? 2 : 1;  // distance of a lane's second chunk
+    const int fpos = (FP8 ? (lane >> 5) : (lane >> 4)) ^ fswz;
     const uint4* fa = sA + (wm * (BM / NWM) + (lane & (MT - 1))) * CHUNKS;
     const uint4* fb = sB + (wn * (BN / 2) + (lane & (MT - 1))) * CHUNKS;
     const uint32_t la0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(sA + wave * WROWS * CHUNKS));
@@ -487,10 +553,45 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
     // what a tile has in flight before its first MFMA: its first four stages, one per ring slot
 #define GG_PROLOGUE(Ab_, Bb_, aoff_, nks_)                    \
     do {                                                      \
+        GG_SC_DMA(0, nks_, 0);                                \
         GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 0, 0, 0, LPS, nks_);  \
         GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 1, 1, 0, LPS, nks_);  \
+        GG_SC_DMA(2, nks_, 2);                                \
         GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 2, 2, 0, LPS, nks_);  \
         GG_ISSUE_RANGE(Ab_, Bb_, aoff_, 3, 3, 0, LPS, nks_);  \
+    } while (0)
+
+    // BSA: the block-scale bytes travel with the stages.  One dword per tile row holds the four scale bytes of a PAIR of
+    // stages (2 x 64 bytes of K = 4 blocks of 32); it is requested, one per thread, straight into LDS with the loads of the
+    // pair's even stage (same block, same ring slot: copy slot / 2), and read back by the lanes one block before the pair's
+    // first MFMA.  sc_row0 / sc_rv / sc_ks0 describe the tile the loads currently point at (switched with Ab / Bb).
+    [[maybe_unused]] int sc_row0 = 0, sc_rv = 1, sc_ks0 = 0;
+    [[maybe_unused]] int sc[TM];
+#define GG_SC_DMA(st, nks_, slot)                                                                                          \
+    do {                                                                                                                   \
+        if constexpr (BSA) {                                                                                               \
+            if (wave_s * WAVE < BM) {                                                                                      \
+                const int stc_ = min((st), (nks_) - 1);                                                                    \
+                const int tid_c = wave_s * WAVE + gg_lane_now();                                                           \
+                const uint32_t vo_ = (uint32_t)(sc_row0 + min(tid_c, sc_rv - 1)) * (uint32_t)p.bs_pitch +                  \
+                                     (uint32_t)(((sc_ks0 + stc_) >> 1) << 2);                                              \
+                gg_dma4(gg_uniform(p.a_bscale), vo_,                                                                       \
+                        __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(&s_hsc[(slot) >> 1][wave_s * WAVE]))); \
+            }                                                                                                              \
+        }                                                                                                                  \
+    } while (0)
+    // lane 32 h + r of a wave takes, for each of its row tiles, the dword of row r shifted so that byte 0 is the scale of
+    // block h of the pair's even stage and byte 2 that of its odd stage (the MFMA's op_sel picks 0 or 2), each raised by
+    // what the weight operand's constant scale byte lacks to 2^0.  One set of registers: a pair's dwords are read behind the
+    // last MFMA of the pair before.
+#define GG_SC_READ(SET_)                                                                                                   \
+    do {                                                                                                                   \
+        if constexpr (BSA) {                                                                                               \
+            const int lnr_ = gg_lane_now();                                                                                \
+            _Pragma("unroll") for (int i_ = 0; i_ < TM; ++i_)                                                               \
+                sc[i_] = (int)(((s_hsc[SET_][(wave_s >> 1) * (BM / NWM) + i_ * MT + (lnr_ & 31)] >> ((lnr_ >> 5) * 8)) & 0x00ff00ffu) + \
+                               (uint32_t)(127 - GG_WSCALE) * 0x00010001u);                                                 \
+        }                                                                                                                  \
     } while (0)
 
     int round = 0, round0 = 0;
@@ -505,6 +606,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         Bb = Bb0;
 #pragma unroll
         for (int r = 0; r < RA; ++r) a_off[r] = a_off0[r];
+        sc_row0 = cur.row0; sc_rv = cur.rv; sc_ks0 = cur.ks0;
         GG_PROLOGUE(Ab, Bb, a_off, (VARK ? cur.nks : nk));
     }
     // The ring runs on from one tile into the next: the last four blocks of a tile refill their slots with the first
@@ -523,7 +625,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 
         typedef typename std::conditional<FP8, floatx16, floatx4>::type acc_t;
         acc_t acc[TM][TN];  // (not cleared where the MFMAs of the tile's first block start the sums)
-        if constexpr (VARK) {
+        if constexpr (!PEEL) {
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -545,15 +647,16 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 #define GG_RD(R, NA_, NB_)                                                                               \
     do {                                                                                                 \
         constexpr int ro_ = (R) / CF, rh_ = (R) % CF;                                                    \
-        if constexpr (ro_ < TM) NA_[ro_ * CF + rh_] = nfa_[ro_ * MT * CHUNKS + (fpos ^ rh_)];            \
-        else NB_[(ro_ - TM) * CF + rh_] = nfb_[(ro_ - TM) * MT * CHUNKS + (fpos ^ rh_)];                 \
+        if constexpr (ro_ < TM) NA_[ro_ * CF + rh_] = nfa_[ro_ * MT * CHUNKS + (fpos ^ (rh_ * FSTEP))];  \
+        else NB_[(ro_ - TM) * CF + rh_] = nfb_[(ro_ - TM) * MT * CHUNKS + (fpos ^ (rh_ * FSTEP))];       \
     } while (0)
-#define GG_ML(I, FA_, FB_, NA_, NB_, slot, Z_)                                                             \
+#define GG_ML(I, FA_, FB_, NA_, NB_, slot, Z_, EVEN_, SET_)                                                \
     do {                                                                                                 \
         if constexpr ((I) < NT) {                                                                        \
             /* boustrophedon over the wave's MFMA tiles: every instruction keeps one operand of the one before it */ \
             constexpr int pa_ = (I) / TN, pb_ = (pa_ & 1) ? TN - 1 - (I) % TN : (I) % TN;                \
-            if constexpr (FP8) mma_fp8_k64<Z_>(acc[pa_][pb_], FB_[2 * pb_], FB_[2 * pb_ + 1], FA_[2 * pa_], FA_[2 * pa_ + 1]); \
+            if constexpr (FP8 && BSA) mma_fp8_k64_bs<Z_, (EVEN_) ? 0 : 2, NWM == 4>(acc[pa_][pb_], FB_[2 * pb_], FB_[2 * pb_ + 1], FA_[2 * pa_], FA_[2 * pa_ + 1], sc[pa_]); \
+            else if constexpr (FP8) mma_fp8_k64<Z_>(acc[pa_][pb_], FB_[2 * pb_], FB_[2 * pb_ + 1], FA_[2 * pa_], FA_[2 * pa_ + 1]); \
             else mma_bf16_k32<Z_>(acc[pa_][pb_], FB_[pb_], FA_[pa_]);                                    \
             __builtin_amdgcn_sched_barrier(0);                                                           \
             constexpr int ld_ = (I) >= LFIRST && ((I) - LFIRST) % LSTEP == 0 ? ((I) - LFIRST) / LSTEP : LPS;  /* load behind this MFMA */ \
@@ -564,12 +667,13 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             __builtin_amdgcn_sched_barrier(0);                                                           \
         }                                                                                                \
     } while (0)
-#define GG_ML8(I, FA_, FB_, NA_, NB_, slot, Z_)                                                          \
-    GG_ML((I) + 0, FA_, FB_, NA_, NB_, slot, Z_); GG_ML((I) + 1, FA_, FB_, NA_, NB_, slot, Z_);           \
-    GG_ML((I) + 2, FA_, FB_, NA_, NB_, slot, Z_); GG_ML((I) + 3, FA_, FB_, NA_, NB_, slot, Z_);           \
-    GG_ML((I) + 4, FA_, FB_, NA_, NB_, slot, Z_); GG_ML((I) + 5, FA_, FB_, NA_, NB_, slot, Z_);           \
-    GG_ML((I) + 6, FA_, FB_, NA_, NB_, slot, Z_); GG_ML((I) + 7, FA_, FB_, NA_, NB_, slot, Z_)
-#define GG_STAGE(FA_, FB_, NA_, NB_, SL, EVEN_, s, last, Z_)                                                      \
+#define GG_ML8(I, FA_, FB_, NA_, NB_, slot, Z_, E_, S_)                                                          \
+    GG_ML((I) + 0, FA_, FB_, NA_, NB_, slot, Z_, E_, S_); GG_ML((I) + 1, FA_, FB_, NA_, NB_, slot, Z_, E_, S_);           \
+    GG_ML((I) + 2, FA_, FB_, NA_, NB_, slot, Z_, E_, S_); GG_ML((I) + 3, FA_, FB_, NA_, NB_, slot, Z_, E_, S_);           \
+    GG_ML((I) + 4, FA_, FB_, NA_, NB_, slot, Z_, E_, S_); GG_ML((I) + 5, FA_, FB_, NA_, NB_, slot, Z_, E_, S_);           \
+    GG_ML((I) + 6, FA_, FB_, NA_, NB_, slot, Z_, E_, S_); GG_ML((I) + 7, FA_, FB_, NA_, NB_, slot, Z_, E_, S_)
+    // SET_: which copy of the block scales (BSA) the stage's pair uses: slot / 2, as a literal (0 where the slot is a run-time value: no BSA there)
+#define GG_STAGE(FA_, FB_, NA_, NB_, SL, EVEN_, s, last, Z_, SET_)                                                \
     do {                                                                                                 \
         if constexpr (EVEN_) { /* (a block in an even slot) */                                           \
             /* from block nks - 4 on the loads fetch the next tile, if it is at hand; not in a tile's first block: the  \
@@ -584,17 +688,24 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                     kbase = nks;                                                                         \
                     nks_ld = VARK ? pk_.nks : nk;                                                        \
                     seam = true;                                                                         \
+                    sc_row0 = pk_.row0; sc_rv = pk_.rv; sc_ks0 = pk_.ks0;                                \
                 }                                                                                        \
             }                                                                                            \
+            /* (the scale dwords of the pair whose even stage this block requests) */                   \
+            GG_SC_DMA((s) + 4 - kbase, nks_ld, SET_ * 2);                                                \
         }                                                                                                \
         GG_STAGE_PTRS(Ab, Bb, (s) + 4 - kbase, ap_, bp_, nks_ld)                                         \
         const uint4* nfa_ = fa + (((SL) + 1) & 3) * ASLOT;                                               \
         const uint4* nfb_ = fb + (((SL) + 1) & 3) * BSLOT;                                               \
+        /* (written-out MFMAs: two wait states between the vector instructions above and an MFMA that reads their results) */ \
+        if constexpr (BSA && NWM == 4) asm volatile("s_nop 1");                                          \
         __builtin_amdgcn_sched_barrier(0);                                                               \
-        GG_ML8(0, FA_, FB_, NA_, NB_, SL, Z_); GG_ML8(8, FA_, FB_, NA_, NB_, SL, Z_);                     \
-        GG_ML8(16, FA_, FB_, NA_, NB_, SL, Z_); GG_ML8(24, FA_, FB_, NA_, NB_, SL, Z_);                   \
-        GG_ML8(32, FA_, FB_, NA_, NB_, SL, Z_); GG_ML8(40, FA_, FB_, NA_, NB_, SL, Z_);                   \
-        GG_ML8(48, FA_, FB_, NA_, NB_, SL, Z_); GG_ML8(56, FA_, FB_, NA_, NB_, SL, Z_);                   \
+        GG_ML8(0, FA_, FB_, NA_, NB_, SL, Z_, EVEN_, SET_); GG_ML8(8, FA_, FB_, NA_, NB_, SL, Z_, EVEN_, SET_);   \
+        GG_ML8(16, FA_, FB_, NA_, NB_, SL, Z_, EVEN_, SET_); GG_ML8(24, FA_, FB_, NA_, NB_, SL, Z_, EVEN_, SET_); \
+        GG_ML8(32, FA_, FB_, NA_, NB_, SL, Z_, EVEN_, SET_); GG_ML8(40, FA_, FB_, NA_, NB_, SL, Z_, EVEN_, SET_); \
+        GG_ML8(48, FA_, FB_, NA_, NB_, SL, Z_, EVEN_, SET_); GG_ML8(56, FA_, FB_, NA_, NB_, SL, Z_, EVEN_, SET_); \
+        /* an odd block ends a pair: the next pair's scale dwords, from the other copy, behind its last MFMA */ \
+        if constexpr (!(EVEN_)) GG_SC_READ(1 - SET_);                                                    \
         if (!(last) || seam) { /* (the last block hands over too when the next tile's stages are behind it) */ \
             gg_wait<2 * LPS, 0>();                                                                       \
             __builtin_amdgcn_s_barrier();                                                                \
@@ -628,7 +739,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                 const int lane_t = gg_lane_now(), tid_t = wave_s * WAVE + lane_t;  // (a fresh lane id: nothing kept live for this)
                 const uint32_t t4 = (uint32_t)min(tid_t, rv - 1) * 4u;
                 if (wave_s * WAVE < BM) {
-                    if constexpr (FP8 || EPI == EPI_GATE)
+                    if ((FP8 || EPI == EPI_GATE) && (!BSA || p.row_scale))  // (BSA: the rows carry no scale of their own; a gate, if any)
                         gg_dma4(gg_uniform((const uint8_t*)(p.row_scale + row0)), t4,
                                 __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)(s_row_scale[tpar] + wave_s * WAVE)));
                     if (p.c_map)
@@ -651,35 +762,36 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
-                    for (int h = 0; h < CF; ++h) fA0[i * CF + h] = fa0[i * MT * CHUNKS + (fpos ^ h)];
+                    for (int h = 0; h < CF; ++h) fA0[i * CF + h] = fa0[i * MT * CHUNKS + (fpos ^ (h * FSTEP))];
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
 #pragma unroll
-                    for (int h = 0; h < CF; ++h) fB0[j * CF + h] = fb0[j * MT * CHUNKS + (fpos ^ h)];
+                    for (int h = 0; h < CF; ++h) fB0[j * CF + h] = fb0[j * MT * CHUNKS + (fpos ^ (h * FSTEP))];
+                GG_SC_READ(0);  // (a tile that starts here starts in slot 0)
                 // the first slot is refilled from the first block on: every wave must hold its stage-0 fragments first
                 gg_wait<63, 0>();
                 __syncthreads();
             }
             // The blocks are written out for the slots 0 .. 3; a tile whose first stage lies in slot 2 (phi = 2: the
             // tiles before it left the ring there) enters at the third.  nk >= 2 and even.
-            if constexpr (!VARK) {
+            if constexpr (PEEL) {
                 // The tile's first two blocks are written out apart, with the slot as a run-time value: the MFMAs of the
                 // very first start the sums (constant zero as their C operand), so that no accumulator has to be cleared
                 // between two tiles.  (Not where the stage count varies from tile to tile: the register allocation of
                 // those instantiations does not survive it.)
                 const int phi_s = __builtin_amdgcn_readfirstlane(phi);
-                GG_STAGE(fA0, fB0, fA1, fB1, phi_s, true, 0, false, true);
-                GG_STAGE(fA1, fB1, fA0, fB0, phi_s + 1, false, 1, 2 >= nks, false);
+                GG_STAGE(fA0, fB0, fA1, fB1, phi_s, true, 0, false, true, 0);
+                GG_STAGE(fA1, fB1, fA0, fB0, phi_s + 1, false, 1, 2 >= nks, false, 0);
                 int ks = phi_s ? 2 : 0;             // phi = 0: on with the slots 2, 3 (the first half of the loop body is
                 const int kmin = phi_s ? 2 : 4;     // skipped once); phi = 2: with the slots 0, 1
                 while (ks < nks) {
                     if (ks >= kmin) {
-                        GG_STAGE(fA0, fB0, fA1, fB1, 0, true, ks, false, false);
-                        GG_STAGE(fA1, fB1, fA0, fB0, 1, false, ks + 1, ks + 2 >= nks, false);
+                        GG_STAGE(fA0, fB0, fA1, fB1, 0, true, ks, false, false, 0);
+                        GG_STAGE(fA1, fB1, fA0, fB0, 1, false, ks + 1, ks + 2 >= nks, false, 0);
                     }
                     if (ks + 2 < nks) {
-                        GG_STAGE(fA0, fB0, fA1, fB1, 2, true, ks + 2, false, false);
-                        GG_STAGE(fA1, fB1, fA0, fB0, 3, false, ks + 3, ks + 4 >= nks, false);
+                        GG_STAGE(fA0, fB0, fA1, fB1, 2, true, ks + 2, false, false, 1);
+                        GG_STAGE(fA1, fB1, fA0, fB0, 3, false, ks + 3, ks + 4 >= nks, false, 1);
                     }
                     ks += 4;
                 }
@@ -687,12 +799,12 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                 int ks = -phi;
                 do {
                     if (ks >= 0) {
-                        GG_STAGE(fA0, fB0, fA1, fB1, 0, true, ks, false, false);
-                        GG_STAGE(fA1, fB1, fA0, fB0, 1, false, ks + 1, ks + 2 >= nks, false);
+                        GG_STAGE(fA0, fB0, fA1, fB1, 0, true, ks, false, false, 0);
+                        GG_STAGE(fA1, fB1, fA0, fB0, 1, false, ks + 1, ks + 2 >= nks, false, 0);
                     }
                     if (ks + 2 < nks) {
-                        GG_STAGE(fA0, fB0, fA1, fB1, 2, true, ks + 2, false, false);
-                        GG_STAGE(fA1, fB1, fA0, fB0, 3, false, ks + 3, ks + 4 >= nks, false);
+                        GG_STAGE(fA0, fB0, fA1, fB1, 2, true, ks + 2, false, false, 1);
+                        GG_STAGE(fA1, fB1, fA0, fB0, 3, false, ks + 3, ks + 4 >= nks, false, 1);
                     }
                     ks += 4;
                 } while (ks < nks);
@@ -703,6 +815,11 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 #undef GG_ML
 #undef GG_RD
 
+        if constexpr (BSA && NWM == 4) {
+            // the last MFMAs of the tile were written out as asm (see mma_fp8_k64_bs): the wait states the compiler would put
+            // between an MFMA and the first read of its result by another kind of instruction (18 for this shape)
+            asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
+        }
         // ---- next tile: decode it and request its first stages now (every slot is free once all waves
         // have passed the barrier: the last fragments of this tile are already in registers)
         // (when the K loop has switched over, the walk only confirms what the look-ahead saw)
@@ -713,6 +830,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             Bb = Bb_n;
 #pragma unroll
             for (int r = 0; r < RA; ++r) a_off[r] = a_off_n[r];
+            sc_row0 = nxt.row0; sc_rv = nxt.rv; sc_ks0 = nxt.ks0;
             __syncthreads();
             GG_PROLOGUE(Ab, Bb, a_off, (VARK ? nxt.nks : nk));
         }
@@ -769,23 +887,27 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             gg_wait<0, 15>();
             __syncthreads();
         }
-        // fp8: a lane stores to TWO rows of a row tile (its accumulators change lanes first, below); bf16: to its own
-        constexpr int NR = FP8 ? 2 : 1;
+        // fp8 with bf16 output: a lane stores to TWO rows of a row tile (its accumulators change lanes first, below);
+        // bf16, and fp8 with quantised output: to its own
+        constexpr int NR = (FP8 && !QOUT) ? 2 : 1;
         bool ok[TM][NR];
         bf16_t* crow[TM][NR];
         float rs[TM];
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             rs[i] = 1.f;
-            if constexpr (FP8 || EPI == EPI_GATE) rs[i] = s_row_scale[tpar][rbase_e + i * MT + (lane_e & (MT - 1))];  // (of the row it computed)
+            if constexpr (FP8 || EPI == EPI_GATE) {
+                if (!BSA || p.row_scale) rs[i] = s_row_scale[tpar][rbase_e + i * MT + (lane_e & (MT - 1))];  // (of the row it computed)
+            }
 #pragma unroll
             for (int h = 0; h < NR; ++h) {
-                const int r = rbase_e + i * MT + (FP8 ? (lane_e & 15) + 16 * h : (lane_e & (MT - 1)));
+                const int r = rbase_e + i * MT + ((FP8 && !QOUT) ? (lane_e & 15) + 16 * h : (lane_e & (MT - 1)));
                 ok[i][h] = r < rv;
                 const size_t grow = (size_t)(row0 + (ok[i][h] ? r : 0));
                 const int crow_i = p.c_map ? s_crow[tpar][r] : 0;
                 ok[i][h] = ok[i][h] && crow_i >= 0;  // a negative map entry: the row has no place in the output
-                crow[i][h] = C + (p.c_map ? (size_t)max(crow_i, 0) : grow) * p.ldc + (DW ? (size_t)g * p.c_group_stride : (size_t)0);
+                // (quantised output: C holds one-byte codes, addressed below from the same row index)
+                crow[i][h] = C + (p.c_map ? (size_t)max(crow_i, 0) : grow) * (QOUT ? (size_t)1 : (size_t)p.ldc) + (DW ? (size_t)g * p.c_group_stride : (size_t)0);
             }
         }
 #pragma unroll
@@ -800,6 +922,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             const int pcol = nt * BN + cbase_e + jg * 32;  // first packed column of the group
             const int colg = EPI == EPI_SWIGLU ? (pcol / 64) * 32 : pcol;  // its first output column
             [[maybe_unused]] uint4 pk[2];  // fp8: the lane's two 16-byte units of the group, stored after they changed lanes
+            [[maybe_unused]] float xq[2][8];  // quantised output: the lane's sixteen values of the group's block of 32 columns
 #pragma unroll
             for (int u = 0; u < NU; ++u) {
                 // the lane's eight consecutive columns: two runs of four accumulators (bf16: the group's two tiles;
@@ -840,6 +963,11 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                         x[4 * t + e] = v;
                     }
                 }
+                if constexpr (QOUT) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) xq[u][e] = x[e];
+                    continue;
+                }
                 uint4 o4;
                 o4.x = gg_pack_bf16(x[0], x[1]);
                 o4.y = gg_pack_bf16(x[2], x[3]);
@@ -868,7 +996,46 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
                     }
                 }
             }
-            if constexpr (FP8) {
+            if constexpr (QOUT) {
+                // The group is one block of 32 output columns of the hidden activation: the lane holds 16 of its values
+                // (columns 8 lsub .. + 7 and 16 + 8 lsub .. + 7), the lane 32 further the other 16.  Block scale = the
+                // smallest power of two under which the block's largest magnitude fits e4m3; codes = the values divided by
+                // it (exact), rounded to e4m3; the two lanes trade a run of 8 codes each, so that each stores 16 contiguous
+                // bytes of its row; one lane of the pair stores the scale byte.
+                float am = 0.f;
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) am = fmaxf(am, fabsf(xq[u][e]));
+                {
+                    const auto sw_ = __builtin_amdgcn_permlane32_swap(__float_as_uint(am), __float_as_uint(am), false, false);
+                    am = fmaxf(__uint_as_float(sw_[0]), __uint_as_float(sw_[1]));
+                }
+                const int sbyte = gg_block_scale_byte(__float_as_uint(am));
+                const float inv = __uint_as_float(gg_block_inv_bits(sbyte));
+                uint32_t cd[2][2];
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    int lo = 0, hi = 0;
+                    lo = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(xq[u][0], inv), __fmul_rn(xq[u][1], inv), lo, false);
+                    lo = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(xq[u][2], inv), __fmul_rn(xq[u][3], inv), lo, true);
+                    hi = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(xq[u][4], inv), __fmul_rn(xq[u][5], inv), hi, false);
+                    hi = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(xq[u][6], inv), __fmul_rn(xq[u][7], inv), hi, true);
+                    cd[u][0] = (uint32_t)lo;
+                    cd[u][1] = (uint32_t)hi;
+                }
+                // lanes 0-31 keep their first run and take the partner's first run (columns 0-15 of the block), lanes 32-63
+                // take the partner's second run and keep their own (columns 16-31)
+                const auto s0_ = __builtin_amdgcn_permlane32_swap(cd[0][0], cd[1][0], false, false);
+                const auto s1_ = __builtin_amdgcn_permlane32_swap(cd[0][1], cd[1][1], false, false);
+                const uint4 codes = make_uint4(s0_[0], s1_[0], s0_[1], s1_[1]);
+                const int col = colg + 16 * lsub;
+                if (ok[i][0] && col < p.N) {
+                    uint8_t* qrow = (uint8_t*)p.C + (size_t)(crow[i][0] - C) * p.ldc;
+                    *(uint4*)(qrow + col) = codes;
+                    if (lsub == 0) p.c_bscale[(size_t)(crow[i][0] - C) * p.bs_pitch + colg / 32] = (uint8_t)sbyte;
+                }
+            } else if constexpr (FP8) {
                 // A lane holds 16 bytes of each half of its row's 64 (columns 8 lsub .. and 16 + 8 lsub ..) and the lane 16
                 // further the same of the row 16 further.  They trade one half each (v_permlane16_swap: lanes 16-31 and
                 // 48-63 of the first operand against lanes 0-15 and 32-47 of the second), after which the first operand
@@ -908,6 +1075,8 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 #undef GG_STAGE_PTRS
 #undef GG_ISSUE_RANGE
 #undef GG_PROLOGUE
+#undef GG_SC_DMA
+#undef GG_SC_READ
 }
 
 // ---- second half of a K-split tile: add its parts in part order, then the epilogue of the GEMM kernel ------------
@@ -971,7 +1140,7 @@ __global__ __launch_bounds__(256) void gg_reduce_parts_kernel(const GemmParams p
         }
         const size_t grow = (size_t)(t.row0 + r);
         float rs = 1.f;
-        if constexpr (FP8 || EPI == EPI_GATE) rs = p.row_scale[grow];
+        if constexpr (FP8 || EPI == EPI_GATE) rs = p.row_scale ? p.row_scale[grow] : 1.f;  // (fp8 down projection: a gate, or nothing)
         float av[4] = {a.x, a.y, a.z, a.w}, bv[4] = {b.x, b.y, b.z, b.w};
         if constexpr (!FP8 && EPI != EPI_NONE && EPI != EPI_GATE) {
             if (p.C2 && col < p.N) {  // the values before the activation, kept for the backward pass (rows are never remapped there)
@@ -1004,7 +1173,24 @@ __global__ __launch_bounds__(256) void gg_reduce_parts_kernel(const GemmParams p
             }
         }
         const int crow = p.c_map ? p.c_map[grow] : 0;
-        if (col < p.N && crow >= 0) {
+        if constexpr (FP8 && EPI == EPI_SWIGLU) {
+            // quantised output, as in the GEMM kernel's epilogue: the eight threads that hold a block of 32 columns of this
+            // row (consecutive lanes; every thread of the block is in the loop together: r depends on threadIdx.x / OC4 only)
+            float am = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3])));
+            if (col >= p.N) am = 0.f;
+#pragma unroll
+            for (int off = 1; off < 8; off <<= 1) am = fmaxf(am, __shfl_xor(am, off, WAVE));
+            const int sbyte = gg_block_scale_byte(__float_as_uint(am));
+            const float inv = __uint_as_float(gg_block_inv_bits(sbyte));
+            int cd = 0;
+            cd = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(x[0], inv), __fmul_rn(x[1], inv), cd, false);
+            cd = __builtin_amdgcn_cvt_pk_fp8_f32(__fmul_rn(x[2], inv), __fmul_rn(x[3], inv), cd, true);
+            if (col < p.N && crow >= 0) {
+                const size_t orow = p.c_map ? (size_t)crow : grow;
+                *(uint32_t*)((uint8_t*)p.C + orow * p.ldc + col) = (uint32_t)cd;
+                if ((col & 31) == 0) p.c_bscale[orow * p.bs_pitch + col / 32] = (uint8_t)sbyte;
+            }
+        } else if (col < p.N && crow >= 0) {
             uint2 o;
             o.x = gg_pack_bf16(x[0], x[1]);
             o.y = gg_pack_bf16(x[2], x[3]);
@@ -1571,22 +1757,27 @@ int launch_gemm(const GemmParams& p_in, int epi, hipStream_t s, void* part_ws = 
     const int bm = small_m ? 128 : 256, nk = p.K * (FP8 ? 1 : 2) / ROWB;
     const long long ub = ((long long)(p.S_rows + bm - 1) / bm + p.E_l) * nt;
     const bool all_split = p.part_ws && red_blocks > 0 && 4 * ub <= grid && nk >= 2 * GG_MIN_PART_STAGES && p.max_units >= 2 * ub;
+    // fp8 without activation is the down projection of the expert MLP: its activation operand is block-scaled
 #define GG_LAUNCH(BMv, NWMv, EPIv)                                                                        \
     do {                                                                                                  \
-        if (!all_split) grouped_gemm_kernel<BMv, NWMv, EPIv, FP8, false><<<grid, NWMv * 2 * WAVE, 0, s>>>(p); \
+        constexpr bool BSAv = FP8 && EPIv == EPI_NONE;                                                    \
+        if (!all_split) grouped_gemm_kernel<BMv, NWMv, EPIv, FP8, false, false, BSAv><<<grid, NWMv * 2 * WAVE, 0, s>>>(p); \
         if (p.part_ws && red_blocks > 0) {                                                                \
             /* (the launch that takes parts stores raw partial sums: one instantiation whatever the epilogue) */ \
-            grouped_gemm_kernel<BMv, NWMv, EPI_NONE, FP8, true><<<grid, NWMv * 2 * WAVE, 0, s>>>(p);       \
+            grouped_gemm_kernel<BMv, NWMv, EPI_NONE, FP8, true, false, BSAv><<<grid, NWMv * 2 * WAVE, 0, s>>>(p); \
             gg_reduce_parts_kernel<BMv, EPIv, FP8><<<red_blocks, 256, 0, s>>>(p, grid);                    \
         }                                                                                                 \
     } while (0)
 #define GG_EPI(EPIv)                          \
     do {                                      \
         if (small_m) GG_LAUNCH(128, 2, EPIv); \
-        else GG_LAUNCH(256, (FP8 ? GG_FP8_NWM : GG_BIG_NWM), EPIv); \
+        else GG_LAUNCH(256, (FP8 ? (EPIv == EPI_NONE ? GG_FP8_BSA_NWM : GG_FP8_NWM) : GG_BIG_NWM), EPIv); \
     } while (0)
     switch (epi) {
-        case EPI_NONE: GG_EPI(EPI_NONE); break;
+        case EPI_NONE:
+            if (FP8 && !p.a_bscale) return moe_fail(MOE_ERR_INVALID, "grouped_gemm: the fp8 down projection needs block scales");
+            GG_EPI(EPI_NONE);
+            break;
         // (no fp8 entry point asks for these two: not instantiated)
         case EPI_GELU: if constexpr (FP8) return moe_fail(MOE_ERR_UNSUPPORTED, "grouped_gemm: fp8 with activation %d", epi); else GG_EPI(EPI_GELU); break;
         case EPI_SILU: if constexpr (FP8) return moe_fail(MOE_ERR_UNSUPPORTED, "grouped_gemm: fp8 with activation %d", epi); else GG_EPI(EPI_SILU); break;
@@ -1806,42 +1997,55 @@ extern "C" int moe_quantize_rows_fp8(const void* x_bf16, int rows, int cols, uin
     return launch_quantize(x_bf16, nullptr, rows, cols, q, scale, n_rows_dev, (hipStream_t)stream);
 }
 
-extern "C" int moe_grouped_mlp_fp8_mapped(const void* a_base_bf16, int a_rows, const int32_t* a_row_map,
-                                          const int32_t* expert_cnt, int S_rows, int H, int F, int E_l,
-                                          const uint8_t* wgu_packed, const float* sg, const float* su,
-                                          const uint8_t* wd_packed, const float* sd, uint8_t* xq_ws, float* xs_ws, void* h_ws,
-                                          uint8_t* hq_ws, float* hs_ws, void* out, int out_rows, const int32_t* c_row_map,
-                                          void* part_ws, size_t part_ws_bytes, moe_stream_t stream) {
-    hipStream_t s = (hipStream_t)stream;
-    MOE_REQUIRE(S_rows >= 0 && H > 0 && F > 0 && E_l > 0 && E_l <= GG_MAXG, MOE_ERR_INVALID, "grouped_mlp_fp8: bad shape");
-    MOE_REQUIRE(H % 128 == 0 && F % 128 == 0, MOE_ERR_UNSUPPORTED, "grouped_mlp_fp8: needs H, F multiples of 128 (H=%d F=%d)", H, F);
-    MOE_REQUIRE(a_rows >= 0 && out_rows >= 0, MOE_ERR_INVALID, "grouped_mlp_fp8: negative buffer rows");
-    if (S_rows == 0) return MOE_OK;
-    MOE_REQUIRE(a_base_bf16 && expert_cnt && wgu_packed && sg && su && wd_packed && sd && xq_ws && xs_ws && h_ws && hq_ws &&
-                    hs_ws && out, MOE_ERR_INVALID, "grouped_mlp_fp8: null pointer");
-    // the row quantisation reads every input row once anyway: with a map it reads it where the transfer left it
-    int rc = launch_quantize(a_base_bf16, a_row_map, S_rows, H, xq_ws, xs_ws, nullptr, s);
-    if (rc) return rc;
+// The two GEMMs of the fp8 SwiGLU expert on quantised rows (xq codes gathered through a_map, xs their scales in GEMM row
+// order): gate/up + SwiGLU with the hidden activation quantised in the epilogue (codes hq, one E8M0 scale byte per row and
+// 32 columns in hscale), then the down projection, which takes those bytes as the scale operand of its MFMAs; row_gate
+// (nullable) multiplies the result rows.
+static int fp8_mlp_gemms(const uint8_t* xq, const int32_t* a_map, const float* xs, const int32_t* expert_cnt, int S_rows, int H, int F,
+                         int E_l, const uint8_t* wgu_packed, const float* sg, const float* su, const uint8_t* wd_packed,
+                         const float* sd, uint8_t* hq_ws, uint8_t* hscale_ws, const float* row_gate, void* out,
+                         const int32_t* c_row_map, void* part_ws, size_t part_ws_bytes, hipStream_t s) {
     GemmParams p{};
-    p.A = xq_ws; p.B = wgu_packed; p.C = h_ws; p.cnt = expert_cnt; p.row_scale = xs_ws; p.col_scale = sg; p.col_scale2 = su;
+    p.A = xq; p.B = wgu_packed; p.C = hq_ws; p.cnt = expert_cnt; p.row_scale = xs; p.col_scale = sg; p.col_scale2 = su;
+    p.a_map = a_map; p.c_bscale = hscale_ws; p.bs_pitch = F / 32;
     p.E_l = E_l; p.K = H; p.N = F; p.Npad = round_up(2 * F, GG_BN); p.ldc = F; p.S_rows = S_rows; p.ncs = F;
-    rc = launch_gemm<true>(p, EPI_SWIGLU, s, part_ws, part_ws_bytes);
-    if (rc) return rc;
-    rc = launch_quantize(h_ws, nullptr, S_rows, F, hq_ws, hs_ws, nullptr, s);
+    int rc = launch_gemm<true>(p, EPI_SWIGLU, s, part_ws, part_ws_bytes);
     if (rc) return rc;
     GemmParams q{};
-    q.A = hq_ws; q.B = wd_packed; q.C = out; q.cnt = expert_cnt; q.row_scale = hs_ws; q.col_scale = sd;
-    q.c_map = c_row_map;
+    q.A = hq_ws; q.B = wd_packed; q.C = out; q.cnt = expert_cnt; q.row_scale = row_gate; q.col_scale = sd;
+    q.c_map = c_row_map; q.a_bscale = hscale_ws; q.bs_pitch = F / 32;
     q.E_l = E_l; q.K = F; q.N = H; q.Npad = round_up(H, GG_BN); q.ldc = H; q.S_rows = S_rows; q.ncs = H;
     return launch_gemm<true>(q, EPI_NONE, s, part_ws, part_ws_bytes);
 }
 
+extern "C" int moe_grouped_mlp_fp8_mapped(const void* a_base_bf16, int a_rows, const int32_t* a_row_map,
+                                          const int32_t* expert_cnt, int S_rows, int H, int F, int E_l,
+                                          const uint8_t* wgu_packed, const float* sg, const float* su,
+                                          const uint8_t* wd_packed, const float* sd, uint8_t* xq_ws, float* xs_ws,
+                                          uint8_t* hq_ws, uint8_t* hscale_ws, const float* row_gate, void* out, int out_rows,
+                                          const int32_t* c_row_map, void* part_ws, size_t part_ws_bytes, moe_stream_t stream) {
+    hipStream_t s = (hipStream_t)stream;
+    MOE_REQUIRE(S_rows >= 0 && H > 0 && F > 0 && E_l > 0 && E_l <= GG_MAXG, MOE_ERR_INVALID, "grouped_mlp_fp8: bad shape");
+    MOE_REQUIRE(H % 128 == 0 && F % 128 == 0, MOE_ERR_UNSUPPORTED, "grouped_mlp_fp8: needs H, F multiples of 128 (H=%d F=%d)", H, F);
+    MOE_REQUIRE(a_rows >= 0 && out_rows >= 0, MOE_ERR_INVALID, "grouped_mlp_fp8: negative buffer rows");
+    MOE_REQUIRE((unsigned long long)S_rows * (unsigned long long)(F / 32) < (1ull << 32), MOE_ERR_UNSUPPORTED,
+                "grouped_mlp_fp8: the block scales must stay under 4 GiB");
+    if (S_rows == 0) return MOE_OK;
+    MOE_REQUIRE(a_base_bf16 && expert_cnt && wgu_packed && sg && su && wd_packed && sd && xq_ws && xs_ws && hq_ws && hscale_ws && out,
+                MOE_ERR_INVALID, "grouped_mlp_fp8: null pointer");
+    // the row quantisation reads every input row once anyway: with a map it reads it where the transfer left it
+    int rc = launch_quantize(a_base_bf16, a_row_map, S_rows, H, xq_ws, xs_ws, nullptr, s);
+    if (rc) return rc;
+    return fp8_mlp_gemms(xq_ws, nullptr, xs_ws, expert_cnt, S_rows, H, F, E_l, wgu_packed, sg, su, wd_packed, sd, hq_ws, hscale_ws,
+                         row_gate, out, c_row_map, part_ws, part_ws_bytes, s);
+}
+
 extern "C" int moe_grouped_mlp_fp8(const void* tokens_bf16, const int32_t* expert_cnt, int S_rows, int H, int F, int E_l,
                                    const uint8_t* wgu_packed, const float* sg, const float* su, const uint8_t* wd_packed,
-                                   const float* sd, uint8_t* xq_ws, float* xs_ws, void* h_ws, uint8_t* hq_ws, float* hs_ws,
-                                   void* out, moe_stream_t stream) {
+                                   const float* sd, uint8_t* xq_ws, float* xs_ws, uint8_t* hq_ws, uint8_t* hscale_ws, void* out,
+                                   moe_stream_t stream) {
     return moe_grouped_mlp_fp8_mapped(tokens_bf16, S_rows, nullptr, expert_cnt, S_rows, H, F, E_l, wgu_packed, sg, su, wd_packed,
-                                      sd, xq_ws, xs_ws, h_ws, hq_ws, hs_ws, out, S_rows, nullptr, nullptr, 0, stream);
+                                      sd, xq_ws, xs_ws, hq_ws, hscale_ws, nullptr, out, S_rows, nullptr, nullptr, 0, stream);
 }
 
 extern "C" int moe_pack_tokens_fp8(const void* x_bf16, int T, int H, const int32_t* topk_idx, const int32_t* pos, int k, int E_l,
@@ -1878,33 +2082,24 @@ extern "C" int moe_pack_tokens_fp8_gated(const void* x_bf16, int T, int H, const
 extern "C" int moe_grouped_mlp_fp8_q_mapped(const uint8_t* a_q, const float* a_scale, int a_rows, const int32_t* a_row_map,
                                             const int32_t* expert_cnt, int S_rows, int H, int F, int E_l,
                                             const uint8_t* wgu_packed, const float* sg, const float* su,
-                                            const uint8_t* wd_packed, const float* sd, float* xs_ws, void* h_ws, uint8_t* hq_ws,
-                                            float* hs_ws, void* out, int out_rows, const int32_t* c_row_map, void* part_ws,
-                                            size_t part_ws_bytes, moe_stream_t stream) {
+                                            const uint8_t* wd_packed, const float* sd, float* xs_ws, uint8_t* hq_ws,
+                                            uint8_t* hscale_ws, const float* row_gate, void* out, int out_rows,
+                                            const int32_t* c_row_map, void* part_ws, size_t part_ws_bytes, moe_stream_t stream) {
     hipStream_t s = (hipStream_t)stream;
     MOE_REQUIRE(S_rows >= 0 && H > 0 && F > 0 && E_l > 0 && E_l <= GG_MAXG, MOE_ERR_INVALID, "grouped_mlp_fp8_q: bad shape");
     MOE_REQUIRE(H % 128 == 0 && F % 128 == 0, MOE_ERR_UNSUPPORTED, "grouped_mlp_fp8_q: needs H, F multiples of 128 (H=%d F=%d)", H, F);
     MOE_REQUIRE(a_rows >= 0 && out_rows >= 0, MOE_ERR_INVALID, "grouped_mlp_fp8_q: negative buffer rows");
     MOE_REQUIRE(!a_row_map || (unsigned long long)a_rows * (unsigned long long)H < (1ull << 32), MOE_ERR_UNSUPPORTED,
                 "grouped_mlp_fp8_q: the gathered buffer must be smaller than 4 GiB (%d rows of %d)", a_rows, H);
+    MOE_REQUIRE((unsigned long long)S_rows * (unsigned long long)(F / 32) < (1ull << 32), MOE_ERR_UNSUPPORTED,
+                "grouped_mlp_fp8_q: the block scales must stay under 4 GiB");
     if (S_rows == 0) return MOE_OK;
-    MOE_REQUIRE(a_q && a_scale && expert_cnt && wgu_packed && sg && su && wd_packed && sd && xs_ws && h_ws && hq_ws && hs_ws && out,
+    MOE_REQUIRE(a_q && a_scale && expert_cnt && wgu_packed && sg && su && wd_packed && sd && xs_ws && hq_ws && hscale_ws && out,
                 MOE_ERR_INVALID, "grouped_mlp_fp8_q: null pointer");
     // the row scales in the order of the GEMM's rows (the codes themselves are gathered by the GEMM as it loads them)
     gather_scale_kernel<<<ceil_div(S_rows, 256), 256, 0, s>>>(a_scale, a_row_map, S_rows, xs_ws);
-    GemmParams p{};
-    p.A = a_q; p.B = wgu_packed; p.C = h_ws; p.cnt = expert_cnt; p.row_scale = xs_ws; p.col_scale = sg; p.col_scale2 = su;
-    p.a_map = a_row_map;
-    p.E_l = E_l; p.K = H; p.N = F; p.Npad = round_up(2 * F, GG_BN); p.ldc = F; p.S_rows = S_rows; p.ncs = F;
-    int rc = launch_gemm<true>(p, EPI_SWIGLU, s, part_ws, part_ws_bytes);
-    if (rc) return rc;
-    rc = launch_quantize(h_ws, nullptr, S_rows, F, hq_ws, hs_ws, nullptr, s);
-    if (rc) return rc;
-    GemmParams q{};
-    q.A = hq_ws; q.B = wd_packed; q.C = out; q.cnt = expert_cnt; q.row_scale = hs_ws; q.col_scale = sd;
-    q.c_map = c_row_map;
-    q.E_l = E_l; q.K = F; q.N = H; q.Npad = round_up(H, GG_BN); q.ldc = H; q.S_rows = S_rows; q.ncs = H;
-    return launch_gemm<true>(q, EPI_NONE, s, part_ws, part_ws_bytes);
+    return fp8_mlp_gemms(a_q, a_row_map, xs_ws, expert_cnt, S_rows, H, F, E_l, wgu_packed, sg, su, wd_packed, sd, hq_ws, hscale_ws,
+                         row_gate, out, c_row_map, part_ws, part_ws_bytes, s);
 }
 
 // ---- backward pass entry points --------------------------------------------------------------------------------------

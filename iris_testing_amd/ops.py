@@ -365,7 +365,9 @@ def quantize_rows_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
 
 def grouped_mlp_fp8(tokens: torch.Tensor, expert_cnt: torch.Tensor, F: int, wgu_packed, sg, su, wd_packed, sd,
                     ws: Optional[dict] = None, out: Optional[torch.Tensor] = None,
-                    part_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    part_ws: Optional[torch.Tensor] = None, row_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp8 SwiGLU expert MLP on bf16 rows.  ws (fp8_workspace) receives the intermediates: "xq" / "xs" the rows quantised per
+    row, "hq" / "hsc" the hidden activation as e4m3 codes with one power-of-two scale byte per row and 32 columns."""
     _req_cuda(tokens, "tokens")
     assert tokens.dtype == torch.bfloat16
     S, H = tokens.shape
@@ -375,23 +377,18 @@ def grouped_mlp_fp8(tokens: torch.Tensor, expert_cnt: torch.Tensor, F: int, wgu_
         ws = fp8_workspace(S, H, F, dev)
     if out is None:
         out = torch.zeros((S, H), dtype=torch.bfloat16, device=dev)
-    if part_ws is None:
-        L.check(L.lib().moe_grouped_mlp_fp8(L.ptr(tokens), L.ptr(expert_cnt), S, H, F, E_l, L.ptr(wgu_packed), L.ptr(sg),
-                                            L.ptr(su), L.ptr(wd_packed), L.ptr(sd), L.ptr(ws["xq"]), L.ptr(ws["xs"]),
-                                            L.ptr(ws["h"]), L.ptr(ws["hq"]), L.ptr(ws["hs"]), L.ptr(out), L.stream_ptr()))
-    else:  # with the K-split scratch (gemm_part_workspace): an under-filled last round of tiles is cut along K
-        L.check(L.lib().moe_grouped_mlp_fp8_mapped(L.ptr(tokens), S, None, L.ptr(expert_cnt), S, H, F, E_l, L.ptr(wgu_packed),
-                                                   L.ptr(sg), L.ptr(su), L.ptr(wd_packed), L.ptr(sd), L.ptr(ws["xq"]),
-                                                   L.ptr(ws["xs"]), L.ptr(ws["h"]), L.ptr(ws["hq"]), L.ptr(ws["hs"]), L.ptr(out), S,
-                                                   None, L.ptr(part_ws), part_ws.numel() * part_ws.element_size(),
-                                                   L.stream_ptr()))
+    L.check(L.lib().moe_grouped_mlp_fp8_mapped(L.ptr(tokens), S, None, L.ptr(expert_cnt), S, H, F, E_l, L.ptr(wgu_packed),
+                                               L.ptr(sg), L.ptr(su), L.ptr(wd_packed), L.ptr(sd), L.ptr(ws["xq"]),
+                                               L.ptr(ws["xs"]), L.ptr(ws["hq"]), L.ptr(ws["hsc"]), L.ptr(row_gate), L.ptr(out), S,
+                                               None, L.ptr(part_ws), 0 if part_ws is None else part_ws.numel() * part_ws.element_size(),
+                                               L.stream_ptr()))
     return out
-
 
 
 def grouped_mlp_fp8_q(a_q: torch.Tensor, a_scale: torch.Tensor, a_row_map: Optional[torch.Tensor], expert_cnt: torch.Tensor,
                       S_rows: int, F: int, wgu_packed, sg, su, wd_packed, sd, ws: dict, out: torch.Tensor,
-                      c_row_map: Optional[torch.Tensor] = None, part_ws: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      c_row_map: Optional[torch.Tensor] = None, part_ws: Optional[torch.Tensor] = None,
+                      row_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """grouped_mlp_fp8 for rows that arrive as fp8 codes and scales (pack_tokens_fp8): a_q [rows,H] uint8, a_scale [rows];
     ws as from fp8_workspace (its "xq" is not used, "xs" receives the scales in row order)."""
     _req_cuda(a_q, "a_q")
@@ -400,13 +397,11 @@ def grouped_mlp_fp8_q(a_q: torch.Tensor, a_scale: torch.Tensor, a_row_map: Optio
     assert a_scale.numel() == a_q.shape[0] and out.dtype == torch.bfloat16 and out.dim() == 2 and out.is_contiguous()
     H = a_q.shape[1]
     assert out.shape[1] == H
-    L.check(L.lib().moe_grouped_mlp_fp8_q_mapped(L.ptr(a_q), L.ptr(a_scale), a_q.shape[0],
-                                                 L.ptr(a_row_map) if a_row_map is not None else None, L.ptr(expert_cnt), S_rows, H, F,
-                                                 expert_cnt.numel(), L.ptr(wgu_packed), L.ptr(sg), L.ptr(su), L.ptr(wd_packed),
-                                                 L.ptr(sd), L.ptr(ws["xs"]), L.ptr(ws["h"]), L.ptr(ws["hq"]), L.ptr(ws["hs"]),
-                                                 L.ptr(out), out.shape[0], L.ptr(c_row_map) if c_row_map is not None else None,
-                                                 L.ptr(part_ws) if part_ws is not None else None,
-                                                 part_ws.numel() * part_ws.element_size() if part_ws is not None else 0,
+    L.check(L.lib().moe_grouped_mlp_fp8_q_mapped(L.ptr(a_q), L.ptr(a_scale), a_q.shape[0], L.ptr(a_row_map), L.ptr(expert_cnt),
+                                                 S_rows, H, F, expert_cnt.numel(), L.ptr(wgu_packed), L.ptr(sg), L.ptr(su),
+                                                 L.ptr(wd_packed), L.ptr(sd), L.ptr(ws["xs"]), L.ptr(ws["hq"]), L.ptr(ws["hsc"]),
+                                                 L.ptr(row_gate), L.ptr(out), out.shape[0], L.ptr(c_row_map), L.ptr(part_ws),
+                                                 0 if part_ws is None else part_ws.numel() * part_ws.element_size(),
                                                  L.stream_ptr()))
     return out
 
@@ -415,10 +410,16 @@ def fp8_workspace(S: int, H: int, F: int, dev) -> dict:
     return {
         "xq": torch.empty((S, H), dtype=torch.uint8, device=dev),
         "xs": torch.empty((S,), dtype=torch.float32, device=dev),
-        "h": torch.empty((S, F), dtype=torch.bfloat16, device=dev),
-        "hq": torch.empty((S, F), dtype=torch.uint8, device=dev),
-        "hs": torch.empty((S,), dtype=torch.float32, device=dev),
+        "hq": torch.empty((S, F), dtype=torch.uint8, device=dev),      # hidden activation: e4m3 codes ...
+        "hsc": torch.empty((S, F // 32), dtype=torch.uint8, device=dev),  # ... and their block scales (E8M0 bytes)
     }
+
+
+def dequantize_hidden_fp8(hq: torch.Tensor, hsc: torch.Tensor) -> torch.Tensor:
+    """The hidden activation an fp8 MLP call left in its workspace, as fp32: code value x 2^(scale byte - 127) per block of 32."""
+    vals = hq.view(torch.float8_e4m3fn).float()
+    scale = torch.exp2(hsc.float() - 127.0)
+    return (vals.view(hq.shape[0], -1, 32) * scale[:, :, None]).view(hq.shape)
 
 
 # ---- a13 ------------------------------------------------------------------------------------

@@ -48,8 +48,8 @@ class DispatchPipeline:
             raise ValueError("gated / padding_free are forms of the fused destination side")
         if self.gated and self.padding_free:
             raise ValueError("gated and padding_free are separate modes")
-        if self.gated and weights.dtype != torch.bfloat16:
-            raise ValueError("the gated return needs bf16 experts")
+        if self.gated and weights.dtype == torch.float32:
+            raise ValueError("the gated return needs bf16 or fp8 experts")
         if self.gated and recv_gate is None:
             raise ValueError("gated: pass the gates that arrive with the rows (harness.recv_gates)")
         if self.padding_free and recv_flat is None:
@@ -95,7 +95,7 @@ class DispatchPipeline:
         self.rows = torch.empty((S, H), dtype=dt, device=dev)
         self.expert_cnt = i32(E_l)
         self.unpack_map = i32(lib.moe_recv_map_ints(W, E_l, S))
-        self.hidden = torch.empty((S, F), dtype=dt, device=dev)
+        self.hidden = torch.empty((S, F), dtype=dt, device=dev) if weights.dtype != torch.uint8 else None
         self.y = torch.zeros((S, H), dtype=dt, device=dev)
         self.ret = torch.empty((W, M, H), dtype=dt, device=dev) if not self.padding_free else None
         self.ret_map = i32(lib.moe_recv_map_ints(W, E_l, W * M))
@@ -106,8 +106,8 @@ class DispatchPipeline:
         if weights.dtype == torch.uint8:
             self.xq = torch.empty((S, H), dtype=torch.uint8, device=dev)
             self.xs = torch.empty((S,), dtype=torch.float32, device=dev)
-            self.hq = torch.empty((S, F), dtype=torch.uint8, device=dev)
-            self.hs = torch.empty((S,), dtype=torch.float32, device=dev)
+            self.hq = torch.empty((S, F), dtype=torch.uint8, device=dev)          # hidden activation: e4m3 codes
+            self.hsc = torch.empty((S, F // 32), dtype=torch.uint8, device=dev)   # and one scale byte per row and 32 columns
         # source side again: what comes back ([W,M,H], same slots as `send`) and the combined output
         if self.padding_free:  # the returned payload: [R,H], row pos[t,kk] is the result of slot (t,kk)
             self.returned = returned if returned is not None else torch.zeros((T * k, H), dtype=dt, device=dev)
@@ -133,9 +133,11 @@ class DispatchPipeline:
     def pack(self, s):
         c, w = self.cfg, self.world
         if self.fp8_dispatch:
-            L.check(L.lib().moe_pack_tokens_fp8(self._p(w.x0), c.tokens, c.hidden, self._p(self.idx), self._p(self.pos), c.topk,
-                                                c.e_local, self._p(self.dst_sizes), self._p(self.dst_offsets), c.world, w.M,
-                                                self._p(self.send_q), self._p(self.send_scale), self._p(self.status), s))
+            L.check(L.lib().moe_pack_tokens_fp8_gated(self._p(w.x0), c.tokens, c.hidden, self._p(self.idx), self._p(self.pos),
+                                                      self._p(self.gate) if self.gated else None, c.topk, c.e_local,
+                                                      self._p(self.dst_sizes), self._p(self.dst_offsets), c.world, w.M,
+                                                      self._p(self.send_q), self._p(self.send_scale),
+                                                      self._p(self.send_gate) if self.gated else None, self._p(self.status), s))
             return
         if self.padding_free:
             L.check(L.lib().moe_pack_payload(self._p(w.x0), self.code, c.tokens, c.hidden, self._p(self.row_token),
@@ -181,8 +183,9 @@ class DispatchPipeline:
                 L.check(lib.moe_grouped_mlp_fp8_q_mapped(self._p(w.recv_q), self._p(w.recv_scale), c.world * w.M,
                                                          self._p(self.row_map), self._p(self.expert_cnt), self.S, c.hidden, c.ffn,
                                                          c.e_local, self._p(ew.w1), self._p(sg), self._p(su), self._p(ew.w2),
-                                                         self._p(sd), self._p(self.xs), self._p(self.hidden), self._p(self.hq),
-                                                         self._p(self.hs), self._p(self.ret), c.world * w.M, self._p(self.row_map),
+                                                         self._p(sd), self._p(self.xs), self._p(self.hq), self._p(self.hsc),
+                                                         self._p(self.row_gate) if self.gated else None, self._p(self.ret),
+                                                         c.world * w.M, self._p(self.row_map),
                                                          self._p(self.part_ws), self.part_ws_bytes, s))
                 return
             src, n_src, a_map = (w.recv, c.world * w.M, self.row_map) if self.fused else (self.rows, self.S, None)
@@ -191,8 +194,9 @@ class DispatchPipeline:
                 src, n_src, dst, n_dst = self.recv_flat, self.S, self.ret_flat, self.S
             L.check(lib.moe_grouped_mlp_fp8_mapped(self._p(src), n_src, self._p(a_map), self._p(self.expert_cnt), self.S, c.hidden,
                                                    c.ffn, c.e_local, self._p(ew.w1), self._p(sg), self._p(su), self._p(ew.w2),
-                                                   self._p(sd), self._p(self.xq), self._p(self.xs), self._p(self.hidden),
-                                                   self._p(self.hq), self._p(self.hs), self._p(dst), n_dst, self._p(c_map),
+                                                   self._p(sd), self._p(self.xq), self._p(self.xs), self._p(self.hq),
+                                                   self._p(self.hsc), self._p(self.row_gate) if self.gated else None,
+                                                   self._p(dst), n_dst, self._p(c_map),
                                                    self._p(self.part_ws), self.part_ws_bytes, s))
         elif ew.dtype == torch.float32:
             L.check(lib.moe_grouped_mlp(self._p(self.rows), self._p(self.expert_cnt), self.code, self.S, c.hidden, c.ffn,

@@ -159,6 +159,35 @@ def quantize_rows_fp8(x: np.ndarray) -> Tuple[np.ndarray, np.ndarray]:
     return q, scale
 
 
+FP8_BLOCK = 32  # columns per block scale of the fp8 hidden activation
+
+
+def quantize_blocks_fp8(x: np.ndarray) -> Tuple[np.ndarray, np.ndarray]:
+    """Block quantisation of the fp8 expert's hidden activation: one power-of-two scale per row and 32 columns.
+
+    For every block: amax = max|x|; scale byte b = the smallest b >= 0 with amax / 2^(b-127) <= 448 (an E8M0 exponent:
+    from the bits of amax = m 2^p, b = p + 127 - 8, one more when m > 1.75; the integer expression below is the one the
+    kernels evaluate); codes = e4m3(x / 2^(b-127)), the division being exact.  Returns (uint8 codes [R,C], uint8 scale
+    bytes [R, C/32]).  Not in the reference (the workload description only says "fp8 MFMA grouped GEMM")."""
+    x = np.asarray(x, dtype=np.float32)
+    R, C = x.shape
+    assert C % FP8_BLOCK == 0
+    xb = x.reshape(R, C // FP8_BLOCK, FP8_BLOCK)
+    amax = np.max(np.abs(xb), axis=2).astype(np.float32)
+    bits = amax.view(np.uint32).astype(np.int64)
+    b = np.maximum(((bits + 0x1FFFFF) >> 23) - 8, 0)
+    inv = ((254 - b).astype(np.uint32) << np.uint32(23)).view(np.float32)  # 2^(127-b), exact
+    q = fp8_e4m3_encode((xb * inv[:, :, None]).astype(np.float32)).reshape(R, C)
+    return q, b.astype(np.uint8)
+
+
+def dequantize_blocks_fp8(q: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """codes [R,C] and scale bytes [R,C/32] -> fp32 values (exact: a power of two times an e4m3 value)."""
+    R, C = q.shape
+    v = fp8_e4m3_decode(q).reshape(R, C // FP8_BLOCK, FP8_BLOCK)
+    return (v * np.exp2(b.astype(np.float32) - 127.0)[:, :, None]).astype(np.float32).reshape(R, C)
+
+
 def quantize_cols_fp8(w: np.ndarray) -> Tuple[np.ndarray, np.ndarray]:
     """Per-output-channel fp8 weights: w [..., K, N] -> (codes [..., K, N], scales [..., N])."""
     w = np.asarray(w, dtype=np.float32)
@@ -572,7 +601,8 @@ def expert_mlp(tokens, cnt, w1, w2, act: str, dtype: str = "bf16", w_up=None, ro
 def expert_up_fp8(tokens, cnt, wg_q, wg_s, wu_q, wu_s):
     """First half of the fp8 SwiGLU expert: bf16 rows quantised per token to e4m3, e4m3 weights with
     per-output-channel fp32 scales, fp32 accumulation, epilogue acc * s_tok[m] * s_ch[n], then
-    h = silu(g) * u rounded to bf16.  [S,H] -> [S,F]."""
+    h = silu(g) * u in fp32, block-quantised (quantize_blocks_fp8) without a rounding to bf16 in between.
+    [S,H] -> (codes [S,F] uint8, scale bytes [S,F/32] uint8)."""
     S, H = tokens.shape
     E_l = wg_q.shape[0]
     h = np.zeros((S, wg_q.shape[2]), dtype=np.float32)
@@ -588,28 +618,33 @@ def expert_up_fp8(tokens, cnt, wg_q, wg_s, wu_q, wu_s):
             u = ((xe @ fp8_e4m3_decode(wu_q[e])) * sx).astype(np.float32) * wu_s[e][None, :]
             h[r:r + c] = (act_silu(g.astype(np.float32)) * u.astype(np.float32)).astype(np.float32)
         r += c
-    return bf16_round(h)
+    return quantize_blocks_fp8(h)
 
 
-def expert_down_fp8(h, cnt, wd_q, wd_s):
-    """Second half: the bf16 hidden activation is re-quantised per row, multiplied by the e4m3 down
-    projection, scaled, and rounded to bf16.  [S,F] -> [S,H]."""
+def expert_down_fp8(hq, hsc, cnt, wd_q, wd_s, row_gate=None):
+    """Second half: the block-quantised hidden activation (codes, scale bytes) times the e4m3 down projection -- every
+    block of 32 k enters the sum with its power-of-two scale, fp32 accumulation -- then the channel scale (and the row's
+    gate where given: one more fp32 multiplication, of the channel scale), rounded to bf16.  -> [S,H]."""
     E_l = wd_q.shape[0]
-    y = np.zeros((h.shape[0], wd_q.shape[2]), dtype=np.float32)
-    hq, hs = quantize_rows_fp8(h)
-    hf = fp8_e4m3_decode(hq)
+    hf = dequantize_blocks_fp8(hq, hsc)
+    y = np.zeros((hf.shape[0], wd_q.shape[2]), dtype=np.float32)
     r = 0
     for e in range(E_l):
         c = int(cnt[e])
         if c:
-            y[r:r + c] = ((hf[r:r + c] @ fp8_e4m3_decode(wd_q[e])) * hs[r:r + c, None]).astype(np.float32) * wd_s[e][None, :]
+            acc = (hf[r:r + c] @ fp8_e4m3_decode(wd_q[e])).astype(np.float32)
+            if row_gate is None:
+                y[r:r + c] = acc * wd_s[e][None, :]
+            else:
+                y[r:r + c] = acc * (wd_s[e][None, :] * np.asarray(row_gate, np.float32)[r:r + c, None]).astype(np.float32)
         r += c
     return bf16_round(y)
 
 
-def expert_mlp_fp8(tokens, cnt, wg_q, wg_s, wu_q, wu_s, wd_q, wd_s):
+def expert_mlp_fp8(tokens, cnt, wg_q, wg_s, wu_q, wu_s, wd_q, wd_s, row_gate=None):
     """fp8 SwiGLU expert = expert_down_fp8(expert_up_fp8(x)).  Not in the reference."""
-    return expert_down_fp8(expert_up_fp8(tokens, cnt, wg_q, wg_s, wu_q, wu_s), cnt, wd_q, wd_s)
+    hq, hsc = expert_up_fp8(tokens, cnt, wg_q, wg_s, wu_q, wu_s)
+    return expert_down_fp8(hq, hsc, cnt, wd_q, wd_s, row_gate)
 
 
 # --------------------------------------------------------------------------------------

@@ -311,12 +311,37 @@ def test_quantize_rows_fp8_bit_exact(R, C):
     assert_bits_equal(q, oq, "fp8 codes")
 
 
+def _hidden_codes_close(hq_gpu, hsc_gpu, hq_want, hsc_want, what, min_same=0.995):
+    """The GPU's block-quantised hidden activation against the oracle's: fp32 sums in another order (and the hardware's exp /
+    reciprocal) move a value that sits on an e4m3 rounding boundary to the neighbouring code, and a block maximum that sits on a
+    power-of-two boundary to the neighbouring scale; everything else must be identical.  Bounds: at least `min_same` of the
+    codes and 99.9 % of the scale bytes identical, no scale byte off by more than one, every dequantised value within one
+    e4m3 step of the oracle's or within 2^-12 of its block's maximum."""
+    same_b = hsc_gpu == hsc_want
+    assert same_b.mean() >= 0.999, f"{what}: only {same_b.mean():.5f} of the block scales agree"
+    assert np.abs(hsc_gpu.astype(np.int32) - hsc_want.astype(np.int32)).max() <= 1, f"{what}: a block scale is off by more than one"
+    same_q = (hq_gpu == hq_want) & np.repeat(same_b, 32, axis=1)
+    got, want = O.dequantize_blocks_fp8(hq_gpu, hsc_gpu).astype(np.float64), O.dequantize_blocks_fp8(hq_want, hsc_want).astype(np.float64)
+    # (a value far below its block's maximum is a sum that nearly cancels: its fp32 summation noise, relative to the block
+    # maximum 448 X, is what bounds it -- 2^-12 of that, a few dozen of the block's smallest steps)
+    step = 2.0 ** -3 * np.abs(want) + 2.0 ** -12 * 448.0 * np.repeat(np.exp2(hsc_want.astype(np.float64) - 127.0), 32, axis=1)
+    bad = np.abs(got - want) > step + 1e-30
+    print(f"{what}: {same_q.mean():.6f} of the codes identical, {same_b.mean():.6f} of the block scales", flush=True)
+    assert same_q.mean() >= min_same, f"{what}: only {same_q.mean():.5f} of the codes agree"
+    if bad.any():
+        at = np.argwhere(bad)[:5]
+        detail = "; ".join(f"[{r},{c}] codes {hq_gpu[r, c]:#04x} / {hq_want[r, c]:#04x}, scale byte {hsc_want[r, c // 32]}, "
+                           f"values {got[r, c]:.6g} / {want[r, c]:.6g}" for r, c in at)
+        raise AssertionError(f"{what}: {int(bad.sum())} hidden activations are more than an e4m3 step from the oracle's: {detail}")
+
+
 @pytest.mark.parametrize("E_l,H,F,S", [(2, 256, 384, 400), (15, 2048, 1408, 2500), (1, 128, 128, 700)])
 def test_expert_mlp_fp8(E_l, H, F, S):
-    """The two GEMMs are checked separately with tight bounds (the second one against the oracle fed
-    with the GPU's own hidden activation).  End to end the bound is loose on purpose: re-quantising
-    a hidden row whose amax differs in its last bf16 bit moves a few per cent of that row's fp8 codes
-    by one step, which is a property of the two-stage quantisation, not of the kernels."""
+    """The two GEMMs are checked separately: the first one's block-quantised hidden activation (codes and scale bytes)
+    against the oracle's, identical but for values on a rounding boundary; the second one with the tight bf16 bound
+    against the oracle fed with the GPU's own codes and scales.  End to end the bound is looser on purpose: a hidden
+    value that takes the neighbouring e4m3 code moves the outputs of its row, which is a property of the quantisation,
+    not of the kernels."""
     rng = np.random.default_rng(H + F)
     cnt = _groups(rng, E_l, S)
     S_tot = int(cnt.sum())
@@ -330,11 +355,18 @@ def test_expert_mlp_fp8(E_l, H, F, S):
     ws = ops.fp8_workspace(S_tot, H, F, DEV)
     sg, su, sd = ew.scales
     out = to_np(ops.grouped_mlp_fp8(_t(x, "bf16"), torch.from_numpy(cnt).to(DEV), F, ew.w1, sg, su, ew.w2, sd, ws=ws))
-    h_gpu = to_np(ws["h"])
-    h_want = O.expert_up_fp8(x, cnt, gq, gs, uq, us)
-    _check(h_gpu, h_want.astype(np.float64), BF16_RTOL, BF16_ATOL, f"fp8 gate/up GEMM + SwiGLU E_l={E_l} H={H} F={F}")
-    y_from_gpu_h = O.expert_down_fp8(h_gpu, cnt, dq, ds)
+    hq_gpu, hsc_gpu = to_np(ws["hq"]), to_np(ws["hsc"])
+    hq_want, hsc_want = O.expert_up_fp8(x, cnt, gq, gs, uq, us)
+    _hidden_codes_close(hq_gpu, hsc_gpu, hq_want, hsc_want, f"fp8 gate/up GEMM + SwiGLU + block quantisation E_l={E_l} H={H} F={F}")
+    assert torch.equal(ops.dequantize_hidden_fp8(ws["hq"], ws["hsc"]).cpu(), torch.from_numpy(O.dequantize_blocks_fp8(hq_gpu, hsc_gpu)))
+    y_from_gpu_h = O.expert_down_fp8(hq_gpu, hsc_gpu, cnt, dq, ds)
     _check(out, y_from_gpu_h.astype(np.float64), BF16_RTOL, BF16_ATOL, f"fp8 down GEMM E_l={E_l} H={H} F={F}")
+    # the gate of the gated return, folded into the channel scale
+    gate = rng.random(S_tot).astype(np.float32)
+    out_g = to_np(ops.grouped_mlp_fp8(_t(x, "bf16"), torch.from_numpy(cnt).to(DEV), F, ew.w1, sg, su, ew.w2, sd, ws=ws,
+                                      row_gate=torch.from_numpy(gate).to(DEV)))
+    _check(out_g, O.expert_down_fp8(to_np(ws["hq"]), to_np(ws["hsc"]), cnt, dq, ds, row_gate=gate).astype(np.float64), BF16_RTOL,
+           BF16_ATOL, f"fp8 down GEMM with row gates E_l={E_l} H={H} F={F}")
     want = O.expert_mlp_fp8(x, cnt, gq, gs, uq, us, dq, ds)
     _check(out, want.astype(np.float64), FP8_RTOL, FP8_ATOL, f"expert_mlp_fp8 end to end E_l={E_l} H={H} F={F}")
     rms = float(np.sqrt(np.mean(want.astype(np.float64) ** 2)))
@@ -343,15 +375,15 @@ def test_expert_mlp_fp8(E_l, H, F, S):
     assert tight.mean() > 0.99
     # against the unquantised fp32 MLP, to show what the quantisation itself costs (reported only)
     ref = O.expert_mlp(x, cnt, wg, wd, "swiglu", "f32", w_up=wu)
-    print("fp8 vs unquantised fp32 MLP:", err_stats(out, ref.astype(np.float64)), flush=True)
+    print("fp8 vs unquantised fp32 MLP (max-abs, max-abs / rms, max-rel):", err_stats(out, ref.astype(np.float64)), flush=True)
 
 
 @pytest.mark.parametrize("E_l,H,F,rows", [(2, 2048, 1408, (300, 220)), (1, 512, 1024, (450,)), (3, 1024, 2048, (130, 0, 260))])
 def test_expert_mlp_fp8_k_split_of_the_last_round(E_l, H, F, rows):
     """The fp8 GEMMs with the partial-sum workspace: few tiles on an otherwise idle chip are cut along K and summed by the
-    reduction kernel, which applies the same scales and epilogue.  Each GEMM is held to the oracle on its own inputs
-    (as in test_expert_mlp_fp8), the result is reproducible from call to call whatever the workspace held, and it is
-    within a rounding step of the unsplit kernels'."""
+    reduction kernel, which applies the same scales, epilogue and block quantisation.  Each GEMM is held to the oracle on
+    its own inputs (as in test_expert_mlp_fp8), the result is reproducible from call to call whatever the workspace held,
+    and the hidden activation is that of the unsplit kernels but for values on a rounding boundary."""
     rng = np.random.default_rng(H + F + E_l)
     cnt = np.array(rows, dtype=np.int32)
     S_tot = int(cnt.sum())
@@ -375,11 +407,10 @@ def test_expert_mlp_fp8_k_split_of_the_last_round(E_l, H, F, rows):
     (split, ws1), (again, _) = outs
     assert torch.equal(split.view(torch.int16), again.view(torch.int16)), "the fp8 K split is not reproducible"
     assert bool(torch.isfinite(split.float()).all())
-    h_gpu = to_np(ws1["h"])
-    _check(h_gpu, O.expert_up_fp8(x, cnt, gq, gs, uq, us).astype(np.float64), BF16_RTOL, BF16_ATOL, "fp8 gate/up, K split")
-    _check(to_np(split), O.expert_down_fp8(h_gpu, cnt, dq, ds).astype(np.float64), BF16_RTOL, BF16_ATOL, "fp8 down, K split")
-    # against the unsplit kernels: the hidden activations within a rounding step (fp32 summation order)
-    a, b = ws1["h"].float(), plain_ws["h"].float()
-    assert bool(((a - b).abs() <= 2.0 ** -6 * torch.maximum(a.abs(), b.abs()) + 1e-6).all())
-    differs = int((ws1["h"].view(torch.int16) != plain_ws["h"].view(torch.int16)).sum().item())
-    print(f"fp8 K split: {differs} of {a.numel()} hidden activations differ in the last bits from the unsplit kernel", flush=True)
+    hq_gpu, hsc_gpu = to_np(ws1["hq"]), to_np(ws1["hsc"])
+    hq_want, hsc_want = O.expert_up_fp8(x, cnt, gq, gs, uq, us)
+    _hidden_codes_close(hq_gpu, hsc_gpu, hq_want, hsc_want, "fp8 gate/up, K split")
+    _check(to_np(split), O.expert_down_fp8(hq_gpu, hsc_gpu, cnt, dq, ds).astype(np.float64), BF16_RTOL, BF16_ATOL, "fp8 down, K split")
+    # against the unsplit kernels: the same codes but for fp32 sums in another order
+    _hidden_codes_close(hq_gpu, hsc_gpu, to_np(plain_ws["hq"]), to_np(plain_ws["hsc"]), "fp8 gate/up, K split against unsplit")
+    assert bool(torch.isfinite(plain.float()).all())

@@ -126,4 +126,4 @@ def test_fused_destination_equals_copies(name):
         q, sc = ops.quantize_rows_fp8(ref.send.view(-1, cfg.hidden))
         assert torch.equal(fused.send_q.view(-1, cfg.hidden), q) and torch.equal(fused.send_scale.view(-1), sc), \
             "quantise-and-pack differs from pack, then quantise"
-        assert torch.equal(fused.hidden.view(torch.int16), wire.hidden.view(torch.int16)), "hidden activations differ"
+        assert torch.equal(fused.hq, wire.hq) and torch.equal(fused.hsc, wire.hsc), "hidden activations differ"

@@ -25,14 +25,14 @@ def _shrunk(name, tokens):
     return cfg if tokens is None else replace(cfg, tokens=tokens)
 
 
-@pytest.mark.parametrize("name,tokens", [("small", None), ("mixtral", 2048), ("finegrained", 512)])
+@pytest.mark.parametrize("name,tokens", [("small", None), ("mixtral", 2048), ("finegrained", 512), ("zipf_k4", 1024)])
 def test_gated_return_against_oracle(name, tokens):
     cfg = _shrunk(name, tokens)
     print(f"case {cfg}", flush=True)
     W, E_l, k, H = cfg.world, cfg.e_local, cfg.topk, cfg.hidden
     world = harness.build_world(cfg, DEV)
     M, S = world.M, world.S
-    ew, raw, _ = harness.expert_weights(cfg, 0, DEV)
+    ew, raw, qs = harness.expert_weights(cfg, 0, DEV)
     recv_gate = harness.recv_gates(world)
     pipe = DispatchPipeline(world, ew, gated=True, recv_gate=recv_gate)
     pipe.step()
@@ -45,7 +45,13 @@ def test_gated_return_against_oracle(name, tokens):
     assert oM == M
     s0 = shards[0]
     # source side: the same send buffer as without gates, and the gates in their slots
-    assert_bits_equal(pipe.send, O.pack_fixed_m(O.send_payload(xs[0], s0["row_token"]), s0["offs"], s0["sizes"], M), "send")
+    o_send = O.pack_fixed_m(O.send_payload(xs[0], s0["row_token"]), s0["offs"], s0["sizes"], M)
+    if pipe.fp8_dispatch:
+        o_q, o_sc = O.pack_fixed_m_fp8(O.send_payload(xs[0], s0["row_token"]), s0["offs"], s0["sizes"], M)
+        assert_bits_equal(pipe.send_q, o_q, "send codes")
+        assert_bits_equal(pipe.send_scale, o_sc, "send scales")
+    else:
+        assert_bits_equal(pipe.send, o_send, "send")
     assert_bits_equal(pipe.send_gate, O.pack_gates(to_np(pipe.gate), s0["idx"], s0["pos"], s0["offs"], E_l, W, M), "send_gate")
     # what arrives at rank 0: source s's gates for destination 0 (the harness assembled them with the same kernel)
     o_rg = np.stack([O.pack_gates(sh["gate"], sh["idx"], sh["pos"], sh["offs"], E_l, W, M)[0] for sh in shards])
@@ -58,7 +64,11 @@ def test_gated_return_against_oracle(name, tokens):
     rows = O.unpack_expert_major(o_recv, o_rc)
     cnt = O.expert_row_counts(o_rc.T)
     f = to_np
-    if cfg.act == "swiglu":
+    if cfg.quant == "fp8":
+        # the down projection on the GPU's own block-quantised hidden activation (the first GEMM is held to the oracle elsewhere)
+        (_, _), (_, _), (dq, ds) = [(f(q), f(s_)) for q, s_ in qs]
+        y = O.expert_down_fp8(f(pipe.hq), f(pipe.hsc), cnt, dq, ds, row_gate=g_rows)
+    elif cfg.act == "swiglu":
         y = O.expert_mlp(rows, cnt, f(raw[0]), f(raw[2]), "swiglu", cfg.dtype, w_up=f(raw[1]), row_gate=g_rows)
     else:
         y = O.expert_mlp(rows, cnt, f(raw[0]), f(raw[1]), cfg.act, cfg.dtype, row_gate=g_rows)

@@ -81,6 +81,25 @@ def _close(got, ref, what, rtol=2.0 ** -7, atol=2.0 ** -7):
     assert not bool(bad.any()), f"{what}: {int(bad.sum())} of {bad.numel()} elements outside tolerance"
 
 
+def _close_fp8_hidden(hq, hsc, ref, what):
+    """The block-quantised hidden activation of the fp8 expert (codes, scale bytes) against an fp32 evaluation of what was
+    quantised: every dequantised value within one e4m3 step of the reference (2^-3 of its magnitude) or within 2^-11 of its
+    block's maximum (the fp32 summation noise of values that nearly cancel, and the block's smallest steps), and every block scale the
+    smallest power of two that fits the reference's block maximum, give or take one where that maximum sits on a boundary."""
+    got = ops.dequantize_hidden_fp8(hq, hsc)
+    S, F = ref.shape
+    amax = ref.abs().view(S, F // 32, 32).amax(dim=2)
+    floor = (amax * 2.0 ** -11).repeat_interleave(32, dim=1)  # (2^-12 of the largest value the block's scale admits: sums that nearly cancel)
+    err = (got - ref).abs()
+    bad = err > 2.0 ** -3 * ref.abs() + floor + 1e-30
+    print(f"{what}: {got.numel()} elements, max-abs {float(err.max()):.3e}, {float((err <= 2.0 ** -4 * 1.01 * ref.abs() + floor).float().mean()):.6f} "
+          f"within half a step", flush=True)
+    assert not bool(bad.any()), f"{what}: {int(bad.sum())} of {bad.numel()} hidden activations further than an e4m3 step from the fp32 value"
+    want_b = torch.ceil(torch.log2(torch.clamp(amax.double(), min=1e-300) / 448.0)).clamp(min=-127.0) + 127.0
+    off = (hsc.double() - want_b).abs()
+    assert float(off.max()) <= 1 and float((off == 0).double().mean()) > 0.999, f"{what}: block scales"
+
+
 def _ref_gemm(X, W, cnt):
     """Per-expert fp32 PyTorch GEMM (vendor BLAS), the reference the reference itself intended
     (unit_tests.py:231-235)."""
@@ -162,15 +181,15 @@ def test_fp8_gemms_every_tile_at_full_size(name):
             u = (xd[r0:r0 + c] @ _dec(uq[e])) * sx * us[e][None, :]
             h_ref[r0:r0 + c] = torch.nn.functional.silu(g) * u
         r0 += c
-    _close(ws["h"], h_ref, f"{name} fp8 gate/up GEMM + SwiGLU vs fp32")
+    _close_fp8_hidden(ws["hq"], ws["hsc"], h_ref, f"{name} fp8 gate/up GEMM + SwiGLU + block quantisation vs fp32")
     del h_ref, xd
-    hd = _dec(ws["hq"])
-    _freivalds(y, hd, _dec(dq), cnt, f"{name} fp8 down GEMM", col_scale=ds, row_scale=ws["hs"])
+    hd = ops.dequantize_hidden_fp8(ws["hq"], ws["hsc"])  # the operand values of the down projection, exactly
+    _freivalds(y, hd, _dec(dq), cnt, f"{name} fp8 down GEMM", col_scale=ds)
     y_ref = torch.empty((S, H), dtype=torch.float32, device=DEV)
     r0 = 0
     for e, c in enumerate(cnt):
         if c:
-            y_ref[r0:r0 + c] = (hd[r0:r0 + c] @ _dec(dq[e])) * ws["hs"][r0:r0 + c, None] * ds[e][None, :]
+            y_ref[r0:r0 + c] = (hd[r0:r0 + c] @ _dec(dq[e])) * ds[e][None, :]
         r0 += c
     _close(y, y_ref, f"{name} fp8 down GEMM vs fp32")
 
@@ -302,7 +321,7 @@ def test_fp8_mlp_over_random_shapes():
         ws = ops.fp8_workspace(S, H, F, DEV)
         y = ops.grouped_mlp_fp8(x, torch.from_numpy(cnt).to(DEV), F, p1, gs, us, p2, ds, ws=ws, part_ws=part if split else None)
         torch.cuda.synchronize()
-        xd, hd = _dec(ws["xq"]), _dec(ws["hq"])
+        xd, hd = _dec(ws["xq"]), ops.dequantize_hidden_fp8(ws["hq"], ws["hsc"])
         h_ref = torch.empty((S, F), dtype=torch.float32, device=DEV)
         y_ref = torch.empty((S, H), dtype=torch.float32, device=DEV)
         r0 = 0
@@ -312,7 +331,7 @@ def test_fp8_mlp_over_random_shapes():
                 g = (xd[r0:r0 + c] @ _dec(gq[e])) * sx * gs[e][None, :]
                 u = (xd[r0:r0 + c] @ _dec(uq[e])) * sx * us[e][None, :]
                 h_ref[r0:r0 + c] = torch.nn.functional.silu(g) * u
-                y_ref[r0:r0 + c] = (hd[r0:r0 + c] @ _dec(dq[e])) * ws["hs"][r0:r0 + c, None] * ds[e][None, :]
+                y_ref[r0:r0 + c] = (hd[r0:r0 + c] @ _dec(dq[e])) * ds[e][None, :]
             r0 += c
-        _close(ws["h"], h_ref, f"case {case} gate/up + SwiGLU")
+        _close_fp8_hidden(ws["hq"], ws["hsc"], h_ref, f"case {case} gate/up + SwiGLU + block quantisation")
         _close(y, y_ref, f"case {case} down")

@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/moe_gfx950.h but not exported"
     assert sorted(L.exported_symbols()) == declared, "ctypes table and header disagree"
-    assert lib.moe_abi_version() == 2
+    assert lib.moe_abi_version() == 3
     assert lib.moe_last_error() == b""
 
 
@@ -131,3 +131,14 @@ def test_bench_refuses_more_than_one_gpu():
     import sys
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert r.returncode == 2 and "--gpus must be 1" in r.stderr and r.stdout.strip() == ""
+
+
+def test_ctypes_table_has_the_argument_count_of_every_declaration():
+    """Every entry of the ctypes signature table has as many arguments as the header's declaration of that symbol."""
+    from iris_testing_amd import _lib as L
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "moe_gfx950.h")).read(), flags=re.S)
+    for name, (_, args) in L._SIGNATURES.items():
+        m = re.search(r"\b" + name + r"\s*\(([^;]*?)\)\s*;", text, re.S)
+        assert m, f"{name} is not declared"
+        params = [x for x in m.group(1).split(",") if x.strip() and x.strip() != "void"]
+        assert len(params) == len(args), f"{name}: header declares {len(params)} arguments, the ctypes table {len(args)}"

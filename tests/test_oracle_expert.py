@@ -71,11 +71,33 @@ def test_fp8_mlp_is_the_dequantised_mlp():
     assert np.abs(out - ref).max() < 0.25 * rms  # fp8 noise, far below signal
 
 
-def _fp8_explicit(x, cnt, gq, gs, uq, us, dq, ds, swap_scales=False, per_expert_scale=False, swap_gate_up=False):
-    """The fp8 SwiGLU expert spelled out with torch's own e4m3 / bf16 casts and float64 arithmetic:
+def _block_quant_torch(h32, block=32, mantissa_rule=True):
+    """Block quantisation spelled out with torch: scale = 2^ceil(log2(amax / 448)) per row and `block` columns (float64
+    logarithm: amax / 448 is a power of two only when it is one exactly, so the ceiling is safe), at least 2^-127; codes with
+    torch's own float8_e4m3fn cast.  mantissa_rule=False plants the scale 2^(floor(log2 amax) - 8), which lets the largest
+    values of a block run past 448.  Returns (codes as float64 values [R,C], scales float64 [R, C/block])."""
+    import torch
+    R, C = h32.shape
+    hb = h32.view(R, C // block, block)
+    amax = hb.abs().amax(dim=2).double()
+    safe = torch.where(amax == 0, torch.ones_like(amax), amax)
+    if mantissa_rule:
+        e = torch.ceil(torch.log2(safe / 448.0))
+    else:
+        e = torch.floor(torch.log2(safe)) - 8
+    e = torch.where(amax == 0, torch.full_like(e, -127.0), e).clamp(min=-127.0)
+    X = torch.exp2(e)
+    q = (hb.double() / X[:, :, None]).float().clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+    return q.double().view(R, C), X
+
+
+def _fp8_explicit(x, cnt, gq, gs, uq, us, dq, ds, swap_scales=False, per_expert_scale=False, swap_gate_up=False, block=32,
+                  mantissa_rule=True, gate=None):
+    """The fp8 SwiGLU expert spelled out with torch's own e4m3 casts and float64 arithmetic:
     quantise rows (amax/448), decode every code with torch.float8_e4m3fn, multiply in float64, scale by
-    s_tok[m] * s_ch[n], SwiGLU, round to bf16, re-quantise, multiply, scale, round.  The keyword arguments
-    plant the plausible mistakes.  Returns (hidden [S,F], out [S,H]) as float32 arrays."""
+    s_tok[m] * s_ch[n], SwiGLU, block-quantise the fp32 result (_block_quant_torch), multiply the dequantised blocks,
+    scale by the channel scale (and the row gate), round to bf16.  The keyword arguments plant the plausible mistakes.
+    Returns (dequantised hidden [S,F] float64, out [S,H] float32)."""
     import torch
     dec = lambda q: torch.from_numpy(np.ascontiguousarray(q)).view(torch.float8_e4m3fn).double()  # noqa: E731
 
@@ -106,16 +128,24 @@ def _fp8_explicit(x, cnt, gq, gs, uq, us, dq, ds, swap_scales=False, per_expert_
                 g, u = u, g
             h[r:r + c] = g / (1.0 + torch.exp(-g)) * u
         r += c
-    hb = h.float().bfloat16().float()
-    hq, hs = quant_rows(hb)
+    hq, X = _block_quant_torch(h.float(), block, mantissa_rule)
+    hd = (hq.view(S, F // block, block) * X[:, :, None]).view(S, F)
     y = torch.zeros((S, dq.shape[2]), dtype=torch.float64)
     r = 0
     for e, c in enumerate(cnt):
         c = int(c)
         if c:
-            y[r:r + c] = (hq[r:r + c] @ dec(dq[e])) * hs[r:r + c, None].double() * torch.from_numpy(ds[e]).double()[None, :]
+            y[r:r + c] = (hd[r:r + c] @ dec(dq[e])) * torch.from_numpy(ds[e]).double()[None, :]
+            if gate is not None:
+                y[r:r + c] *= torch.from_numpy(gate[r:r + c]).double()[:, None]
         r += c
-    return hb.numpy(), y.float().bfloat16().float().numpy()
+    return hd.numpy(), y.float().bfloat16().float().numpy()
+
+
+def _within_an_fp8_step(got, ref):
+    """|got - ref| <= 2^-3 |ref| + 2^-9 max|ref| of the row: one e4m3 rounding step of a value inside its block."""
+    floor = 2.0 ** -9 * np.abs(ref).max(axis=1, keepdims=True)
+    return np.abs(got.astype(np.float64) - ref) <= 2.0 ** -3 * np.abs(ref) + floor
 
 
 def _within_a_bf16_step(got, ref):
@@ -123,6 +153,37 @@ def _within_a_bf16_step(got, ref):
     a rounding) and a floor for outputs that cancel to almost nothing."""
     rms = float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))
     return np.abs(got.astype(np.float64) - ref) <= 2.0 ** -7 * np.abs(ref) + 2.0 ** -10 * rms
+
+
+def test_fp8_block_quantisation_against_torch():
+    """quantize_blocks_fp8 (integer arithmetic on the bits of the block maximum) against the logarithm-and-ceiling form with
+    torch's own e4m3 cast, codes and scale bytes bit for bit: values over twelve binades, blocks whose maximum is 448 2^k
+    exactly (the scale must not move up there), one ulp above it (it must), all-zero blocks, tiny values."""
+    import torch
+    rng = np.random.default_rng(31)
+    R, C = 64, 256
+    x = (rng.standard_normal((R, C)) * np.exp2(rng.integers(-6, 6, (R, C // 32)).repeat(32, axis=1))).astype(np.float32)
+    x[0, :32] = 0.0
+    x[1, 32:64] = np.float32(1e-40)
+    for k, row in zip((-3, 0, 5), (2, 3, 4)):
+        x[row, :32] = np.clip(x[row, :32], -1, 1) * np.float32(2.0 ** k)
+        x[row, 7] = np.float32(448.0 * 2.0 ** k)                                   # amax = 448 2^k: fits exactly
+        x[row, 64:96] = np.clip(x[row, 64:96], -1, 1) * np.float32(2.0 ** k)
+        x[row, 70] = np.nextafter(np.float32(448.0 * 2.0 ** k), np.float32(np.inf))  # one ulp more: the next power of two
+    q, b = O.quantize_blocks_fp8(x)
+    qt, X = _block_quant_torch(torch.from_numpy(x))
+    assert np.array_equal(np.exp2(b.astype(np.float64) - 127.0), X.numpy()), "scale bytes"
+    assert np.array_equal(O.fp8_e4m3_decode(q).astype(np.float64), qt.numpy()), "codes"
+    assert b[2, 0] + 1 == b[2, 2] and b[3, 0] + 1 == b[3, 2] and b[4, 0] + 1 == b[4, 2]
+    assert b[0, 0] == 0 and (q[0, :32] == 0).all()
+    # nothing saturates: every block's largest code is at most 448, and at least 224 (the scale is the smallest that fits) unless it sits at its floor
+    top = np.abs(O.fp8_e4m3_decode(q)).reshape(R, C // 32, 32).max(axis=2)
+    assert (top <= 448).all() and (top[b > 0] >= 224).all()
+    # dequantisation is the exact product
+    assert np.array_equal(O.dequantize_blocks_fp8(q, b).astype(np.float64), qt.numpy() * X.numpy().repeat(32, axis=1))
+    # planted: the scale without the mantissa rule overflows the largest values of about half the blocks
+    qb, Xb = _block_quant_torch(torch.from_numpy(x), mantissa_rule=False)
+    assert (Xb.numpy() != X.numpy()).mean() > 0.1
 
 
 def test_fp8_expert_halves_against_an_explicit_dequantised_evaluation():
@@ -136,20 +197,37 @@ def test_fp8_expert_halves_against_an_explicit_dequantised_evaluation():
     wu = (rng.standard_normal((E_l, H, Fd)) * rng.uniform(0.25, 2.0, (E_l, 1, Fd)) / np.sqrt(H)).astype(np.float32)
     wd = (rng.standard_normal((E_l, Fd, H)) * rng.uniform(0.25, 2.0, (E_l, 1, H)) / np.sqrt(Fd)).astype(np.float32)
     (gq, gs), (uq, us), (dq, ds) = (O.quantize_cols_fp8(w) for w in (wg, wu, wd))
-    h_ref, _ = _fp8_explicit(x, cnt, gq, gs, uq, us, dq, ds)
-    h = O.expert_up_fp8(x, cnt, gq, gs, uq, us)
-    assert _within_a_bf16_step(h, h_ref).all(), "expert_up_fp8 differs from the explicit evaluation"
-    # the second half on the same hidden activation (the explicit evaluation re-quantises what it is given)
-    _, y_ref = _fp8_explicit(x, cnt, gq, gs, uq, us, dq, ds)
-    y = O.expert_down_fp8(h_ref, cnt, dq, ds)
-    assert _within_a_bf16_step(y, y_ref).all(), "expert_down_fp8 differs from the explicit evaluation"
-    # planted mistakes must fail the same bound, by a wide margin
-    for kw in (dict(swap_scales=True), dict(per_expert_scale=True), dict(swap_gate_up=True)):
-        h_bad, y_bad = _fp8_explicit(x, cnt, gq, gs, uq, us, dq, ds, **kw)
-        frac = 1.0 - _within_a_bf16_step(h, h_bad).mean()
-        assert frac > 0.5, f"{kw}: only {frac:.2f} of the hidden activations notice"
-    # the row quantisation on its own, codes and scales, against torch's cast
+    h_ref, y_ref = _fp8_explicit(x, cnt, gq, gs, uq, us, dq, ds)
+    hq, hsc = O.expert_up_fp8(x, cnt, gq, gs, uq, us)
+    h = O.dequantize_blocks_fp8(hq, hsc)
+    # fp32 against float64 sums: a value that sits on an e4m3 rounding boundary may take the neighbouring code, nothing more
+    assert _within_an_fp8_step(h, h_ref).all(), "expert_up_fp8 differs from the explicit evaluation"
+    assert (h == h_ref).mean() > 0.98, "too many hidden activations differ from the explicit evaluation"
+    # the second half on the oracle's own hidden activation, against the same products in float64
     import torch
+    dec = lambda q: torch.from_numpy(np.ascontiguousarray(q)).view(torch.float8_e4m3fn).double().numpy()  # noqa: E731
+    gate = rng.random(S).astype(np.float32)
+    for g_ in (None, gate):
+        y = O.expert_down_fp8(hq, hsc, cnt, dq, ds, row_gate=g_)
+        want = np.zeros((S, H))
+        r = 0
+        for e, c in enumerate(cnt):
+            want[r:r + c] = (h[r:r + c].astype(np.float64) @ dec(dq[e])) * ds[e][None, :].astype(np.float64)
+            r += c
+        if g_ is not None:
+            want *= g_[:, None].astype(np.float64)
+        assert _within_a_bf16_step(y, want).all(), "expert_down_fp8 differs from the explicit evaluation"
+    assert _within_a_bf16_step(O.expert_mlp_fp8(x, cnt, gq, gs, uq, us, dq, ds), y_ref).mean() > 0.9  # (end to end: code flips move a few outputs)
+    # planted mistakes: where the right evaluation reproduces more than 98 % of the hidden activations exactly, each of
+    # these reproduces less than half (and leaves a good part of them further than an e4m3 step away)
+    for kw in (dict(swap_scales=True), dict(per_expert_scale=True), dict(swap_gate_up=True)):
+        h_bad, _ = _fp8_explicit(x, cnt, gq, gs, uq, us, dq, ds, **kw)
+        same = (h == h_bad).mean()
+        assert same < 0.5, f"{kw}: {same:.2f} of the hidden activations are unchanged"
+        assert 1.0 - _within_an_fp8_step(h, h_bad).mean() > 0.15, kw
+    # (the block size and the scale rule are pinned by test_fp8_block_quantisation_against_torch, bytes and codes bit for
+    # bit: with power-of-two scales they only show in a block's smallest values, which is why they are not planted here)
+    # the row quantisation on its own, codes and scales, against torch's cast
     q, s = O.quantize_rows_fp8(x)
     xt = torch.from_numpy(x)
     amax = xt.abs().amax(dim=1)
