@@ -2,7 +2,7 @@
 """Routed tokens/s through the MoE dispatch + expert + combine hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config mixtral] [--no-cpu-baseline]
-                    [--unfused | --gated | --padding-free] [--backward] [--stream-ceiling]
+                    [--unfused | --gated | --padding-free] [--backward] [--stream-ceiling] [--mfma-ceiling]
 
 A "step" is one pass of rank 0's share of the path over one batch of synthetic tokens (see
 iris_testing_amd/pipeline.py): route + count + pack as a source, unpack + grouped expert MLP + return
@@ -204,12 +204,34 @@ def backward_leg(cfg, world, raw, steps):
     }
 
 
-def stream_ceiling_leg(cfg, steps):
+def mfma_ceiling_leg(steps):
+    """What the matrix cores sustain from registers (moe_diag_mfma_loop: the grouped GEMM's wave layout, no LDS, no memory),
+    on all-zero operands and on operands drawn like N(0,1): the chip runs against a power limit, so the second figure, not the
+    published peak, is what a GEMM on the workload's data can approach."""
+    import torch
+    L_ = __import__("iris_testing_amd._lib", fromlist=["x"])
+    lib = L_.lib()
+    sink = torch.empty(lib.moe_diag_mfma_loop_sink_floats(), dtype=torch.float32, device="cuda")
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    out = {"what": "register-only MFMA loop, 4 waves per compute unit, 128 x 128 outputs per wave (bf16: 16x16x32, fp8: 32x32x64)",
+           "workgroups": cus}
+    for fp8, name, peak in ((0, "bf16", PEAK["mfma_bf16"]), (1, "fp8", PEAK["mfma_fp8"])):
+        for rnd, dname in ((0, "zeros"), (1, "normal")):
+            iters = 100000  # (about 50 ms per launch, several launches back to back: the power limit acts on sustained load)
+            fl = lib.moe_diag_mfma_loop_flops(fp8, iters, cus)
+            ms = _timed(lambda: L_.check(lib.moe_diag_mfma_loop(fp8, rnd, iters, cus, L_.ptr(sink), L_.stream_ptr())), max(steps, 3), torch)
+            out[f"{name}_{dname}"] = {"ms": round(ms, 3), "TFLOP/s": round(fl / ms / 1e9, 1), "frac_of_published_peak": round(fl / ms / 1e9 / peak, 4)}
+    return out
+
+
+def stream_ceiling_leg(cfg, steps, world=None):
     """What the memory system sustains for the three traffic mixes of the row-moving stages, measured with the product's own
     kernels on buffers of 1 GiB: a plain row copy (moe_pack_payload with the identity map: one byte read per byte written),
     a pure write (moe_zero_padding_rows over a buffer that is all padding) and read-mostly sums (moe_combine with unit gates
     and k rows read per row written).  From the first two, the read rate R and write rate W of the model
-    time = read bytes / R + written bytes / W."""
+    time = read bytes / R + written bytes / W.  Then the same three at the sizes of this workload's own stages (the copy on
+    as many rows as the unpack moves, the sums on as many tokens as the combine, slots in sequence): a launch's start-up
+    and drain do not shrink with the buffer, so the rates of a 0.4 GB launch are lower than those of a 2 GB one."""
     import torch
     from iris_testing_amd import ops
     dev = "cuda"
@@ -255,6 +277,28 @@ def stream_ceiling_leg(cfg, steps):
         model_ms = (rd / read_rate + wr / write_rate) / 1e6
         out["combine_unit_gates"][f"k={k}"] = {"ms": round(ms, 4), "GB/s": round((rd + wr) / ms / 1e6, 1), "read_share": round(rd / (rd + wr), 3),
                                                 "model_GB/s": round((rd + wr) / model_ms / 1e6, 1)}
+    if world is not None and cfg.dtype == "bf16":
+        # the same kernels at this workload's sizes
+        S, T, k = world.S, cfg.tokens, cfg.topk
+        n_copy = min(S, rows)
+
+        def copy_w():
+            L_.check(lib.moe_pack_payload(p(src), 1, rows, H, p(ident), n_copy, p(dst), st()))
+        ms_c = _timed(copy_w, steps, torch)
+        n_slots = min(T * k, rows)
+        Tw = n_slots // k
+        idx = torch.zeros((Tw, k), dtype=torch.int32, device=dev)
+        pos = (torch.arange(Tw, device=dev, dtype=torch.int32)[:, None] + Tw * torch.arange(k, device=dev, dtype=torch.int32)[None, :]).contiguous()
+        zero = torch.zeros(1, dtype=torch.int32, device=dev)
+        o = torch.empty((Tw, H), dtype=torch.bfloat16, device=dev)
+
+        def comb_w():
+            L_.check(lib.moe_combine(p(src), 1, 1, rows, H, p(idx), p(pos), None, p(zero), Tw, k, 1, p(o), None, st()))
+        ms_s = _timed(comb_w, steps, torch)
+        out["at_workload_size"] = {
+            "copy": {"rows": n_copy, "MB": round(2 * n_copy * H * B / 1e6, 1), "ms": round(ms_c, 4), "GB/s": round(2 * n_copy * H * B / ms_c / 1e6, 1)},
+            "combine_unit_gates": {"tokens": Tw, "k": k, "MB": round((Tw * k + Tw) * H * B / 1e6, 1), "ms": round(ms_s, 4),
+                                   "GB/s": round((Tw * k + Tw) * H * B / ms_s / 1e6, 1)}}
     return out
 
 
@@ -281,6 +325,8 @@ def main():
     ap.add_argument("--backward", action="store_true", help="also time forward + backward of rank 0's expert MLP")
     ap.add_argument("--stream-ceiling", action="store_true",
                     help="also measure copy / write / read-mostly rates of the row-moving kernels on 1 GiB buffers")
+    ap.add_argument("--mfma-ceiling", action="store_true",
+                    help="also measure what the matrix cores sustain from registers, on all-zero and on N(0,1)-like operands")
     ap.add_argument("--cpu-sample-tokens", type=int, default=0, help="0 = sized for roughly 10-30 s")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -429,7 +475,9 @@ def main():
         else:
             out["backward"] = backward_leg(cfg, world, raw, max(args.steps // 4, 2))
     if args.stream_ceiling:
-        out["stream_ceiling"] = stream_ceiling_leg(cfg, max(args.steps // 2, 3))
+        out["stream_ceiling"] = stream_ceiling_leg(cfg, max(args.steps // 2, 3), world)
+    if args.mfma_ceiling:
+        out["mfma_ceiling"] = mfma_ceiling_leg(max(args.steps // 4, 3))
 
     if not args.no_cpu_baseline:
         def to_np(t):

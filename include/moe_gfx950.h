@@ -362,6 +362,16 @@ int moe_combine(const void* ret, int dtype, int W, int M, int H, const int32_t* 
                 const float* gate, const int32_t* dst_offsets, int T, int k, int E_l, void* out,
                 int32_t* status, moe_stream_t stream);
 
+/* ---- diagnostics (no counterpart in the reference, no part of the hot path) ------------------------------------------
+ * moe_diag_mfma_loop: a register-only MFMA loop in the grouped GEMM's wave layout (4 waves per workgroup, 128 x 128 outputs per
+ * wave; bf16 on 16x16x32, fp8 on 32x32x64), `workgroups` workgroups, `iters` passes over the wave's MFMA tiles; operands all
+ * zero (random_data = 0) or drawn like N(0,1) (random_data = 1: the matrix cores run against a power limit, and what they
+ * sustain depends on the operand values).  sink: moe_diag_mfma_loop_sink_floats() floats of scratch.  The caller times the
+ * launch; moe_diag_mfma_loop_flops gives its flop count.  Used by `bench.py --mfma-ceiling`. */
+size_t moe_diag_mfma_loop_sink_floats(void);
+double moe_diag_mfma_loop_flops(int fp8, int iters, int workgroups);
+int moe_diag_mfma_loop(int fp8, int random_data, int iters, int workgroups, float* sink, moe_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

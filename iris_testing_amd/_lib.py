@@ -80,6 +80,9 @@ _SIGNATURES = {
     "moe_zero_padding_rows": (c_int, [P, c_int, c_int, c_int, c_int, P, c_int, P]),
     "moe_grouped_mlp_fp8_mapped": (c_int, [P, c_int, P, P, c_int, c_int, c_int, c_int, P, P, P, P, P, P, P, P, P, P, P, c_int, P, P,
                                            c_size_t, P]),  # (.., xq_ws, xs_ws, hq_ws, hscale_ws, row_gate, out, out_rows, ..)
+    "moe_diag_mfma_loop_sink_floats": (c_size_t, []),
+    "moe_diag_mfma_loop_flops": (ctypes.c_double, [c_int, c_int, c_int]),
+    "moe_diag_mfma_loop": (c_int, [c_int, c_int, c_int, c_int, P, P]),
     "moe_combine": (c_int, [P, c_int, c_int, c_int, c_int, P, P, P, P, c_int, c_int, c_int, P, P, P]),
 }
 

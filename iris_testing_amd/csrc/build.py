@@ -11,7 +11,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "libmoe_gfx950.so")
-SOURCES = ["capi.hip", "route.hip", "dispatch.hip", "grouped_gemm.hip"]
+SOURCES = ["capi.hip", "route.hip", "dispatch.hip", "grouped_gemm.hip", "diag.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
@@ -38,7 +38,7 @@ def _compile(src: str, verbose: bool) -> str:
 
 def build(verbose: bool = True) -> str:
     srcs = [s for s in SOURCES if os.path.exists(os.path.join(HERE, s))]
-    with ThreadPoolExecutor(max_workers=4) as ex:
+    with ThreadPoolExecutor(max_workers=5) as ex:
         objs = list(ex.map(lambda s: _compile(s, verbose), srcs))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     if verbose:

@@ -68,10 +68,31 @@ typedef float rt_f4 __attribute__((ext_vector_type(4)));
 typedef float rt_f16 __attribute__((ext_vector_type(16)));
 typedef unsigned int rt_u4 __attribute__((ext_vector_type(4)));
 
-template <typename XT, int SHAPE, int TB, int G, int NWV, int CPR /* 16-byte chunks of a token row per slab */>
-__global__ __launch_bounds__(NWV * WAVE, (NWV == 4 && TB == 2 ? 2 : 1)) void route_logits_mfma_kernel(const XT* __restrict__ x, const XT* __restrict__ w,
-                                                                        float* __restrict__ part /*[RT_P][T][E]*/, int T,
-                                                                        int Hrow, int E) {
+// One segment chain of a team of NWV waves for NTOK tokens and EB experts: the accumulators of the calling wave.
+// TEAM1 = false: the team is the whole workgroup (block barriers around every slab).  TEAM1 = true: the team is the calling
+// wave alone (NWV = 1), xs / wsT are its private part of the LDS and the hand-overs between its lanes are wave-local ones,
+// so that the waves of a workgroup -- one segment each -- run independently.
+template <bool TEAM1>
+__device__ __forceinline__ void rt_team_sync() {
+    if constexpr (TEAM1) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    } else {
+        __syncthreads();
+    }
+}
+
+template <int SHAPE>
+struct RtAcc {
+    typedef typename std::conditional<SHAPE == 16, rt_f16, rt_f4>::type type;
+};
+
+template <typename XT, int SHAPE, int TB, int G, int NWV, int CPR /* 16-byte chunks of a token row per slab */, bool TEAM1, int D>
+__device__ __forceinline__ void route_segment_chain(const XT* __restrict__ x, const XT* __restrict__ w, int T, int Hrow, int E, int seg,
+                                                    int t0, int eb0, int tid, int wave, float (*xs)[CPR * VecLoad<XT>::N + 4],
+                                                    float (*wsT)[CPR * VecLoad<XT>::N + 4],
+                                                    typename RtAcc<SHAPE>::type (&acc)[TB][G]) {
     static_assert(SHAPE == 4 || SHAPE == 16, "experts per MFMA");
     constexpr int NTH = NWV * WAVE;
     constexpr int NTOK = TB * RT_TB;           // tokens per block
@@ -79,23 +100,15 @@ __global__ __launch_bounds__(NWV * WAVE, (NWV == 4 && TB == 2 ? 2 : 1)) void rou
     constexpr int VN = VecLoad<XT>::N;         // elements per 16 bytes
     constexpr int KC = CPR * VN;               // h per slab: CPR x 16 bytes of every token row
     constexpr int NCH = CPR;                   // chunks (VN consecutive h) per slab
-    constexpr int XS = KC + 4;                 // padded fp32 row (conflict-free 128-bit row reads)
     constexpr int XPT = NTOK * CPR / NTH;      // 16-byte x chunks per thread and slab
     constexpr int WQ = KC * EB / (4 * NTH);    // groups of four h of one expert per thread and slab
-    // slabs in flight per block (in registers, until their turn in LDS)
-    constexpr int D = 2;
+    // D: slabs in flight per team (in registers, until their turn in LDS)
     constexpr int NACC = SHAPE == 16 ? 16 : 4;
-    typedef typename std::conditional<SHAPE == 16, rt_f16, rt_f4>::type acc_t;
-    static_assert((KC * EB) % (4 * NTH) == 0 && (NTOK * CPR) % NTH == 0 && (CPR == 8 || CPR == 16), "router slab split");
-    __shared__ __align__(16) float xs[NTOK][XS];
-    __shared__ __align__(16) float wsT[EB][KC + 4];
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    // (the segment is the fastest-running block index: the blocks that are resident together then read whole token
-    // rows between them, not the same eighth of every row, which would load the memory channels unevenly)
-    const int t0 = blockIdx.y * NTOK, eb0 = blockIdx.z * EB;
-    // this block's segment of the reduction: h in [h0, h0 + H) of rows that are Hrow long (H = 0: an empty segment)
-    const int seg = blockIdx.x, seg_len = route_segment_len(Hrow);
+    static_assert((KC * EB) % (4 * NTH) == 0 && (NTOK * CPR) % NTH == 0 && (CPR == 4 || CPR == 8 || CPR == 16), "router slab split");
+    static_assert(!TEAM1 || NWV == 1, "a team of one wave");
+    const int lane = tid & 63;
+    // this team's segment of the reduction: h in [h0, h0 + H) of rows that are Hrow long (H = 0: an empty segment)
+    const int seg_len = route_segment_len(Hrow);
     const int h0 = min(seg * seg_len, Hrow);
     const int H = min(seg_len, Hrow - h0);
     const float* wrow[G];
@@ -104,7 +117,6 @@ __global__ __launch_bounds__(NWV * WAVE, (NWV == 4 && TB == 2 ? 2 : 1)) void rou
     for (int g = 0; g < G; ++g) wrow[g] = &wsT[(wave * G + g) * SHAPE + lane % SHAPE][0];
 #pragma unroll
     for (int b = 0; b < TB; ++b) xrow[b] = &xs[b * RT_TB + lane][0];
-    acc_t acc[TB][G];
 #pragma unroll
     for (int b = 0; b < TB; ++b)
 #pragma unroll
@@ -213,7 +225,7 @@ __global__ __launch_bounds__(NWV * WAVE, (NWV == 4 && TB == 2 ? 2 : 1)) void rou
         for (int d = 0; d < D; ++d) {
             const int k0 = kb + d * KC;
             RT_STASH(d);
-            __syncthreads();
+            rt_team_sync<TEAM1>();
             RT_FETCH(d, k0 + D * KC);
             // only the h that exist take part: a padded step would add +0 and could turn a -0 chain into +0
             const int sh = k0 - min(k0, ks_max);        // where h = k0 sits in the slab
@@ -232,7 +244,8 @@ __global__ __launch_bounds__(NWV * WAVE, (NWV == 4 && TB == 2 ? 2 : 1)) void rou
 #define RT_PAIR(c) /* chunks c (even) and c + 1 */                                         \
     RT_CHUNK(xa, wa, xb, wb, ((c) + 1) * VN);                                              \
     RT_CHUNK(xb, wb, xa, wa, ((c) + 2 < NCH ? (c) + 2 : NCH - 1) * VN)
-                    RT_PAIR(0); RT_PAIR(2); RT_PAIR(4); RT_PAIR(6);
+                    RT_PAIR(0); RT_PAIR(2);
+                    if constexpr (NCH >= 8) { RT_PAIR(4); RT_PAIR(6); }
                     if constexpr (NCH == 16) { RT_PAIR(8); RT_PAIR(10); RT_PAIR(12); RT_PAIR(14); }
 #undef RT_PAIR
                 } else {
@@ -243,13 +256,31 @@ __global__ __launch_bounds__(NWV * WAVE, (NWV == 4 && TB == 2 ? 2 : 1)) void rou
                     }
                 }
             }
-            __syncthreads();
+            rt_team_sync<TEAM1>();
         }
     }
 #undef RT_CHUNK
 #undef RT_MFMA
 #undef RT_STASH
 #undef RT_FETCH
+}
+
+// The segment chains as separate workgroups: grid = (segments, token blocks, expert blocks); every block stores its
+// partial sums to its plane of the workspace, and a second kernel (topk_gate_kernel) folds the planes.
+template <typename XT, int SHAPE, int TB, int G, int NWV, int CPR>
+__global__ __launch_bounds__(NWV * WAVE, (NWV == 4 && TB == 2 ? 2 : 1)) void route_logits_mfma_kernel(const XT* __restrict__ x, const XT* __restrict__ w,
+                                                                        float* __restrict__ part /*[RT_P][T][E]*/, int T,
+                                                                        int Hrow, int E) {
+    constexpr int NTOK = TB * RT_TB, EB = NWV * G * SHAPE, KC = CPR * VecLoad<XT>::N, NACC = SHAPE == 16 ? 16 : 4;
+    __shared__ __align__(16) float xs[NTOK][KC + 4];
+    __shared__ __align__(16) float wsT[EB][KC + 4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // (the segment is the fastest-running block index: the blocks that are resident together then read whole token
+    // rows between them, not the same eighth of every row, which would load the memory channels unevenly)
+    const int t0 = blockIdx.y * NTOK, eb0 = blockIdx.z * EB;
+    const int seg = blockIdx.x;
+    typename RtAcc<SHAPE>::type acc[TB][G];
+    route_segment_chain<XT, SHAPE, TB, G, NWV, CPR, false, 2>(x, w, T, Hrow, E, seg, t0, eb0, tid, wave, xs, wsT, acc);
     float* out = part + (size_t)seg * T * E;
 #pragma unroll
     for (int g = 0; g < G; ++g) {
@@ -283,19 +314,17 @@ __device__ __forceinline__ unsigned tk_xchg(int off, unsigned x) {
     }
 }
 
+// One pass of a wave: TPW = 64 / G tokens from tbase on.  part: the segments' partial sums, plane p at part + p * plane,
+// token t's row at t_part * E inside a plane (global workspace: t_part = t, plane = T E; a workgroup's own LDS copy:
+// t_part = t - first token of the workgroup).
 template <int G>
-__global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict__ part /*[RT_P][T][E]*/,
-                                                         const float* __restrict__ bias, float* __restrict__ logits,
-                                                         int32_t* __restrict__ idx, float* __restrict__ gate, int T, int E,
-                                                         int k) {
-    constexpr int TPW = WAVE / G;  // tokens per wave
+__device__ __forceinline__ void topk_gate_pass(const float* __restrict__ part, size_t plane, int t_part0, const float* __restrict__ bias,
+                                               float* __restrict__ logits, int32_t* __restrict__ idx, float* __restrict__ gate, int T,
+                                               int E, int k, int tbase) {
     const int lane = lane_id();
     const int gl = lane % G;
-    const int wave_global = (blockIdx.x * blockDim.x + threadIdx.x) / WAVE;
-    const int n_waves = (gridDim.x * blockDim.x) / WAVE;
     const float NEG_INF = -__builtin_huge_valf();
-
-    for (int tbase = wave_global * TPW; tbase < T; tbase += n_waves * TPW) {
+    {
         const int t = tbase + lane / G;
         const bool live = t < T;
         float v[TK_MAXV];
@@ -307,11 +336,11 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict_
             float sum[4] = {NEG_INF, NEG_INF, NEG_INF, NEG_INF};
             if (live && eh < E) {
                 // the segments' partial sums in segment order, then the bias: this fixes the logit's bits
-                const float* pp = part + (size_t)t * E + eh;
+                const float* pp = part + (size_t)(t - t_part0) * E + eh;
                 if (vec) {  // (eh + 3 < E then)
                     float4 sp[RT_P];
 #pragma unroll
-                    for (int p = 0; p < RT_P; ++p) sp[p] = *reinterpret_cast<const float4*>(pp + (size_t)p * T * E);
+                    for (int p = 0; p < RT_P; ++p) sp[p] = *reinterpret_cast<const float4*>(pp + (size_t)p * plane);
                     sum[0] = sp[0].x; sum[1] = sp[0].y; sum[2] = sp[0].z; sum[3] = sp[0].w;
 #pragma unroll
                     for (int p = 1; p < RT_P; ++p) {
@@ -324,7 +353,7 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict_
                         if (eh + c < E) {
                             float a = pp[c];
 #pragma unroll
-                            for (int p = 1; p < RT_P; ++p) a = __fadd_rn(a, pp[(size_t)p * T * E + c]);
+                            for (int p = 1; p < RT_P; ++p) a = __fadd_rn(a, pp[(size_t)p * plane + c]);
                             sum[c] = a;
                         }
                     }
@@ -389,24 +418,71 @@ __global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict_
             }
         }
         // softmax denominator: per-lane ascending partial sum, then a butterfly over the token's lanes
-        float part = 0.f;
+        float part_sum = 0.f;
 #pragma unroll
         for (int i = 0; i < TK_MAXV; ++i) {
             const int e = e0 + i;
-            if (e < E) part += expf(v[i] - row_max);
+            if (e < E) part_sum += expf(v[i] - row_max);
         }
 #pragma unroll
-        for (int off = 1; off < G; off <<= 1) part += __uint_as_float(tk_xchg(off, __float_as_uint(part)));
+        for (int off = 1; off < G; off <<= 1) part_sum += __uint_as_float(tk_xchg(off, __float_as_uint(part_sum)));
         // lane gl writes selection gl (and gl + G when k > G): one exp and one division per lane instead of k in one lane
         if (live && gl < k) {
             idx[(size_t)t * k + gl] = my_e;
-            gate[(size_t)t * k + gl] = expf(my_v - row_max) / part;
+            gate[(size_t)t * k + gl] = expf(my_v - row_max) / part_sum;
         }
         if (live && gl + G < k) {
             idx[(size_t)t * k + gl + G] = my_e2;
-            gate[(size_t)t * k + gl + G] = expf(my_v2 - row_max) / part;
+            gate[(size_t)t * k + gl + G] = expf(my_v2 - row_max) / part_sum;
         }
     }
+}
+
+template <int G>
+__global__ __launch_bounds__(256) void topk_gate_kernel(const float* __restrict__ part /*[RT_P][T][E]*/,
+                                                         const float* __restrict__ bias, float* __restrict__ logits,
+                                                         int32_t* __restrict__ idx, float* __restrict__ gate, int T, int E,
+                                                         int k) {
+    constexpr int TPW = WAVE / G;  // tokens per wave
+    const int wave_global = (blockIdx.x * blockDim.x + threadIdx.x) / WAVE;
+    const int n_waves = (gridDim.x * blockDim.x) / WAVE;
+    for (int tbase = wave_global * TPW; tbase < T; tbase += n_waves * TPW)
+        topk_gate_pass<G>(part, (size_t)T * E, 0, bias, logits, idx, gate, T, E, k, tbase);
+}
+
+// Logits and top-k in one launch, for up to 16 experts.  A workgroup takes 64 tokens; wave p runs the chains of segment p for
+// all experts (G groups of four), on its own slabs in its own part of the LDS, at its own pace (no block barrier inside the
+// reduction); the eight waves then leave their partial sums in LDS, meet once, and each folds the sums of eight of the
+// tokens in segment order and selects -- the arithmetic of the two-kernel path (route_segment_chain, topk_gate_pass), without
+// the partial sums' trip through memory and without the second launch.
+template <typename XT, int G, int CPR, int D>
+__global__ __launch_bounds__(RT_P * WAVE, 1) void route_fused_kernel(const XT* __restrict__ x, const XT* __restrict__ w,
+                                                                      const float* __restrict__ bias, float* __restrict__ logits,
+                                                                      int32_t* __restrict__ idx, float* __restrict__ gate, int T,
+                                                                      int Hrow, int E, int k) {
+    constexpr int KC = CPR * VecLoad<XT>::N, EB = G * 4;
+    __shared__ __align__(16) float xs[RT_P][RT_TB][KC + 4];
+    __shared__ __align__(16) float wsT[RT_P][EB][KC + 4];
+    static_assert(sizeof(float) * RT_P * RT_TB * EB <= sizeof(float) * RT_P * RT_TB * (KC + 4), "the partial sums reuse the token slabs");
+    const int lane = threadIdx.x & 63, seg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int t0 = blockIdx.x * RT_TB;
+    rt_f4 acc[1][G];
+    route_segment_chain<XT, 4, 1, G, 1, CPR, true, D>(x, w, T, Hrow, E, seg, t0, 0, lane, 0, xs[seg], wsT[seg], acc);
+    // partial sums: plane seg, row = token of the workgroup, E columns (lane l holds tokens 4 (l / 4) + v, expert 4 g + l % 4)
+    float* part = &xs[0][0][0];
+    __syncthreads();  // (every wave is done with its slabs)
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const int e = g * 4 + lane % 4;
+        if (e < E) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) part[((size_t)seg * RT_TB + 4 * (lane / 4) + v) * E + e] = acc[0][g][v];
+        }
+    }
+    __syncthreads();
+    // eight lanes per token (eight experts each: E <= 16 takes two of them... G lanes hold 8 G' experts): 8 tokens per wave
+    constexpr int TG = 8;
+    topk_gate_pass<TG>(part, (size_t)RT_TB * E, t0, bias, logits, idx, gate, T, E, k, t0 + seg * (WAVE / TG));
 }
 
 // Block shapes.  Many tokens: 128 tokens per block and slabs of 64 h, so that every wave runs two chains per group of
@@ -460,6 +536,26 @@ extern "C" int moe_route_topk(const void* x, const void* router, const float* bi
     MOE_REQUIRE(ws_bytes >= moe_route_workspace_bytes(T, E), MOE_ERR_WORKSPACE, "route_topk: workspace %zu < %zu", ws_bytes,
                 moe_route_workspace_bytes(T, E));
     MOE_REQUIRE((((uintptr_t)ws | (uintptr_t)logits) & 15) == 0, MOE_ERR_INVALID, "route_topk: ws and logits must be 16-byte aligned");
+    if (E <= 16 && T > 2048) {
+        // few experts, many tokens: logits and top-k in one launch, the partial sums never leave the workgroup (the workspace
+        // is not used).  With few tokens the launch would be a handful of workgroups, each walking its rows slab after slab
+        // (measured: 22 us against 13 for 512 tokens): those keep the two launches, whose first spreads the segments
+        // over eight times as many workgroups.
+        // (two or four groups of four experts per wave: a wave's 64 lanes move a slab of 32 h of 8 or 16 experts, no less)
+        const int blocks = ceil_div(T, RT_TB);
+    // (slabs in flight per wave: four of 32 h or three of 64 h with two groups of experts, two with four -- what the registers hold)
+#define RT_FUSED(XTv, Gv, CPRv) \
+    route_fused_kernel<XTv, Gv, CPRv, (Gv == 2 ? (CPRv * VecLoad<XTv>::N == 32 ? 4 : 2) : 2)><<<blocks, RT_P * WAVE, 0, s>>>((const XTv*)x, (const XTv*)router, bias, logits, topk_idx, topk_gate, T, H, E, k)
+        if (dtype == MOE_F32) {
+            if (E <= 8) RT_FUSED(float, 2, 8);
+            else RT_FUSED(float, 4, 8);
+        } else {
+            if (E <= 8) RT_FUSED(bf16_t, 2, 8);  // (slabs of 64 h: 128 contiguous bytes of a token row per request)
+            else RT_FUSED(bf16_t, 4, 4);
+        }
+#undef RT_FUSED
+        return moe_check_launch("route_fused");
+    }
     float* part = (float*)ws;
     int rc = dtype == MOE_F32 ? launch_logits<float>((const float*)x, (const float*)router, part, T, H, E, s)
                               : launch_logits<bf16_t>((const bf16_t*)x, (const bf16_t*)router, part, T, H, E, s);
