@@ -302,6 +302,74 @@ def stream_ceiling_leg(cfg, steps, world=None):
     return out
 
 
+def gemm_phases_leg(cfg, pipe, steps):
+    """Where time goes inside the grouped GEMMs of this workload (moe_diag_gemm_trace: the same kernels with wall-clock stamps):
+    per tile the K loop, the epilogue and the gap to the next K loop, averaged over all workgroups and tiles but each
+    workgroup's first; the duration of one MFMA block (64 bytes of K of a 256 x 256 tile) of workgroup 0 early and late in the
+    launch (the clock falls under sustained load); and the same launch with the epilogue's stores suppressed."""
+    import numpy as np
+    import torch
+    L_ = __import__("iris_testing_amd._lib", fromlist=["x"])
+    lib = L_.lib()
+    words = lib.moe_diag_gemm_trace_words()
+    TW = 256  # words per workgroup
+    n_wg = (words - 4096) // TW
+    buf = torch.zeros(words, dtype=torch.int64, device="cuda")
+    fp8 = cfg.quant == "fp8"
+    s = L_.stream_ptr()
+    out = {"clock": "100 MHz wall clock, times in microseconds", "workgroups": n_wg}
+    for name, sel, fn in (("gate_up", 0x200, pipe.mlp_up), ("down", 0x100, pipe.mlp_up if fp8 else pipe.mlp_down)):
+        out[name] = {}
+        variants = (("with_stores", 0), ("stores_suppressed", 1))
+        call_ms = {label: [] for label, _ in variants}
+        stamps = {}
+        for rep in range(3):  # (the two variants in turn: what the clock does under sustained load then weighs on both alike)
+            for label, bit in variants:
+                L_.check(lib.moe_diag_gemm_trace(buf.data_ptr(), words, sel | bit))
+                try:
+                    call_ms[label].append(_timed(lambda: fn(s), max(steps // 2, 2), torch))
+                    if rep == 2:
+                        buf.zero_()
+                        fn(s)
+                        torch.cuda.synchronize()
+                        stamps[label] = buf.cpu().numpy()
+                finally:
+                    L_.check(lib.moe_diag_gemm_trace(None, 0, 0))
+        for label, bit in variants:
+            ms = sum(call_ms[label]) / len(call_ms[label])
+            h = stamps[label]
+            tiles = h[:n_wg * TW].reshape(n_wg, TW)
+            kl, ep, gap = [], [], []
+            per_wg = []
+            for w in range(n_wg):
+                ev = tiles[w][tiles[w] > 0]
+                n = len(ev) // 3
+                per_wg.append(n)
+                if n < 2:
+                    continue
+                e = ev[:3 * n].reshape(n, 3).astype(np.float64) / 100.0
+                kl += list(e[1:, 1] - e[1:, 0])
+                ep += list(e[1:, 2] - e[1:, 1])
+                gap += list(e[1:, 0] - e[:-1, 1])
+            blk = h[n_wg * TW:]
+            d = np.diff(blk[blk > 0].astype(np.float64)) / 100.0
+            med = float(np.median(d)) if len(d) else float("nan")
+            body = d[d < 2.0 * med] if len(d) else d   # (blocks inside a K loop: the stamps across a tile boundary hold the epilogue)
+            q = max(len(body) // 4, 1)
+            stamped = h[h > 0]
+            out[name][label] = {
+                "call_ms": round(ms, 4), "tiles_per_workgroup": [int(min(per_wg)), int(max(per_wg))],
+                "k_loop_us": round(float(np.mean(kl)), 2), "epilogue_us": round(float(np.mean(ep)), 2),
+                "k_loop_end_to_next_k_loop_us": round(float(np.mean(gap)), 2),
+                "block_us_first_quarter": round(float(np.median(body[:q])), 3), "block_us_last_quarter": round(float(np.median(body[-q:])), 3),
+                "blocks_stamped": int(len(d) + 1), "launch_span_us": round(float(stamped.max() - stamped.min()) / 100.0, 1)}
+    if fp8:
+        out["note"] = "fp8: one call runs both GEMMs (call_ms is the call; the stamps are of the GEMM named)"
+    pipe.step()
+    torch.cuda.synchronize()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -325,6 +393,8 @@ def main():
     ap.add_argument("--backward", action="store_true", help="also time forward + backward of rank 0's expert MLP")
     ap.add_argument("--stream-ceiling", action="store_true",
                     help="also measure copy / write / read-mostly rates of the row-moving kernels on 1 GiB buffers")
+    ap.add_argument("--gemm-phases", action="store_true",
+                    help="also trace the phases of the grouped GEMMs' tiles (moe_diag_gemm_trace), with and without the epilogue's stores")
     ap.add_argument("--mfma-ceiling", action="store_true",
                     help="also measure what the matrix cores sustain from registers, on all-zero and on N(0,1)-like operands")
     ap.add_argument("--cpu-sample-tokens", type=int, default=0, help="0 = sized for roughly 10-30 s")
@@ -478,6 +548,11 @@ def main():
         out["stream_ceiling"] = stream_ceiling_leg(cfg, max(args.steps // 2, 3), world)
     if args.mfma_ceiling:
         out["mfma_ceiling"] = mfma_ceiling_leg(max(args.steps // 4, 3))
+    if args.gemm_phases:
+        if cfg.dtype == "f32":
+            out["gemm_phases"] = {"skipped": "the fp32 expert runs the plain LDS-tiled kernel"}
+        else:
+            out["gemm_phases"] = gemm_phases_leg(cfg, pipe, max(args.steps // 2, 3))
 
     if not args.no_cpu_baseline:
         def to_np(t):

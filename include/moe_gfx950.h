@@ -372,6 +372,20 @@ size_t moe_diag_mfma_loop_sink_floats(void);
 double moe_diag_mfma_loop_flops(int fp8, int iters, int workgroups);
 int moe_diag_mfma_loop(int fp8, int random_data, int iters, int workgroups, float* sink, moe_stream_t stream);
 
+/* moe_diag_gemm_trace: where time goes inside the grouped GEMM.  After a call with a device buffer of `words` >=
+ * moe_diag_gemm_trace_words() 64-bit words, the forward grouped-GEMM launches of the calling process (through any entry point
+ * above; 256-row tiles, no activation or SwiGLU) run an instantiation of the same kernel that writes the device's 100 MHz wall
+ * clock into the buffer, take whole tiles only (no K split of the last round), and overwrite what the launch before left:
+ *   words [256 w, 256 w + 256) of workgroup w: for each of its tiles in turn, the clock at the start of the tile's K loop, at the
+ *     end of its K loop and at the end of its epilogue (the first 85 tiles);
+ *   words [256 G, 256 G + 4096), G = number of workgroups = compute units: the clock at the end of every MFMA block (one 64-byte
+ *     K stage of a 256 x 256 tile) of workgroup 0.
+ * flags: bit 0: the epilogue computes but stores nothing (what the stores cost); 0x100: only launches without activation are
+ * traced (the down projection); 0x200: only launches with one (gate/up).  trace == NULL ends it.  Not thread-safe; the
+ * launches compute the same results (unless bit 0 is set).  Used by `bench.py --gemm-phases`. */
+size_t moe_diag_gemm_trace_words(void);
+int moe_diag_gemm_trace(unsigned long long* trace, size_t words, int flags);
+
 #ifdef __cplusplus
 }
 #endif

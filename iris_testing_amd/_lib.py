@@ -83,6 +83,8 @@ _SIGNATURES = {
     "moe_diag_mfma_loop_sink_floats": (c_size_t, []),
     "moe_diag_mfma_loop_flops": (ctypes.c_double, [c_int, c_int, c_int]),
     "moe_diag_mfma_loop": (c_int, [c_int, c_int, c_int, c_int, P, P]),
+    "moe_diag_gemm_trace_words": (c_size_t, []),
+    "moe_diag_gemm_trace": (c_int, [P, c_size_t, c_int]),
     "moe_combine": (c_int, [P, c_int, c_int, c_int, c_int, P, P, P, P, c_int, c_int, c_int, P, P, P]),
 }
 

@@ -78,7 +78,14 @@ struct GemmParams {
     int dw_rows;
     int dw_src_rows;  // rows of the untransposed operands: the counts are clamped to it, as the operand kernels clamp them
     size_t c_group_stride;
+    // Time stamps (the TRACE instantiation only; see moe_diag_gemm_trace): GG_TRACE_TILE_WORDS words per workgroup -- for
+    // every tile the wall clock (100 MHz) at the start of its K loop, at the end of its K loop and at the end of its
+    // epilogue -- then GG_TRACE_BLOCK_WORDS words of workgroup 0: the clock at the end of each of its MFMA blocks.
+    // trace_flags & 1: the epilogue computes but stores nothing.
+    unsigned long long* trace;
+    int trace_flags;
 };
+constexpr int GG_TRACE_TILE_WORDS = 256, GG_TRACE_BLOCK_WORDS = 4096;
 
 constexpr int GG_MAX_PARTS = 16;   // parts per tile at most
 constexpr int GG_RED_SLABS = 32;   // blocks per tile in the reduction of the parts
@@ -396,8 +403,18 @@ __device__ __forceinline__ void gg_wait() {
 // SPLIT = false: the launch that takes whole tiles.  SPLIT = true: the launch that takes the tiles of an
 // under-filled last round in parts of the K range and leaves fp32 partial sums in the workspace (GemmParams).
 // BSA: the activation operand carries block scales (fp8 down projection: GemmParams::a_bscale), applied by the MFMAs.
-template <int BM, int NWM, int EPI, bool FP8, bool SPLIT, bool DW = false, bool BSA = false>
+// TRACE: the same kernel with time stamps (GemmParams::trace); product launches never use it.
+template <int BM, int NWM, int EPI, bool FP8, bool SPLIT, bool DW = false, bool BSA = false, bool TRACE = false>
 __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const GemmParams p) {
+    static_assert(!TRACE || (!SPLIT && !DW), "time stamps: whole-tile forward launches only");
+    [[maybe_unused]] int tr_tile = 0, tr_blk = 0;  // (TRACE) words written so far
+#define GG_TRACE_TILE()                                                                                                    \
+    do {                                                                                                                   \
+        if constexpr (TRACE) {                                                                                             \
+            if (threadIdx.x == 0 && tr_tile < GG_TRACE_TILE_WORDS) p.trace[(size_t)blockIdx.x * GG_TRACE_TILE_WORDS + tr_tile] = wall_clock64(); \
+            ++tr_tile;                                                                                                     \
+        }                                                                                                                  \
+    } while (0)
     static_assert(!DW || (!SPLIT && !FP8 && EPI == EPI_NONE), "the weight-gradient mode is a plain bf16 GEMM");
     static_assert(!BSA || FP8, "block scales belong to the fp8 MFMA");
     constexpr bool VARK = SPLIT || DW;  // the K range differs from tile to tile
@@ -710,7 +727,13 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             gg_wait<2 * LPS, 0>();                                                                       \
             __builtin_amdgcn_s_barrier();                                                                \
         }                                                                                                \
+        if constexpr (TRACE) {                                                                           \
+            if (blockIdx.x == 0 && threadIdx.x == 0 && tr_blk < GG_TRACE_BLOCK_WORDS)                    \
+                p.trace[(size_t)gridDim.x * GG_TRACE_TILE_WORDS + tr_blk] = wall_clock64();              \
+            ++tr_blk;                                                                                    \
+        }                                                                                                \
     } while (0)
+        GG_TRACE_TILE();
         int kbase = 0, nks_ld = nks;  // the loads of block s fetch stage s + 4 - kbase of the tile (Ab, Bb, a_off) point to
         bool seam = false;            // ... which is the next tile from block nks - 4 on
         {
@@ -823,6 +846,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
         // ---- next tile: decode it and request its first stages now (every slot is free once all waves
         // have passed the barrier: the last fragments of this tile are already in registers)
         // (when the K loop has switched over, the walk only confirms what the look-ahead saw)
+        GG_TRACE_TILE();
         const GgTile nxt = gg_walk<BM, SPLIT, DW>(s_tiles, g_tile_start, g_row_start, p.E_l, Nt, p.S_rows, plan, nk, my, (int)gridDim.x, round, round0, p.dw_rows);
         if (!seam && nxt.rv > 0) {
             GG_TILE_PTRS(nxt, Ab_n, Bb_n, a_off_n, GG_MAPROW_GLOBAL);
@@ -902,7 +926,7 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
 #pragma unroll
             for (int h = 0; h < NR; ++h) {
                 const int r = rbase_e + i * MT + ((FP8 && !QOUT) ? (lane_e & 15) + 16 * h : (lane_e & (MT - 1)));
-                ok[i][h] = r < rv;
+                ok[i][h] = r < rv && !(TRACE && (p.trace_flags & 1));
                 const size_t grow = (size_t)(row0 + (ok[i][h] ? r : 0));
                 const int crow_i = p.c_map ? s_crow[tpar][r] : 0;
                 ok[i][h] = ok[i][h] && crow_i >= 0;  // a negative map entry: the row has no place in the output
@@ -1063,11 +1087,13 @@ __global__ __launch_bounds__(NWM * 2 * WAVE, 1) void grouped_gemm_kernel(const G
             // (that would need every accumulator in a VGPR at once)
             __builtin_amdgcn_sched_barrier(0);
         }
+        GG_TRACE_TILE();
         cur = nxt;
         pre = seam;
         phi = phi_n;
         tpar ^= 1;
     }
+#undef GG_TRACE_TILE
 #undef GG_TILE_PTRS
 #undef GG_MAPROW_GLOBAL
 #undef GG_MAPROW_LDS
@@ -1732,10 +1758,19 @@ int num_cus() {
 
 int round_up(int a, int b) { return (a + b - 1) / b * b; }
 
+// moe_diag_gemm_trace: where the next forward GEMM launches of this process leave time stamps (not thread-safe: a diagnostic)
+struct { unsigned long long* buf; int flags; } g_trace = {nullptr, 0};
+
 template <bool FP8>
 int launch_gemm(const GemmParams& p_in, int epi, hipStream_t s, void* part_ws = nullptr, size_t part_ws_bytes = 0) {
     const int grid = num_cus();
     GemmParams p = p_in;
+    const bool traced = g_trace.buf && (!(g_trace.flags & 0x300) || (g_trace.flags & (epi == EPI_NONE ? 0x100 : 0x200)));
+    if (traced) {  // (see moe_diag_gemm_trace: whole tiles only, so that every tile leaves its stamps)
+        p.trace = g_trace.buf;
+        p.trace_flags = g_trace.flags;
+        part_ws = nullptr;
+    }
     // 256-row or 128-row tiles: the host knows only the total row count, so it compares the estimated number
     // of rounds of the persistent grid (every group adds about half a tile of ragged tail); a 128-row tile
     // costs about 0.62 of a 256-row one
@@ -1761,6 +1796,12 @@ int launch_gemm(const GemmParams& p_in, int epi, hipStream_t s, void* part_ws = 
 #define GG_LAUNCH(BMv, NWMv, EPIv)                                                                        \
     do {                                                                                                  \
         constexpr bool BSAv = FP8 && EPIv == EPI_NONE;                                                    \
+        if (traced) {                                                                                     \
+            if constexpr (BMv == 256 && (EPIv == EPI_NONE || EPIv == EPI_SWIGLU))                         \
+                grouped_gemm_kernel<BMv, NWMv, EPIv, FP8, false, false, BSAv, true><<<grid, NWMv * 2 * WAVE, 0, s>>>(p); \
+            else return moe_fail(MOE_ERR_UNSUPPORTED, "grouped_gemm: no time-stamping instantiation for this launch (256-row tiles, no activation or SwiGLU)"); \
+            break;                                                                                        \
+        }                                                                                                 \
         if (!all_split) grouped_gemm_kernel<BMv, NWMv, EPIv, FP8, false, false, BSAv><<<grid, NWMv * 2 * WAVE, 0, s>>>(p); \
         if (p.part_ws && red_blocks > 0) {                                                                \
             /* (the launch that takes parts stores raw partial sums: one instantiation whatever the epilogue) */ \
@@ -1816,6 +1857,16 @@ int launch_prepack(const T* w, const T* w_up, int E_l, int K, int N, T* out, hip
 
 }  // namespace moe_gg
 using namespace moe_gg;
+
+extern "C" size_t moe_diag_gemm_trace_words(void) { return (size_t)num_cus() * GG_TRACE_TILE_WORDS + GG_TRACE_BLOCK_WORDS; }
+
+extern "C" int moe_diag_gemm_trace(unsigned long long* trace, size_t words, int flags) {
+    MOE_REQUIRE(!trace || words >= moe_diag_gemm_trace_words(), MOE_ERR_WORKSPACE, "diag_gemm_trace: %zu words, %zu needed", words,
+                moe_diag_gemm_trace_words());
+    g_trace.buf = trace;
+    g_trace.flags = trace ? flags : 0;
+    return MOE_OK;
+}
 
 extern "C" size_t moe_prepack_bytes(int dtype, int E_l, int K, int N) {
     if (dtype == MOE_F32) return 0;
