@@ -158,6 +158,26 @@ def test_route_block_shapes_for_many_tokens(E, dtype):
     np.testing.assert_allclose(to_np(gate), o_gate, rtol=1e-5, atol=1e-30)
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("T,H,E,k,bias", [(2049, 8, 1, 1, True), (2111, 72, 2, 2, False), (2050, 4096, 8, 8, True), (2300, 520, 9, 9, False),
+                                          (2177, 264, 13, 5, True), (3000, 8192, 16, 16, True), (2112, 64, 5, 1, False)])
+def test_route_one_launch_edge_shapes(T, H, E, k, bias, dtype):
+    """Up to 16 experts and more than 2048 tokens run logits and top-k in one launch: one token in the last workgroup, a single
+    expert, as many selections as experts, rows shorter than one segment per wave (most chains empty), rows of 16 KB, expert counts
+    on either side of the two-group / four-group split, with and without bias -- bit-exact against the oracle."""
+    g = torch.Generator().manual_seed(T + 7 * E)
+    x = torch.randn(T, H, generator=g)
+    w = torch.randn(H, E, generator=g) * H ** -0.5
+    b = torch.randn(E, generator=g) if bias else None
+    if dtype == "bf16":
+        x, w = x.bfloat16(), w.bfloat16()
+    idx, gate, logits = ops.route_topk(x.to(DEV), w.to(DEV).contiguous(), k, None if b is None else b.to(DEV))
+    o_idx, o_gate, o_logits = O.route(to_np(x), to_np(w), k, None if b is None else b.numpy())
+    assert_bits_equal(logits, o_logits, f"logits T={T} H={H} E={E} {dtype}")
+    assert_bits_equal(idx, o_idx, f"top-k T={T} H={H} E={E} k={k} {dtype}")
+    np.testing.assert_allclose(to_np(gate), o_gate, rtol=1e-5, atol=1e-30)
+
+
 @pytest.mark.parametrize("E,k,W", [(8, 8, 4), (512, 16, 64), (6, 1, 3), (60, 7, 1), (40, 12, 4), (16, 16, 2)])  # (the last two: more selections than lanes per token)
 def test_route_edge_shapes(E, k, W):
     T, H = 77, 72
