@@ -43,6 +43,35 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert lib.moe_count_workspace_bytes(1000, 2, 8) == 4 * (2 * 8 * 16 + 2 * 8 + 1)
 
 
+def test_argument_errors_of_the_fused_variants_and_diagnostics_without_a_gpu():
+    """The gated / flat-payload / fp8 entry points and the diagnostics validate before they touch the GPU."""
+    from iris_testing_amd import _lib as L
+    lib = L.lib()
+    # gates and their output buffer go together
+    rc = lib.moe_pack_tokens_gated(None, 1, 4, 64, None, None, 1, 2, 2, None, None, 2, 4, None, None, None, None)
+    assert rc == -1 and b"go together" in lib.moe_last_error()
+    rc = lib.moe_recv_row_map_gated(None, 2, 2, 4, 8, 1, None, None, None, None)
+    assert rc == -1
+    rc = lib.moe_recv_row_map_flat(None, 0, 2, 8, None, None, None)
+    assert rc == -1
+    # the gated down projection needs its gates; bf16 GEMMs need K % 64 == 0
+    rc = lib.moe_grouped_gemm_mapped_gated(1, 8, None, 1, 1, 8, 64, 64, 1, None, 1, 8, None, None, 0, None)
+    assert rc == -1 and b"null pointer" in lib.moe_last_error()
+    rc = lib.moe_grouped_gemm_mapped_gated(1, 8, None, 1, 1, 8, 48, 64, 1, 1, 1, 8, None, None, 0, None)
+    assert rc == -2 and b"K %" in lib.moe_last_error()
+    # fp8 expert: H and F in multiples of 128
+    rc = lib.moe_grouped_mlp_fp8_q_mapped(1, 1, 8, None, 1, 8, 256, 96, 1, 1, 1, 1, 1, 1, 1, 1, 1, None, 1, 8, None, None, 0, None)
+    assert rc == -2 and b"multiples of 128" in lib.moe_last_error()
+    rc = lib.moe_grouped_mlp_fp8_mapped(1, 8, None, 1, 8, 200, 128, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, None, 1, 8, None, None, 0, None)
+    assert rc == -2 and b"multiples of 128" in lib.moe_last_error()
+    # time stamps need a buffer of the advertised size; switching them off needs none
+    assert lib.moe_diag_gemm_trace_words() >= 128 + 4096
+    rc = lib.moe_diag_gemm_trace(1, 16, 0)
+    assert rc == -3 and b"words" in lib.moe_last_error()
+    assert lib.moe_diag_gemm_trace(None, 0, 0) == 0
+    assert lib.moe_diag_mfma_loop_flops(0, 1, 1) == 2.0 * 4 * 128 * 128 * 32
+
+
 def test_static_scratch_count_rejects_oversized_inputs_without_a_gpu():
     """The allocation-free counting entry point checks its size limit before it touches the GPU."""
     from iris_testing_amd import _lib as L
