@@ -208,3 +208,34 @@ def test_flat_row_map_with_empty_blocks_and_rows_past_the_total():
     assert_bits_equal(row_map[:S], want, "flat row map")
     assert (to_np(row_map)[S:] == 0).all()
     assert_bits_equal(cnt, rc.sum(0).astype(np.int32), "expert counts")
+
+
+@pytest.mark.parametrize("name,mode", [("small", "gated"), ("small", "padding_free"), ("zipf_k1", "gated"), ("zipf_k1", "padding_free")])
+def test_graph_replay_of_the_wider_forms_equals_eager(name, mode):
+    """The gated and the padding-free step captured as one HIP graph: every replay (outputs cleared before it, eager work and
+    synchronisation between replays) reproduces the eager step bit for bit."""
+    cfg = CONFIGS[name]
+    world = harness.build_world(cfg, DEV)
+    ew, _, _ = harness.expert_weights(cfg, 0, DEV)
+    gated, flat = mode == "gated", mode == "padding_free"
+    pipe = DispatchPipeline(world, ew, gated=gated, padding_free=flat,
+                            fp8_dispatch=False if flat else None,
+                            recv_gate=harness.recv_gates(world) if gated else None,
+                            recv_flat=harness.recv_flat(world) if flat else None)
+    pipe.returned.copy_(torch.randn(pipe.returned.shape, device=DEV).to(pipe.returned.dtype))
+    pipe.step()
+    torch.cuda.synchronize()
+    assert int(pipe.status.item()) == 0
+    names = ["idx", "gate", "send_counts", "pos", "row_map", "out"] + (["ret_flat"] if flat else ["ret"]) + (["row_gate"] if gated else [])
+    eager = {n: getattr(pipe, n).clone() for n in names}
+    graph = pipe.capture()
+    for rep in range(3):
+        for n in names:
+            getattr(pipe, n).zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for n in names:
+            assert torch.equal(getattr(pipe, n), eager[n]), f"{mode} replay {rep}: {n} differs from the eager step"
+        pipe.step()  # eager work between replays
+        torch.cuda.synchronize()
