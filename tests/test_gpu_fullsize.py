@@ -127,3 +127,75 @@ def test_fused_destination_equals_copies(name):
         assert torch.equal(fused.send_q.view(-1, cfg.hidden), q) and torch.equal(fused.send_scale.view(-1), sc), \
             "quantise-and-pack differs from pack, then quantise"
         assert torch.equal(fused.hq, wire.hq) and torch.equal(fused.hsc, wire.hsc), "hidden activations differ"
+
+
+@pytest.mark.parametrize("name", ["mixtral", "finegrained", "zipf_k2", "zipf_k8"])
+def test_full_size_gated_and_flat_payload_forms(name):
+    """The two wider forms of the copy-free destination side at the published sizes, through size-independent properties:
+    * flat payload: the expert's result rows, read back through the two row maps, are bit for bit those of the fixed-M form, and
+      the combined output over a flat returned payload that holds the same rows equals the fixed-M one;
+    * gated return: every returned row is the plain row times its gate, rounded once from the fp32 product instead of twice
+      (within one bf16 step of gate * plain row), padding rows stay zero; and the combine without gates, over returned rows that were
+      weighted and rounded at their source, agrees with the combine-side multiply within the k + 2 roundings that separate them."""
+    cfg = CONFIGS[name]
+    print(f"case {cfg}", flush=True)
+    world = harness.build_world(cfg, DEV)
+    ew, _, _ = harness.expert_weights(cfg, 0, DEV)
+    W, M, H, S, T, k = cfg.world, world.M, cfg.hidden, world.S, cfg.tokens, cfg.topk
+    base = DispatchPipeline(world, ew)
+    base.ret.fill_(float("nan"))
+    base.step()
+    g = torch.Generator(device="cpu").manual_seed(11)
+    base.returned.copy_(torch.randn(base.returned.shape, generator=g).to(base.returned.dtype).to(DEV))  # (stands in for what the other ranks return)
+    base.combine(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert int(base.status.item()) == 0
+    rows_base = base.ret.view(W * M, H)[base.row_map[:S].long()]
+
+    # ---- flat payload
+    flat = DispatchPipeline(world, ew, padding_free=True, fp8_dispatch=False, recv_flat=harness.recv_flat(world))
+    flat.ret_flat.fill_(float("nan"))
+    flat.step()
+    torch.cuda.synchronize()
+    rows_flat = flat.ret_flat[flat.row_map[:S].long()]
+    assert torch.equal(rows_flat.view(torch.int16), rows_base.view(torch.int16)), "flat payload: expert result rows differ"
+    assert not bool(torch.isnan(flat.ret_flat[:S].float()).any()), "flat payload: a result row was not written"
+    # the returned payload in position order, holding the rows the fixed-M form holds in its slots
+    idx, pos = base.idx.long(), base.pos.long()
+    dst = idx // cfg.e_local
+    slot = dst * M + (pos - base.dst_offsets.long()[dst])
+    flat.returned[pos.reshape(-1)] = base.returned.view(W * M, H)[slot.reshape(-1)]
+    flat.combine(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.equal(flat.out.view(torch.int16), base.out.view(torch.int16)), "flat payload: combined output differs"
+
+    # ---- gated return
+    gated = DispatchPipeline(world, ew, gated=True, recv_gate=harness.recv_gates(world))
+    gated.ret.fill_(float("nan"))
+    gated.step()
+    torch.cuda.synchronize()
+    assert int(gated.status.item()) == 0
+    g_rows = gated.row_gate[:S]
+    got = gated.ret.view(W * M, H)[gated.row_map[:S].long()].float()
+    want = g_rows[:, None] * rows_base.float()
+    # one rounding moved: the two differ by at most one bf16 step of the larger magnitude (2^-7 relative), plus the step of
+    # the plain row that was rounded before the multiplication
+    bound = 2.0 ** -7 * torch.maximum(got.abs(), want.abs()) + 1e-30
+    assert bool(((got - want).abs() <= bound).all()), "gated return: a row is further than one bf16 step from gate * plain row"
+    pad = torch.ones(W * M, dtype=torch.bool, device=DEV)
+    pad[gated.row_map[:S].long()] = False
+    assert bool((gated.ret.view(W * M, H)[pad] == 0).all()), "gated return: padding rows must be zero"
+    # the combine without gates over rows weighted at their source: each returned row of the plain form times its slot's gate,
+    # rounded to bf16; against the plain form's combine, which multiplies in fp32 and rounds once
+    gate = base.gate
+    terms = gate[:, :, None] * base.returned.view(W * M, H)[slot].float()           # [T,k,H] fp32
+    gated.returned.zero_()
+    gated.returned.view(W * M, H)[slot.reshape(-1)] = terms.reshape(-1, H).to(gated.returned.dtype)
+    gated.combine(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert int(gated.status.item()) == 0
+    a, b = gated.out.float(), base.out.float()
+    mag = terms.abs().sum(dim=1)
+    del terms
+    # k terms rounded to bf16 (2^-9 relative each) before the sum, and the two sums rounded once each
+    assert bool(((a - b).abs() <= (k + 2) * 2.0 ** -9 * mag + 1e-30).all()), "gated return: combined output too far from the combine-side multiply"
