@@ -352,6 +352,15 @@ def gemm_phases_leg(cfg, pipe, steps):
                 ep += list(e[1:, 2] - e[1:, 1])
                 gap += list(e[1:, 0] - e[:-1, 1])
             blk = h[n_wg * TW:]
+            # workgroup 0: from the start of a tile's K loop to the end of its first MFMA block (the hand-over at the end of that
+            # block waits, in issue order, behind the stores of the epilogue before it)
+            ev0 = tiles[0][tiles[0] > 0]
+            b0 = blk[blk > 0]
+            first = []
+            for ti in range(1, len(ev0) // 3):
+                after = b0[b0 > ev0[3 * ti]]
+                if len(after) and after[0] <= ev0[3 * ti + 1]:
+                    first.append((after[0] - ev0[3 * ti]) / 100.0)
             d = np.diff(blk[blk > 0].astype(np.float64)) / 100.0
             med = float(np.median(d)) if len(d) else float("nan")
             body = d[d < 2.0 * med] if len(d) else d   # (blocks inside a K loop: the stamps across a tile boundary hold the epilogue)
@@ -362,6 +371,7 @@ def gemm_phases_leg(cfg, pipe, steps):
                 "k_loop_us": round(float(np.mean(kl)), 2), "epilogue_us": round(float(np.mean(ep)), 2),
                 "k_loop_end_to_next_k_loop_us": round(float(np.mean(gap)), 2),
                 "block_us_first_quarter": round(float(np.median(body[:q])), 3), "block_us_last_quarter": round(float(np.median(body[-q:])), 3),
+                "first_block_of_a_tile_us": round(float(np.median(first)), 2) if first else None,
                 "blocks_stamped": int(len(d) + 1), "launch_span_us": round(float(stamped.max() - stamped.min()) / 100.0, 1)}
     if fp8:
         out["note"] = "fp8: one call runs both GEMMs (call_ms is the call; the stamps are of the GEMM named)"
